@@ -1,0 +1,266 @@
+// Vector multiply-add throughput kernels (VALU, register resident).
+//
+// Every work-item holds 16 independent accumulators and advances each of them by
+// `steps` dependent multiply-adds, so a lane always has 16 FMAs in flight and the
+// chain latency is hidden without relying on occupancy.  Seeds come from the
+// counter generator (stream MI355_STREAM_MAD, element item*16 + j), nothing is read
+// from memory, and the only store is the per-item sum of the 16 accumulators.
+//
+// The `width` variants (x, x2, x4) group the same 16 accumulators into vectors of
+// 1, 2 or 4 lanes; the arithmetic per accumulator is identical, so all widths of
+// one kind produce identical results.
+#include "internal.h"
+#include "seeded_rng.h"
+#include "numeric_formats.h"
+
+namespace {
+
+constexpr int kAcc = 16;
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+__device__ inline _Float16 bits_to_half(uint16_t h) {
+  _Float16 r;
+  __builtin_memcpy(&r, &h, 2);
+  return r;
+}
+
+// ---- fp32 / fp64 -----------------------------------------------------------
+template <typename T, int W>
+__global__ void __launch_bounds__(256)
+mad_fp_kernel(uint64_t seed, T a, uint32_t steps, uint64_t n_items, T *__restrict__ out) {
+  typedef T Vec __attribute__((ext_vector_type(W)));
+  const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (item >= n_items) return;
+  constexpr int NV = kAcc / W;
+  typename std::conditional<W == 1, T, Vec>::type x0[NV], x[NV];
+#pragma unroll
+  for (int v = 0; v < NV; v++) {
+    if constexpr (W == 1) {
+      x0[v] = (T)mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + v));
+    } else {
+#pragma unroll
+      for (int l = 0; l < W; l++)
+        x0[v][l] = (T)mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + v * W + l));
+    }
+    x[v] = x0[v];
+  }
+#pragma unroll 2
+  for (uint32_t s = 0; s < steps; s++) {
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+      if constexpr (W == 1) x[v] = __builtin_fma(x[v], a, x0[v]);
+      else x[v] = __builtin_elementwise_fma(x[v], (Vec)(a), x0[v]);
+    }
+  }
+  T sum = (T)0;
+#pragma unroll
+  for (int v = 0; v < NV; v++) {
+    if constexpr (W == 1) sum += x[v];
+    else {
+#pragma unroll
+      for (int l = 0; l < W; l++) sum += x[v][l];
+    }
+  }
+  out[item] = sum;
+}
+
+// ---- fp16: width 1 scalar half FMA, width 2 packed half2 FMA ---------------------
+template <int W>
+__global__ void __launch_bounds__(256)
+mad_f16_kernel(uint64_t seed, uint16_t a_bits, uint32_t steps, uint64_t n_items, uint16_t *__restrict__ out) {
+  const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (item >= n_items) return;
+  const _Float16 a = bits_to_half(a_bits);
+  _Float16 sum = (_Float16)0;
+  if constexpr (W == 1) {
+    _Float16 x0[kAcc], x[kAcc];
+#pragma unroll
+    for (int j = 0; j < kAcc; j++) {
+      x0[j] = bits_to_half(mi355_f32_to_f16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j))));
+      x[j] = x0[j];
+    }
+#pragma unroll 2
+    for (uint32_t s = 0; s < steps; s++) {
+#pragma unroll
+      for (int j = 0; j < kAcc; j++) x[j] = __builtin_fmaf16(x[j], a, x0[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < kAcc; j++) sum += x[j];
+  } else {
+    half2v x0[kAcc / 2], x[kAcc / 2];
+    const half2v av = {a, a};
+#pragma unroll
+    for (int v = 0; v < kAcc / 2; v++) {
+#pragma unroll
+      for (int l = 0; l < 2; l++)
+        x0[v][l] = bits_to_half(mi355_f32_to_f16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + v * 2 + l))));
+      x[v] = x0[v];
+    }
+#pragma unroll 2
+    for (uint32_t s = 0; s < steps; s++) {
+#pragma unroll
+      for (int v = 0; v < kAcc / 2; v++) x[v] = __builtin_elementwise_fma(x[v], av, x0[v]);
+    }
+#pragma unroll
+    for (int v = 0; v < kAcc / 2; v++) {
+      sum += x[v][0];
+      sum += x[v][1];
+    }
+  }
+  uint16_t bits;
+  __builtin_memcpy(&bits, &sum, 2);
+  out[item] = bits;
+}
+
+// ---- narrow operands, fp32 accumulator: acc = fma(float(xn), float(an), acc) --------
+// kHalf: operands are IEEE half (maps to the mixed-precision FMA); otherwise bf16.
+template <bool kHalf>
+__global__ void __launch_bounds__(256)
+mad_mixed_kernel(uint64_t seed, uint16_t a_bits, uint32_t steps, uint64_t n_items, float *__restrict__ out) {
+  const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (item >= n_items) return;
+  float acc[kAcc];
+  float sum = 0.0f;
+  if constexpr (kHalf) {
+    const _Float16 a = bits_to_half(a_bits);
+    _Float16 xn[kAcc];
+#pragma unroll
+    for (int j = 0; j < kAcc; j++) {
+      xn[j] = bits_to_half(mi355_f32_to_f16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j))));
+      acc[j] = (float)xn[j];
+    }
+#pragma unroll 2
+    for (uint32_t s = 0; s < steps; s++) {
+#pragma unroll
+      for (int j = 0; j < kAcc; j++) acc[j] = __builtin_fmaf((float)xn[j], (float)a, acc[j]);
+    }
+  } else {
+    const float a = mi355_bf16_to_f32(a_bits);
+    float xn[kAcc];
+#pragma unroll
+    for (int j = 0; j < kAcc; j++) {
+      xn[j] = mi355_bf16_to_f32(mi355_f32_to_bf16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j))));
+      acc[j] = xn[j];
+    }
+#pragma unroll 2
+    for (uint32_t s = 0; s < steps; s++) {
+#pragma unroll
+      for (int j = 0; j < kAcc; j++) acc[j] = __builtin_fmaf(xn[j], a, acc[j]);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kAcc; j++) sum += acc[j];
+  out[item] = sum;
+}
+
+// ---- int32: x = x*a + x0, wrapping --------------------------------------------
+template <int W>
+__global__ void __launch_bounds__(256)
+mad_i32_kernel(uint64_t seed, uint32_t a, uint32_t steps, uint64_t n_items, uint32_t *__restrict__ out) {
+  const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (item >= n_items) return;
+  uint32_t x0[kAcc], x[kAcc];
+#pragma unroll
+  for (int j = 0; j < kAcc; j++) {
+    x0[j] = (uint32_t)(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j) >> 32);
+    x[j] = x0[j];
+  }
+#pragma unroll 2
+  for (uint32_t s = 0; s < steps; s++) {
+#pragma unroll
+    for (int j = 0; j < kAcc; j++) x[j] = x[j] * a + x0[j];
+  }
+  uint32_t sum = 0;
+#pragma unroll
+  for (int j = 0; j < kAcc; j++) sum += x[j];
+  out[item] = sum;
+}
+
+// ---- int8 dot product: acc = sdot4(x, y, acc); y ^= acc; C independent chains -----
+template <int C>
+__global__ void __launch_bounds__(256)
+mad_i8dp_kernel(uint64_t seed, uint32_t steps, uint64_t n_items, int32_t *__restrict__ out) {
+  const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (item >= n_items) return;
+  int32_t x[C], y[C], acc[C];
+#pragma unroll
+  for (int c = 0; c < C; c++) {
+    x[c] = (int32_t)(uint32_t)(mi355_rng_word(seed, MI355_STREAM_MAD, item * 8 + c) >> 32);
+    y[c] = (int32_t)(uint32_t)(mi355_rng_word(seed, MI355_STREAM_MAD_Y, item * 8 + c) >> 32);
+    acc[c] = 0;
+  }
+#pragma unroll 4
+  for (uint32_t s = 0; s < steps; s++) {
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+      acc[c] = __builtin_amdgcn_sdot4(x[c], y[c], acc[c], false);
+      y[c] ^= acc[c];
+    }
+  }
+  uint32_t sum = 0;
+#pragma unroll
+  for (int c = 0; c < C; c++) sum += (uint32_t)acc[c];
+  out[item] = (int32_t)sum;
+}
+
+}  // namespace
+
+extern "C" int mi355_compute_mad(mi355_dev *dev, int kind, int width, uint64_t seed, uint64_t n_items,
+                                 uint32_t steps, void *out, uint32_t block_size) {
+  MI355_ENTER(dev);
+  MI355_REQUIRE(dev, out != nullptr, "compute_mad: null output");
+  MI355_REQUIRE(dev, n_items > 0, "compute_mad: zero items");
+  MI355_REQUIRE(dev, block_size == 64 || block_size == 128 || block_size == 256,
+                "compute_mad: block_size %u not in {64,128,256}", block_size);
+  const uint64_t blocks64 = (n_items + block_size - 1) / block_size;
+  MI355_REQUIRE(dev, blocks64 <= 0x7fffffffull, "compute_mad: too many items");
+  const dim3 grid((uint32_t)blocks64), block(block_size);
+  hipStream_t st = dev->stream;
+#define BAD_WIDTH() return mi355_fail(dev, MI355_ERR_ARG, "compute_mad: width %d not valid for kind %d", width, kind)
+  switch (kind) {
+    case MI355_MAD_F32:
+      if (width == 1) mad_fp_kernel<float, 1><<<grid, block, 0, st>>>(seed, 1.0001f, steps, n_items, (float *)out);
+      else if (width == 2) mad_fp_kernel<float, 2><<<grid, block, 0, st>>>(seed, 1.0001f, steps, n_items, (float *)out);
+      else if (width == 4) mad_fp_kernel<float, 4><<<grid, block, 0, st>>>(seed, 1.0001f, steps, n_items, (float *)out);
+      else BAD_WIDTH();
+      break;
+    case MI355_MAD_F64:
+      if (width == 1) mad_fp_kernel<double, 1><<<grid, block, 0, st>>>(seed, 1.0001, steps, n_items, (double *)out);
+      else if (width == 2) mad_fp_kernel<double, 2><<<grid, block, 0, st>>>(seed, 1.0001, steps, n_items, (double *)out);
+      else if (width == 4) mad_fp_kernel<double, 4><<<grid, block, 0, st>>>(seed, 1.0001, steps, n_items, (double *)out);
+      else BAD_WIDTH();
+      break;
+    case MI355_MAD_F16:  // a = 1 - 2^-10 (0x3bfe): 1.0001 itself rounds to 1.0 in half
+      if (width == 1) mad_f16_kernel<1><<<grid, block, 0, st>>>(seed, 0x3bfe, steps, n_items, (uint16_t *)out);
+      else if (width == 2) mad_f16_kernel<2><<<grid, block, 0, st>>>(seed, 0x3bfe, steps, n_items, (uint16_t *)out);
+      else BAD_WIDTH();
+      break;
+    case MI355_MAD_MP:
+      if (width != 1) BAD_WIDTH();
+      mad_mixed_kernel<true><<<grid, block, 0, st>>>(seed, 0x3bfe, steps, n_items, (float *)out);
+      break;
+    case MI355_MAD_BF16:  // a = 1 - 2^-8 (0x3f7f)
+      if (width != 1) BAD_WIDTH();
+      mad_mixed_kernel<false><<<grid, block, 0, st>>>(seed, 0x3f7f, steps, n_items, (float *)out);
+      break;
+    case MI355_MAD_I32:
+      if (width == 1) mad_i32_kernel<1><<<grid, block, 0, st>>>(seed, 3u, steps, n_items, (uint32_t *)out);
+      else if (width == 2) mad_i32_kernel<2><<<grid, block, 0, st>>>(seed, 3u, steps, n_items, (uint32_t *)out);
+      else if (width == 4) mad_i32_kernel<4><<<grid, block, 0, st>>>(seed, 3u, steps, n_items, (uint32_t *)out);
+      else BAD_WIDTH();
+      break;
+    case MI355_MAD_I8DP:
+      if (width == 1) mad_i8dp_kernel<1><<<grid, block, 0, st>>>(seed, steps, n_items, (int32_t *)out);
+      else if (width == 2) mad_i8dp_kernel<2><<<grid, block, 0, st>>>(seed, steps, n_items, (int32_t *)out);
+      else if (width == 4) mad_i8dp_kernel<4><<<grid, block, 0, st>>>(seed, steps, n_items, (int32_t *)out);
+      else if (width == 8) mad_i8dp_kernel<8><<<grid, block, 0, st>>>(seed, steps, n_items, (int32_t *)out);
+      else BAD_WIDTH();
+      break;
+    default:
+      return mi355_fail(dev, MI355_ERR_ARG, "compute_mad: unknown kind %d", kind);
+  }
+#undef BAD_WIDTH
+  MI355_LAUNCH_CHECK(dev, "compute_mad");
+  return MI355_OK;
+}

@@ -1,0 +1,49 @@
+// Operand layouts of the gfx950 matrix instructions, as used by every MFMA/SMFMAC
+// kernel of this backend.  Lanes are numbered 0..63 within a wavefront.
+//
+// 16x16xK shapes (K = 32 f16/bf16, 64 i8, 128 f8f6f4):
+//   A operand: lane l holds row (l % 16), K elements [ (l/16)*K/4 , (l/16+1)*K/4 ), low
+//              element in the low bits of the first register.
+//   B operand: lane l holds column (l % 16), same K range.
+//   C/D:       register r of lane l is element (row 4*(l/16) + r, column l % 16).
+// 32x32x16 f16/bf16:
+//   A operand: lane l holds row (l % 32), K elements [ (l/32)*8, (l/32)*8 + 8 ).
+//   B operand: lane l holds column (l % 32), same K range.
+//   C/D:       register r (0..15) of lane l is element
+//              (row 8*(r/4) + 4*(l/32) + r%4, column l % 32).
+// Scaled f8f6f4, 16x16x128: lane l carries the E8M0 scale of its own 32-element K
+//   block (row/column l % 16, block l/16) in the byte of the scale register that
+//   op_sel names.
+// SMFMAC 16x16xK (K = 64 for 16-bit, 128 for 8-bit data): A holds the K/2 kept values
+//   of row (l % 16): lane l has kept values [ (l/16)*K/8, (l/16+1)*K/8 ), which belong
+//   to dense K range [ (l/16)*K/4, (l/16+1)*K/4 ) -- the range of B that lane l/16
+//   group holds.  The index register carries two 2-bit positions per group of four,
+//   first kept value in the lower bits, groups in K order from bit 0.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef _Float16 half8v  __attribute__((ext_vector_type(8)));
+typedef _Float16 half16v __attribute__((ext_vector_type(16)));
+typedef __bf16   bf16x8v  __attribute__((ext_vector_type(8)));
+typedef __bf16   bf16x16v __attribute__((ext_vector_type(16)));
+typedef float    f32x4v  __attribute__((ext_vector_type(4)));
+typedef float    f32x16v __attribute__((ext_vector_type(16)));
+typedef int      i32x4v  __attribute__((ext_vector_type(4)));
+typedef int      i32x8v  __attribute__((ext_vector_type(8)));
+typedef int      i32x16v __attribute__((ext_vector_type(16)));
+
+// f8f6f4 format selectors (cbsz for A, blgp for B).
+#define MI355_F8F6F4_E4M3 0
+#define MI355_F8F6F4_E5M2 1
+#define MI355_F8F6F4_E2M3 2
+#define MI355_F8F6F4_E3M2 3
+#define MI355_F8F6F4_E2M1 4
+
+// Unaligned-safe vector loads from byte addresses (operands are only element aligned).
+template <typename V>
+__device__ inline V load_bytes(const uint8_t *p) {
+  V v;
+  __builtin_memcpy(&v, p, sizeof(V));
+  return v;
+}

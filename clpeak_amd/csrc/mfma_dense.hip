@@ -1,0 +1,201 @@
+// Dense MFMA throughput kernels, register resident.
+//
+// One workgroup = 4 wavefronts (one per SIMD of a CU); the default launch of 2048
+// waves puts 2 waves on every SIMD of a 256-CU part.  Each wave loads the fragments
+// of its 4 chains from the logical A/B matrices once, then issues
+//     acc[c] = MFMA(a[c], b[c], acc[c])        c = 0..3, `iters` times
+// so that 4 independent accumulator tiles are always in flight and a dependent
+// MFMA never waits for its predecessor.  The final accumulator tiles are written
+// to memory in row-major order.  MFMA-bound: 2*M*N*K flops per instruction, no
+// memory traffic inside the loop.
+#include "internal.h"
+#include "mfma_common.h"
+
+namespace {
+
+constexpr int kChains = 4;
+
+// The hot loop is written as inline assembly: with the builtins the register
+// allocator rotates the accumulator tiles through copies on every trip, and each
+// copy next to an MFMA costs wait states.  One block = kBlock rounds over the 4
+// chains, accumulating in place (vDst == SrcC), which the matrix pipe executes
+// back to back with no software wait states: the next MFMA that touches the same
+// accumulator is 3 independent MFMAs away.
+constexpr int kBlock = 8;
+
+#define MI355_REP8(x) x x x x x x x x
+// %0-%3 accumulators, %4-%7 A fragments, %8-%11 B fragments
+#define MI355_ROUND(INSN, TAIL)                \
+  INSN " %0, %4, %8, %0" TAIL "\n"             \
+  INSN " %1, %5, %9, %1" TAIL "\n"             \
+  INSN " %2, %6, %10, %2" TAIL "\n"            \
+  INSN " %3, %7, %11, %3" TAIL "\n"
+// scaled: %12-%15 scale A, %16-%19 scale B
+#define MI355_ROUND_SCALED(INSN, TAIL)                   \
+  INSN " %0, %4, %8, %0, %12, %16 op_sel_hi:[0,0,0]" TAIL "\n"   \
+  INSN " %1, %5, %9, %1, %13, %17 op_sel_hi:[0,0,0]" TAIL "\n"   \
+  INSN " %2, %6, %10, %2, %14, %18 op_sel_hi:[0,0,0]" TAIL "\n"  \
+  INSN " %3, %7, %11, %3, %15, %19 op_sel_hi:[0,0,0]" TAIL "\n"
+
+#define MI355_DEFINE_STEPS(INSN, TAIL)                                                             \
+  __device__ static void block(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&)[4], \
+                               const int (&)[4]) {                                                 \
+    asm volatile(MI355_REP8(MI355_ROUND(INSN, TAIL))                                               \
+                 : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
+                 : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3])); \
+  }                                                                                                \
+  __device__ static void single(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&)[4], \
+                                const int (&)[4]) {                                                \
+    asm volatile(MI355_ROUND(INSN, TAIL)                                                           \
+                 : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
+                 : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3])); \
+  }
+
+#define MI355_DEFINE_STEPS_SCALED(INSN, TAIL)                                                      \
+  __device__ static void block(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&sa)[4], \
+                               const int (&sb)[4]) {                                               \
+    asm volatile(MI355_REP8(MI355_ROUND_SCALED(INSN, TAIL))                                        \
+                 : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
+                 : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), \
+                   "v"(sa[0]), "v"(sa[1]), "v"(sa[2]), "v"(sa[3]), "v"(sb[0]), "v"(sb[1]), "v"(sb[2]), "v"(sb[3])); \
+  }                                                                                                \
+  __device__ static void single(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&sa)[4], \
+                                const int (&sb)[4]) {                                              \
+    asm volatile(MI355_ROUND_SCALED(INSN, TAIL)                                                    \
+                 : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
+                 : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), \
+                   "v"(sa[0]), "v"(sa[1]), "v"(sa[2]), "v"(sa[3]), "v"(sb[0]), "v"(sb[1]), "v"(sb[2]), "v"(sb[3])); \
+  }
+
+// ---- per-kind traits ---------------------------------------------------------
+// Each trait supplies: tile shape, bytes per K-contiguous row, register types, how a
+// lane loads its fragment from a logical row, and the instruction blocks.
+
+typedef int i32x6v __attribute__((ext_vector_type(6)));
+
+// A lane's fragment is `bytes` contiguous bytes of its row, starting at chunk * bytes.
+template <typename Frag, int ROWS_MOD, int ROW_BYTES, int BYTES>
+__device__ inline Frag load_fragment(const uint8_t *rows, int lane) {
+  return load_bytes<Frag>(rows + (lane % ROWS_MOD) * ROW_BYTES + (lane / ROWS_MOD) * BYTES);
+}
+
+#define MI355_DENSE_TRAIT(NAME, M_, N_, K_, ROW_BYTES, FRAG, ACC, OUT, INSN)                       \
+  struct NAME {                                                                                    \
+    static constexpr int M = M_, N = N_, K = K_, row_bytes = ROW_BYTES, acc_regs = M_ * N_ / 64;   \
+    static constexpr bool scaled = false;                                                          \
+    using Frag = FRAG; using Acc = ACC; using Out = OUT;                                           \
+    __device__ static Frag load(const uint8_t *rows, int lane) {                                   \
+      return load_fragment<Frag, M_, ROW_BYTES, 16>(rows, lane);                                   \
+    }                                                                                              \
+    MI355_DEFINE_STEPS(INSN, "")                                                                   \
+  };
+
+MI355_DENSE_TRAIT(F16_16x16x32, 16, 16, 32, 64, half8v, f32x4v, float, "v_mfma_f32_16x16x32_f16")
+MI355_DENSE_TRAIT(BF16_16x16x32, 16, 16, 32, 64, bf16x8v, f32x4v, float, "v_mfma_f32_16x16x32_bf16")
+MI355_DENSE_TRAIT(F16_32x32x16, 32, 32, 16, 32, half8v, f32x16v, float, "v_mfma_f32_32x32x16_f16")
+MI355_DENSE_TRAIT(BF16_32x32x16, 32, 32, 16, 32, bf16x8v, f32x16v, float, "v_mfma_f32_32x32x16_bf16")
+MI355_DENSE_TRAIT(I8_16x16x64, 16, 16, 64, 64, i32x4v, i32x4v, int32_t, "v_mfma_i32_16x16x64_i8")
+
+// f8f6f4, 16x16x128: a lane's 32 elements are BITS*4 bytes in BITS/... registers
+// (8 for 8-bit, 6 for 6-bit, 4 for 4-bit codes); cbsz / blgp name the A / B format.
+#define MI355_F8F6F4_TRAIT(NAME, BITS, FRAG, SCALED, TAIL)                                         \
+  struct NAME {                                                                                    \
+    static constexpr int M = 16, N = 16, K = 128, row_bytes = 128 * BITS / 8, acc_regs = 4;        \
+    static constexpr bool scaled = SCALED;                                                         \
+    using Frag = FRAG; using Acc = f32x4v; using Out = float;                                      \
+    __device__ static Frag load(const uint8_t *rows, int lane) {                                   \
+      return load_fragment<Frag, 16, row_bytes, BITS * 4>(rows, lane);                             \
+    }                                                                                              \
+    MI355_DEFINE_STEPS_SCALED("v_mfma_scale_f32_16x16x128_f8f6f4", TAIL)                           \
+  };
+
+MI355_F8F6F4_TRAIT(FP8_16x16x128, 8, i32x8v, false, "")
+MI355_F8F6F4_TRAIT(BF8_16x16x128, 8, i32x8v, false, " cbsz:1 blgp:1")
+MI355_F8F6F4_TRAIT(FP6_E2M3_16x16x128, 6, i32x6v, true, " cbsz:2 blgp:2")
+MI355_F8F6F4_TRAIT(FP6_E3M2_16x16x128, 6, i32x6v, true, " cbsz:3 blgp:3")
+MI355_F8F6F4_TRAIT(FP4_E2M1_16x16x128, 4, i32x4v, true, " cbsz:4 blgp:4")
+
+template <typename Tr>
+__global__ void __launch_bounds__(256)
+mfma_dense_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B,
+                  const uint8_t *__restrict__ sA, const uint8_t *__restrict__ sB,
+                  typename Tr::Out *__restrict__ out, uint32_t iters) {
+  const int lane = threadIdx.x % 64;
+  const uint64_t wave = (uint64_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
+  constexpr size_t a_bytes = (size_t)Tr::M * Tr::row_bytes, b_bytes = (size_t)Tr::N * Tr::row_bytes;
+
+  typename Tr::Frag a[kChains], b[kChains];
+  typename Tr::Acc acc[kChains];
+  int sa[kChains], sb[kChains];
+#pragma unroll
+  for (int c = 0; c < kChains; c++) {
+    const uint64_t u = wave * kChains + c;
+    a[c] = Tr::load(A + u * a_bytes, lane);
+    b[c] = Tr::load(B + u * b_bytes, lane);
+    if constexpr (Tr::scaled) {
+      // scale[wave][chain][row][K/32]: this lane's row (lane%16) and K block (lane/16).
+      sa[c] = sA[(u * Tr::M + lane % 16) * (Tr::K / 32) + lane / 16];
+      sb[c] = sB[(u * Tr::N + lane % 16) * (Tr::K / 32) + lane / 16];
+    } else {
+      sa[c] = 0x7f;  // E8M0 1.0
+      sb[c] = 0x7f;
+    }
+#pragma unroll
+    for (int r = 0; r < Tr::acc_regs; r++) acc[c][r] = 0;
+  }
+
+  const uint32_t blocks = iters / kBlock, rest = iters % kBlock;
+#pragma unroll 1
+  for (uint32_t it = 0; it < blocks; it++) Tr::block(acc, a, b, sa, sb);
+#pragma unroll 1
+  for (uint32_t it = 0; it < rest; it++) Tr::single(acc, a, b, sa, sb);
+  // The compiler cannot see the matrix instructions inside the asm blocks, so it will
+  // not insert the wait states a VALU/VMEM read of their results needs: cover the
+  // longest case (a 16-pass MFMA result read by a store) by hand.
+  asm volatile("s_nop 15\n s_nop 15" ::: "memory");
+
+#pragma unroll
+  for (int c = 0; c < kChains; c++) {
+    typename Tr::Out *tile = out + (wave * kChains + c) * (uint64_t)(Tr::M * Tr::N);
+    if constexpr (Tr::M == 16) {
+#pragma unroll
+      for (int r = 0; r < 4; r++) tile[(4 * (lane / 16) + r) * 16 + lane % 16] = acc[c][r];
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; r++) tile[(8 * (r / 4) + 4 * (lane / 32) + r % 4) * 32 + lane % 32] = acc[c][r];
+    }
+  }
+}
+
+template <typename Tr>
+int launch(mi355_dev *dev, const void *A, const void *B, const uint8_t *sA, const uint8_t *sB, void *out,
+           uint32_t waves, uint32_t iters) {
+  if (Tr::scaled && (!sA || !sB)) return mi355_fail(dev, MI355_ERR_ARG, "mfma_dense: scaled kind needs scaleA and scaleB");
+  mfma_dense_kernel<Tr><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)A, (const uint8_t *)B, sA, sB,
+                                                           (typename Tr::Out *)out, iters);
+  MI355_LAUNCH_CHECK(dev, "mfma_dense");
+  return MI355_OK;
+}
+
+}  // namespace
+
+extern "C" int mi355_mfma_dense(mi355_dev *dev, int kind, const void *A, const void *B, const uint8_t *scaleA,
+                                const uint8_t *scaleB, void *out, uint32_t waves, uint32_t iters) {
+  MI355_ENTER(dev);
+  MI355_REQUIRE(dev, A && B && out, "mfma_dense: null buffer");
+  MI355_REQUIRE(dev, waves > 0 && waves % 4 == 0, "mfma_dense: waves (%u) must be a positive multiple of 4", waves);
+  MI355_REQUIRE(dev, (((uintptr_t)A | (uintptr_t)B | (uintptr_t)out) & 15u) == 0, "mfma_dense: buffers must be 16-byte aligned");
+  switch (kind) {
+    case MI355_MFMA_F16_16x16x32:  return launch<F16_16x16x32>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_BF16_16x16x32: return launch<BF16_16x16x32>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_F16_32x32x16:  return launch<F16_32x32x16>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_BF16_32x32x16: return launch<BF16_32x32x16>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_I8_16x16x64:   return launch<I8_16x16x64>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_FP8_16x16x128: return launch<FP8_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_BF8_16x16x128: return launch<BF8_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_MXFP6_E2M3:    return launch<FP6_E2M3_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_MXFP6_E3M2:    return launch<FP6_E3M2_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_MXFP4_E2M1:    return launch<FP4_E2M1_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    default: return mi355_fail(dev, MI355_ERR_ARG, "mfma_dense: unknown kind %d", kind);
+  }
+}

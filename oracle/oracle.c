@@ -1,0 +1,585 @@
+/*
+ * oracle.c -- CPU restatement of the seeded workloads of the MI355X clpeak backend.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the product (the C-ABI library, the C++ host
+ * layer, the Python package) may include, link or call this file; only tests/,
+ * __graft_entry__.smoke() and the cpu_baseline leg of bench.py do, as the checker.
+ *
+ * What it restates and from where (paths relative to the reference checkout):
+ *  - read-reduce order of the bandwidth kernels: component-wise running sums, then
+ *    x+y+z+w left to right -- src/rocm/rocm_kernels/global_bandwidth.hip:19-26, 38-46, 58-66
+ *    (the stride pattern is the grid-stride one the workload configuration asks for,
+ *    not the reference's block-strided 16 fetches);
+ *  - the MAD chain "one multiply-add per statement, store the accumulator" --
+ *    include/common/common.h:60-97, src/rocm/rocm_kernels/compute_sp.hip:18-35,
+ *    compute_int8_dp.hip:37-53 (sdot4 + xor feedback);
+ *  - MFMA / SMFMAC op accounting 2*M*N*K per instruction, dense-equivalent K for
+ *    sparse -- src/rocm/mfma.cpp:158-161, src/rocm/sparse_mfma.cpp:141-144;
+ *  - GEMM operand convention (K contiguous in both operands, fp32 accumulate, bf16
+ *    out) -- src/rocm/hipblaslt_gemm.cpp:381-400.
+ * The reference never checks a kernel result (its kernels run on constants), so the
+ * numeric definitions here are this project's own; each is pinned by the checks in
+ * tests/test_oracle_*.py (known-answer vectors of SplitMix64, numpy/torch
+ * conversions of every narrow format, closed forms of the affine recurrence, brute
+ * force on small matrices).
+ *
+ * Everything is plain C, no fast-math, no contraction: build with oracle/Makefile.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------------- */
+/* Seeded generator                                                            */
+/* ------------------------------------------------------------------------- */
+
+uint64_t orc_rng_word(uint64_t seed, uint32_t stream, uint64_t i)
+{
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull * (i + 1) + 0xD6E8FEB86659FD93ull * (uint64_t)stream;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+static float u01_of(uint64_t z) { return (float)(uint32_t)(z >> 40) / 16777216.0f; }
+static float upm1_of(uint64_t z) { return (float)((int32_t)(uint32_t)(z >> 40) - 8388608) / 8388608.0f; }
+
+float orc_u01(uint64_t seed, uint32_t stream, uint64_t i) { return u01_of(orc_rng_word(seed, stream, i)); }
+float orc_upm1(uint64_t seed, uint32_t stream, uint64_t i) { return upm1_of(orc_rng_word(seed, stream, i)); }
+
+/* integer uniform in [0,m) from the high 32 bits */
+uint32_t orc_below(uint64_t seed, uint32_t stream, uint64_t i, uint32_t m)
+{
+    return (uint32_t)(((orc_rng_word(seed, stream, i) >> 32) * (uint64_t)m) >> 32);
+}
+
+/* Standard normal by Box-Muller on two words (2i, 2i+1) of the stream, in double. */
+double orc_normal(uint64_t seed, uint32_t stream, uint64_t i)
+{
+    const uint64_t z1 = orc_rng_word(seed, stream, 2 * i);
+    const uint64_t z2 = orc_rng_word(seed, stream, 2 * i + 1);
+    const double u1 = ((double)(z1 >> 11) + 1.0) * 0x1.0p-53; /* (0,1] */
+    const double u2 = (double)(z2 >> 11) * 0x1.0p-53;         /* [0,1) */
+    return sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2);
+}
+
+void orc_fill_f32(float *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist, uint64_t first)
+{
+    for (uint64_t i = 0; i < n; i++) {
+        const uint64_t z = orc_rng_word(seed, stream, first + i);
+        dst[i] = dist == 0 ? u01_of(z) : upm1_of(z);
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Narrow formats: closed-form decode, encode by nearest-value search          */
+/* ------------------------------------------------------------------------- */
+/* A format is (E exponent bits, M mantissa bits, bias, ieee_specials).
+ * ieee_specials: 1 = top exponent is Inf/NaN (f16, e5m2); 2 = only S.1111.111 is NaN
+ * (e4m3fn); 0 = every code is finite (fp6, fp4). */
+typedef struct { int E, M, bias, specials, saturate; } orc_fmt;
+
+static const orc_fmt FMT_F16  = {5, 10, 15, 1, 0};
+static const orc_fmt FMT_BF16 = {8, 7, 127, 1, 0};
+static const orc_fmt FMT_E4M3 = {4, 3, 7, 2, 1};
+static const orc_fmt FMT_E5M2 = {5, 2, 15, 1, 1};
+static const orc_fmt FMT_E2M3 = {2, 3, 1, 0, 1};
+static const orc_fmt FMT_E3M2 = {3, 2, 3, 0, 1};
+static const orc_fmt FMT_E2M1 = {2, 1, 1, 0, 1};
+
+static const orc_fmt *fmt_by_id(int id)
+{
+    switch (id) {
+    case 0: return &FMT_F16;
+    case 1: return &FMT_BF16;
+    case 2: return &FMT_E4M3;
+    case 3: return &FMT_E5M2;
+    case 4: return &FMT_E2M3;
+    case 5: return &FMT_E3M2;
+    case 6: return &FMT_E2M1;
+    default: return NULL;
+    }
+}
+
+static uint32_t fmt_max_finite(const orc_fmt *f)
+{
+    const uint32_t all = (1u << (f->E + f->M)) - 1u;
+    if (f->specials == 1) return all - (1u << f->M);       /* exponent all-ones reserved */
+    if (f->specials == 2) return all - 1u;                  /* only the last code is NaN  */
+    return all;
+}
+
+static double fmt_decode_mag(const orc_fmt *f, uint32_t mag)
+{
+    const uint32_t e = mag >> f->M, m = mag & ((1u << f->M) - 1u);
+    if (e == 0) return ldexp((double)m, 1 - f->bias - f->M);
+    return ldexp((double)((1u << f->M) | m), (int)e - f->bias - f->M);
+}
+
+static double fmt_decode(const orc_fmt *f, uint32_t code)
+{
+    const uint32_t sbit = 1u << (f->E + f->M);
+    const uint32_t mag = code & (sbit - 1u);
+    const double s = (code & sbit) ? -1.0 : 1.0;
+    if (mag > fmt_max_finite(f)) {
+        if (f->specials == 1 && (mag & ((1u << f->M) - 1u)) == 0) return s * INFINITY;
+        return NAN;
+    }
+    return s * fmt_decode_mag(f, mag);
+}
+
+/* Nearest finite code to x, ties to the even code; saturating formats clamp to the
+ * largest finite code, the IEEE ones (f16, bf16) round to infinity from the halfway
+ * point past it. */
+static uint32_t fmt_encode(const orc_fmt *f, double x)
+{
+    const uint32_t sbit = 1u << (f->E + f->M);
+    const uint32_t s = signbit(x) ? sbit : 0u;
+    const double ax = fabs(x);
+    const uint32_t maxc = fmt_max_finite(f);
+    if (isnan(x)) return s | maxc;
+    const double maxv = fmt_decode_mag(f, maxc);
+    if (ax >= maxv) {
+        if (!f->saturate) {
+            const double step = maxv - fmt_decode_mag(f, maxc - 1);
+            if (ax >= maxv + step / 2) return s | (maxc + 1); /* infinity */
+        }
+        return s | maxc;
+    }
+    uint32_t lo = 0, hi = maxc; /* decode(lo) <= ax < decode(hi) */
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) / 2;
+        if (fmt_decode_mag(f, mid) <= ax) lo = mid; else hi = mid;
+    }
+    const double dl = ax - fmt_decode_mag(f, lo), dh = fmt_decode_mag(f, hi) - ax;
+    uint32_t pick;
+    if (dl < dh) pick = lo;
+    else if (dh < dl) pick = hi;
+    else pick = (lo & 1u) ? hi : lo;
+    return s | pick;
+}
+
+/* format ids: 0 f16, 1 bf16, 2 e4m3fn, 3 e5m2, 4 e2m3, 5 e3m2, 6 e2m1 */
+double orc_decode(int fmt, uint32_t code)
+{
+    const orc_fmt *f = fmt_by_id(fmt);
+    return f ? fmt_decode(f, code) : NAN;
+}
+
+uint32_t orc_encode(int fmt, double x)
+{
+    const orc_fmt *f = fmt_by_id(fmt);
+    return f ? fmt_encode(f, x) : 0;
+}
+
+double orc_e8m0(uint32_t byte) { return byte == 0xff ? NAN : ldexp(1.0, (int)byte - 127); }
+
+/* ------------------------------------------------------------------------- */
+/* Global bandwidth read-reduce                                                */
+/* ------------------------------------------------------------------------- */
+/* T threads; thread t adds vectors t, t+T, ... component-wise in that order, then
+ * combines ((x+y)+z)+w.  Swept in memory order, which visits each thread's vectors
+ * in the same order as the strided walk does. */
+void orc_global_bandwidth(int width, const float *in, uint64_t n_floats, uint64_t T, float *out)
+{
+    const uint64_t nvec = n_floats / (uint64_t)width;
+    float *acc = (float *)calloc((size_t)T * (size_t)width, sizeof(float));
+    for (uint64_t i = 0; i < nvec; i++) {
+        float *a = acc + (i % T) * (uint64_t)width;
+        const float *v = in + i * (uint64_t)width;
+        for (int c = 0; c < width; c++) a[c] = a[c] + v[c];
+    }
+    for (uint64_t t = 0; t < T; t++) {
+        const float *a = acc + t * (uint64_t)width;
+        float s = a[0];
+        for (int c = 1; c < width; c++) s = s + a[c];
+        out[t] = s;
+    }
+    free(acc);
+}
+
+/* Same partial for one thread, with the buffer regenerated from the seed (uniform
+ * [0,1), stream `stream`): lets a test check sampled threads of a buffer too large
+ * to hold on the host. */
+float orc_global_bandwidth_thread(int width, uint64_t seed, uint32_t stream, uint64_t n_floats,
+                                  uint64_t T, uint64_t t)
+{
+    const uint64_t nvec = n_floats / (uint64_t)width;
+    float a[4] = {0, 0, 0, 0};
+    for (uint64_t i = t; i < nvec; i += T)
+        for (int c = 0; c < width; c++) a[c] = a[c] + u01_of(orc_rng_word(seed, stream, i * (uint64_t)width + c));
+    float s = a[0];
+    for (int c = 1; c < width; c++) s = s + a[c];
+    return s;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Vector MAD chains                                                           */
+/* ------------------------------------------------------------------------- */
+enum { MAD_F32 = 0, MAD_F16 = 1, MAD_F64 = 2, MAD_MP = 3, MAD_BF16 = 4, MAD_I32 = 5, MAD_I8DP = 6 };
+#define STREAM_MAD 1u
+#define STREAM_MAD_Y 9u
+
+static int32_t sdot4(uint32_t x, uint32_t y, int32_t acc)
+{
+    uint32_t r = (uint32_t)acc;
+    for (int b = 0; b < 4; b++) {
+        const int32_t xb = (int8_t)(x >> (8 * b)), yb = (int8_t)(y >> (8 * b));
+        r += (uint32_t)(xb * yb);
+    }
+    return (int32_t)r;
+}
+
+/* items [first, first+n): out is n elements of the kind's output type.
+ * `width` only matters for MAD_I8DP, where it is the number of chains. */
+int orc_compute_mad(int kind, int width, uint64_t seed, uint64_t first, uint64_t n, uint32_t steps, void *out)
+{
+    #pragma omp parallel for schedule(static)
+    for (uint64_t q = 0; q < n; q++) {
+        const uint64_t item = first + q;
+        switch (kind) {
+        case MAD_F32: {
+            float x0[16], x[16];
+            for (int j = 0; j < 16; j++) x[j] = x0[j] = upm1_of(orc_rng_word(seed, STREAM_MAD, item * 16 + j));
+            const float a = 1.0001f;
+            for (uint32_t s = 0; s < steps; s++)
+                for (int j = 0; j < 16; j++) x[j] = __builtin_fmaf(x[j], a, x0[j]);
+            float sum = 0.0f;
+            for (int j = 0; j < 16; j++) sum = sum + x[j];
+            ((float *)out)[q] = sum;
+            break;
+        }
+        case MAD_F64: {
+            double x0[16], x[16];
+            for (int j = 0; j < 16; j++) x[j] = x0[j] = (double)upm1_of(orc_rng_word(seed, STREAM_MAD, item * 16 + j));
+            const double a = 1.0001;
+            for (uint32_t s = 0; s < steps; s++)
+                for (int j = 0; j < 16; j++) x[j] = __builtin_fma(x[j], a, x0[j]);
+            double sum = 0.0;
+            for (int j = 0; j < 16; j++) sum = sum + x[j];
+            ((double *)out)[q] = sum;
+            break;
+        }
+        case MAD_F16: {
+            /* half FMA = exact a*b+c rounded once to half.  |x| stays below 2^11 and every
+             * operand is a multiple of 2^-24, so the exact value needs < 53 bits: the double
+             * FMA below is exact and fmt_encode does the single rounding. */
+            double x0[16], x[16];
+            const double a = 1.0 - 0x1.0p-10;
+            for (int j = 0; j < 16; j++) {
+                const uint32_t c = fmt_encode(&FMT_F16, (double)upm1_of(orc_rng_word(seed, STREAM_MAD, item * 16 + j)));
+                x[j] = x0[j] = fmt_decode(&FMT_F16, c);
+            }
+            for (uint32_t s = 0; s < steps; s++)
+                for (int j = 0; j < 16; j++) x[j] = fmt_decode(&FMT_F16, fmt_encode(&FMT_F16, __builtin_fma(x[j], a, x0[j])));
+            double sum = 0.0;
+            for (int j = 0; j < 16; j++) sum = fmt_decode(&FMT_F16, fmt_encode(&FMT_F16, sum + x[j]));
+            ((uint16_t *)out)[q] = (uint16_t)fmt_encode(&FMT_F16, sum);
+            break;
+        }
+        case MAD_MP:
+        case MAD_BF16: {
+            float xn[16], acc[16];
+            const float a = kind == MAD_MP ? (float)(1.0 - 0x1.0p-10) : (float)(1.0 - 0x1.0p-8);
+            for (int j = 0; j < 16; j++) {
+                const double u = (double)upm1_of(orc_rng_word(seed, STREAM_MAD, item * 16 + j));
+                xn[j] = (float)(kind == MAD_MP ? fmt_decode(&FMT_F16, fmt_encode(&FMT_F16, u))
+                                               : fmt_decode(&FMT_BF16, fmt_encode(&FMT_BF16, u)));
+                acc[j] = xn[j];
+            }
+            for (uint32_t s = 0; s < steps; s++)
+                for (int j = 0; j < 16; j++) acc[j] = __builtin_fmaf(xn[j], a, acc[j]);
+            float sum = 0.0f;
+            for (int j = 0; j < 16; j++) sum = sum + acc[j];
+            ((float *)out)[q] = sum;
+            break;
+        }
+        case MAD_I32: {
+            uint32_t x0[16], x[16];
+            for (int j = 0; j < 16; j++) x[j] = x0[j] = (uint32_t)(orc_rng_word(seed, STREAM_MAD, item * 16 + j) >> 32);
+            for (uint32_t s = 0; s < steps; s++)
+                for (int j = 0; j < 16; j++) x[j] = x[j] * 3u + x0[j];
+            uint32_t sum = 0;
+            for (int j = 0; j < 16; j++) sum += x[j];
+            ((uint32_t *)out)[q] = sum;
+            break;
+        }
+        case MAD_I8DP: {
+            uint32_t sum = 0;
+            for (int c = 0; c < width; c++) {
+                const uint32_t x = (uint32_t)(orc_rng_word(seed, STREAM_MAD, item * 8 + c) >> 32);
+                uint32_t y = (uint32_t)(orc_rng_word(seed, STREAM_MAD_Y, item * 8 + c) >> 32);
+                int32_t acc = 0;
+                for (uint32_t s = 0; s < steps; s++) {
+                    acc = sdot4(x, y, acc);
+                    y ^= (uint32_t)acc;
+                }
+                sum += (uint32_t)acc;
+            }
+            ((int32_t *)out)[q] = (int32_t)sum;
+            break;
+        }
+        default:
+            break;
+        }
+    }
+    return (kind >= MAD_F32 && kind <= MAD_I8DP) ? 0 : -1;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Matrix instructions on logical operands                                     */
+/* ------------------------------------------------------------------------- */
+/* dense kinds (same numbering as the C ABI) */
+enum {
+    MF_F16_16 = 0, MF_BF16_16 = 1, MF_F16_32 = 2, MF_BF16_32 = 3, MF_I8 = 4,
+    MF_FP8 = 5, MF_BF8 = 6, MF_FP6_E2M3 = 7, MF_FP6_E3M2 = 8, MF_FP4 = 9
+};
+
+typedef struct { int M, N, K, fmt, bits, scaled, is_int; } mf_shape;
+
+static int mf_shape_of(int kind, mf_shape *s)
+{
+    switch (kind) {
+    case MF_F16_16:  *s = (mf_shape){16, 16, 32, 0, 16, 0, 0}; return 0;
+    case MF_BF16_16: *s = (mf_shape){16, 16, 32, 1, 16, 0, 0}; return 0;
+    case MF_F16_32:  *s = (mf_shape){32, 32, 16, 0, 16, 0, 0}; return 0;
+    case MF_BF16_32: *s = (mf_shape){32, 32, 16, 1, 16, 0, 0}; return 0;
+    case MF_I8:      *s = (mf_shape){16, 16, 64, -1, 8, 0, 1}; return 0;
+    case MF_FP8:     *s = (mf_shape){16, 16, 128, 2, 8, 0, 0}; return 0;
+    case MF_BF8:     *s = (mf_shape){16, 16, 128, 3, 8, 0, 0}; return 0;
+    case MF_FP6_E2M3:*s = (mf_shape){16, 16, 128, 4, 6, 1, 0}; return 0;
+    case MF_FP6_E3M2:*s = (mf_shape){16, 16, 128, 5, 6, 1, 0}; return 0;
+    case MF_FP4:     *s = (mf_shape){16, 16, 128, 6, 4, 1, 0}; return 0;
+    default: return -1;
+    }
+}
+
+/* Element k of a K-contiguous row of `bits`-wide codes, little-endian bit order. */
+static uint32_t packed_get(const uint8_t *row, int bits, int k)
+{
+    const uint32_t bit = (uint32_t)k * (uint32_t)bits, byte = bit >> 3, sh = bit & 7u;
+    uint32_t v = row[byte];
+    if (sh + (uint32_t)bits > 8) v |= (uint32_t)row[byte + 1] << 8;
+    if (sh + (uint32_t)bits > 16) v |= (uint32_t)row[byte + 2] << 16;
+    return (v >> sh) & ((1u << bits) - 1u);
+}
+
+static size_t row_bytes(int K, int bits) { return (size_t)K * (size_t)bits / 8; }
+
+/* One (wave, chain): out[M][N] after `iters` accumulations.  P = exact dot product
+ * (double; every product of two narrow values and every power-of-two scale is exact,
+ * and a sum of <=128 such terms stays far inside 53 bits for the seeded ranges), then
+ * acc <- fl32(acc + P) `iters` times.  abs_out (optional) gets iters * sum|a*b|, the
+ * scale against which a tolerance is stated. */
+static void mf_tile(const mf_shape *s, const uint8_t *A, const uint8_t *B, const uint8_t *sA, const uint8_t *sB,
+                    uint32_t iters, void *out, double *abs_out)
+{
+    const size_t rb = row_bytes(s->K, s->bits);
+    for (int m = 0; m < s->M; m++)
+        for (int n = 0; n < s->N; n++) {
+            const uint8_t *ar = A + (size_t)m * rb, *br = B + (size_t)n * rb;
+            if (s->is_int) {
+                int64_t p = 0;
+                for (int k = 0; k < s->K; k++) p += (int64_t)(int8_t)ar[k] * (int64_t)(int8_t)br[k];
+                uint32_t acc = 0;
+                for (uint32_t t = 0; t < iters; t++) acc += (uint32_t)(int32_t)p;
+                ((int32_t *)out)[m * s->N + n] = (int32_t)acc;
+                if (abs_out) abs_out[m * s->N + n] = 0.0;
+                continue;
+            }
+            double p = 0.0, pa = 0.0;
+            for (int k0 = 0; k0 < s->K; k0 += 32) {
+                double bs = 1.0;
+                if (s->scaled) bs = orc_e8m0(sA[m * (s->K / 32) + k0 / 32]) * orc_e8m0(sB[n * (s->K / 32) + k0 / 32]);
+                double q = 0.0, qa = 0.0;
+                const int kend = k0 + 32 < s->K ? k0 + 32 : s->K;
+                for (int k = k0; k < kend; k++) {
+                    const double a = orc_decode(s->fmt, packed_get(ar, s->bits, k));
+                    const double b = orc_decode(s->fmt, packed_get(br, s->bits, k));
+                    q += a * b;
+                    qa += fabs(a * b);
+                }
+                p += bs * q;
+                pa += bs * qa;
+            }
+            float acc = 0.0f;
+            for (uint32_t t = 0; t < iters; t++) acc = (float)((double)acc + p);
+            ((float *)out)[m * s->N + n] = acc;
+            if (abs_out) abs_out[m * s->N + n] = pa * (double)iters;
+        }
+}
+
+/* Layout as in the C ABI: A[wave][chain][M][K], B[wave][chain][N][K], scales
+ * [wave][chain][M|N][K/32], out[wave][chain][M][N]; 4 chains per wave. */
+int orc_mfma_dense(int kind, const void *A, const void *B, const uint8_t *scaleA, const uint8_t *scaleB,
+                   void *out, double *abs_out, uint32_t waves, uint32_t iters)
+{
+    mf_shape s;
+    if (mf_shape_of(kind, &s)) return -1;
+    const size_t a_sz = (size_t)s.M * row_bytes(s.K, s.bits), b_sz = (size_t)s.N * row_bytes(s.K, s.bits);
+    const size_t sa_sz = (size_t)s.M * (size_t)(s.K / 32), sb_sz = (size_t)s.N * (size_t)(s.K / 32);
+    const size_t o_n = (size_t)s.M * (size_t)s.N;
+    #pragma omp parallel for schedule(static)
+    for (uint64_t u = 0; u < (uint64_t)waves * 4; u++) {
+        mf_tile(&s, (const uint8_t *)A + u * a_sz, (const uint8_t *)B + u * b_sz,
+                s.scaled ? scaleA + u * sa_sz : NULL, s.scaled ? scaleB + u * sb_sz : NULL, iters,
+                (uint8_t *)out + u * o_n * 4, abs_out ? abs_out + u * o_n : NULL);
+    }
+    return 0;
+}
+
+/* sparse kinds (same numbering as the C ABI) */
+enum { SP_F16 = 0, SP_BF16 = 1, SP_FP8 = 2, SP_BF8 = 3, SP_I8 = 4 };
+
+/* Ac[wave][chain][16][K/2], meta[wave][chain][16][K/4], B[wave][chain][16][K]:
+ * decompress A with the metadata (bits[1:0] = slot of the first kept value, bits[3:2]
+ * = slot of the second) and run the dense product. */
+int orc_smfmac(int kind, const void *Ac, const uint8_t *meta, const void *B, void *out, double *abs_out,
+               uint32_t waves, uint32_t iters)
+{
+    mf_shape s;
+    switch (kind) {
+    case SP_F16:  s = (mf_shape){16, 16, 64, 0, 16, 0, 0}; break;
+    case SP_BF16: s = (mf_shape){16, 16, 64, 1, 16, 0, 0}; break;
+    case SP_FP8:  s = (mf_shape){16, 16, 128, 2, 8, 0, 0}; break;
+    case SP_BF8:  s = (mf_shape){16, 16, 128, 3, 8, 0, 0}; break;
+    case SP_I8:   s = (mf_shape){16, 16, 128, -1, 8, 0, 1}; break;
+    default: return -1;
+    }
+    const int eb = s.bits / 8;
+    const size_t ac_sz = (size_t)16 * (size_t)(s.K / 2) * (size_t)eb, b_sz = (size_t)16 * (size_t)s.K * (size_t)eb;
+    const size_t m_sz = (size_t)16 * (size_t)(s.K / 4), o_n = 256;
+    int bad = 0;
+    #pragma omp parallel for schedule(static)
+    for (uint64_t u = 0; u < (uint64_t)waves * 4; u++) {
+        uint8_t dense[16 * 128 * 2];
+        memset(dense, 0, sizeof(dense));
+        const uint8_t *ac = (const uint8_t *)Ac + u * ac_sz, *mt = meta + u * m_sz;
+        for (int m = 0; m < 16; m++)
+            for (int g = 0; g < s.K / 4; g++) {
+                const uint8_t md = mt[m * (s.K / 4) + g];
+                const int p0 = md & 3, p1 = (md >> 2) & 3;
+                if (p0 == p1) bad = 1;
+                memcpy(dense + ((size_t)m * s.K + 4 * g + p0) * eb, ac + ((size_t)m * (s.K / 2) + 2 * g) * eb, (size_t)eb);
+                memcpy(dense + ((size_t)m * s.K + 4 * g + p1) * eb, ac + ((size_t)m * (s.K / 2) + 2 * g + 1) * eb, (size_t)eb);
+            }
+        mf_tile(&s, dense, (const uint8_t *)B + u * b_sz, NULL, NULL, iters, (uint8_t *)out + u * o_n * 4,
+                abs_out ? abs_out + u * o_n : NULL);
+    }
+    return bad ? -2 : 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* GEMM tiles                                                                  */
+/* ------------------------------------------------------------------------- */
+/* C[m][n] = scale * sum_k A[m][k]*B[n][k] for m in [m0,m0+tm), n in [n0,n0+tn), summed
+ * in double, returned as double (the test rounds / compares).  fmt: 1 bf16, 2 e4m3fn. */
+int orc_gemm_tile(int fmt, const void *A, const void *B, uint32_t K, uint32_t lda, uint32_t ldb,
+                  uint32_t m0, uint32_t n0, uint32_t tm, uint32_t tn, double scale, double *C)
+{
+    if (fmt != 1 && fmt != 2) return -1;
+    const int eb = fmt == 1 ? 2 : 1;
+    /* decode the rows once */
+    double *a = (double *)malloc((size_t)tm * K * sizeof(double));
+    double *b = (double *)malloc((size_t)tn * K * sizeof(double));
+    if (!a || !b) { free(a); free(b); return -3; }
+    for (uint32_t i = 0; i < tm; i++)
+        for (uint32_t k = 0; k < K; k++) {
+            const uint8_t *p = (const uint8_t *)A + ((size_t)(m0 + i) * lda + k) * eb;
+            a[(size_t)i * K + k] = orc_decode(fmt, eb == 2 ? (uint32_t)(p[0] | (p[1] << 8)) : p[0]);
+        }
+    for (uint32_t j = 0; j < tn; j++)
+        for (uint32_t k = 0; k < K; k++) {
+            const uint8_t *p = (const uint8_t *)B + ((size_t)(n0 + j) * ldb + k) * eb;
+            b[(size_t)j * K + k] = orc_decode(fmt, eb == 2 ? (uint32_t)(p[0] | (p[1] << 8)) : p[0]);
+        }
+    #pragma omp parallel for schedule(static)
+    for (uint32_t i = 0; i < tm; i++)
+        for (uint32_t j = 0; j < tn; j++) {
+            double acc = 0.0;
+            const double *ar = a + (size_t)i * K, *br = b + (size_t)j * K;
+            for (uint32_t k = 0; k < K; k++) acc += ar[k] * br[k];
+            C[(size_t)i * tn + j] = acc * scale;
+        }
+    free(a);
+    free(b);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Seeded operand builders (inputs of the matrix tests)                        */
+/* ------------------------------------------------------------------------- */
+/* codes[i] = encode(fmt, sigma * N(0,1)) for elements first..first+n of `stream`;
+ * out_bytes: 2 per element for f16/bf16, 1 otherwise (unpacked codes). */
+void orc_fill_normal_codes(int fmt, double sigma, uint64_t seed, uint32_t stream, uint64_t first, uint64_t n, void *out)
+{
+    const orc_fmt *f = fmt_by_id(fmt);
+    #pragma omp parallel for schedule(static)
+    for (uint64_t i = 0; i < n; i++) {
+        const uint32_t c = fmt_encode(f, sigma * orc_normal(seed, stream, first + i));
+        if (fmt <= 1) ((uint16_t *)out)[i] = (uint16_t)c; else ((uint8_t *)out)[i] = (uint8_t)c;
+    }
+}
+
+/* int8 uniform in [-8,7] from the top 4 bits of the word */
+void orc_fill_int8(uint64_t seed, uint32_t stream, uint64_t first, uint64_t n, int8_t *out)
+{
+    for (uint64_t i = 0; i < n; i++) out[i] = (int8_t)((int)(orc_rng_word(seed, stream, first + i) >> 60) - 8);
+}
+
+/* E8M0 bytes 127 + e, e uniform in {-4..4} */
+void orc_fill_e8m0(uint64_t seed, uint32_t stream, uint64_t first, uint64_t n, uint8_t *out)
+{
+    for (uint64_t i = 0; i < n; i++) out[i] = (uint8_t)(127 - 4 + (int)orc_below(seed, stream, first + i, 9));
+}
+
+/* 2:4 keep patterns: one of the 6 ordered pairs (p0 < p1) per group, as the metadata
+ * byte p0 | p1 << 2. */
+void orc_fill_sparse_meta(uint64_t seed, uint32_t stream, uint64_t first, uint64_t n, uint8_t *out)
+{
+    static const uint8_t pat[6] = {0 | 1 << 2, 0 | 2 << 2, 0 | 3 << 2, 1 | 2 << 2, 1 | 3 << 2, 2 | 3 << 2};
+    for (uint64_t i = 0; i < n; i++) out[i] = pat[orc_below(seed, stream, first + i, 6)];
+}
+
+/* Pack n codes of `bits` (4 or 6) bits each into a little-endian bit stream. */
+void orc_pack_bits(const uint8_t *codes, uint64_t n, int bits, uint8_t *out)
+{
+    memset(out, 0, (size_t)((n * (uint64_t)bits + 7) / 8));
+    for (uint64_t i = 0; i < n; i++) {
+        const uint64_t bit = i * (uint64_t)bits;
+        const uint32_t v = (uint32_t)(codes[i] & ((1u << bits) - 1u)) << (bit & 7u);
+        out[bit >> 3] |= (uint8_t)v;
+        if ((bit & 7u) + (uint32_t)bits > 8) out[(bit >> 3) + 1] |= (uint8_t)(v >> 8);
+    }
+}
+
+/* bf16 / e4m3 images of the seeded uniform stream, as the device fills define them. */
+void orc_fill_bf16(uint16_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist, uint64_t first)
+{
+    #pragma omp parallel for schedule(static)
+    for (uint64_t i = 0; i < n; i++) {
+        const uint64_t z = orc_rng_word(seed, stream, first + i);
+        dst[i] = (uint16_t)fmt_encode(&FMT_BF16, (double)(dist == 0 ? u01_of(z) : upm1_of(z)));
+    }
+}
+
+void orc_fill_e4m3(uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist, float scale, uint64_t first)
+{
+    #pragma omp parallel for schedule(static)
+    for (uint64_t i = 0; i < n; i++) {
+        const uint64_t z = orc_rng_word(seed, stream, first + i);
+        const float v = (dist == 0 ? u01_of(z) : upm1_of(z)) * scale; /* fp32 product, as on the device */
+        dst[i] = (uint8_t)fmt_encode(&FMT_E4M3, (double)v);
+    }
+}
+
+/* float64 sum of n uniform [0,1) elements of a stream (the CPU reference sum of the
+ * bandwidth buffer). */
+double orc_sum_u01(uint64_t seed, uint32_t stream, uint64_t n)
+{
+    double total = 0.0;
+    #pragma omp parallel for schedule(static) reduction(+:total)
+    for (uint64_t i = 0; i < n; i++) total += (double)u01_of(orc_rng_word(seed, stream, i));
+    return total;
+}

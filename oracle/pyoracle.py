@@ -1,0 +1,183 @@
+"""ctypes binding of oracle/liboracle.so -- the CPU oracle (test infrastructure).
+
+Import this only from tests/, from __graft_entry__.smoke() and from the cpu_baseline
+leg of bench.py.  The product never does.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+FMT_F16, FMT_BF16, FMT_E4M3, FMT_E5M2, FMT_E2M3, FMT_E3M2, FMT_E2M1 = range(7)
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} not found: build it with `make -C oracle`")
+        L = C.CDLL(LIB_PATH)
+        vp, u64, u32, i32 = C.c_void_p, C.c_uint64, C.c_uint32, C.c_int
+        L.orc_rng_word.argtypes = [u64, u32, u64]; L.orc_rng_word.restype = u64
+        L.orc_u01.argtypes = [u64, u32, u64]; L.orc_u01.restype = C.c_float
+        L.orc_upm1.argtypes = [u64, u32, u64]; L.orc_upm1.restype = C.c_float
+        L.orc_below.argtypes = [u64, u32, u64, u32]; L.orc_below.restype = u32
+        L.orc_normal.argtypes = [u64, u32, u64]; L.orc_normal.restype = C.c_double
+        L.orc_fill_f32.argtypes = [vp, u64, u64, u32, i32, u64]; L.orc_fill_f32.restype = None
+        L.orc_decode.argtypes = [i32, u32]; L.orc_decode.restype = C.c_double
+        L.orc_encode.argtypes = [i32, C.c_double]; L.orc_encode.restype = u32
+        L.orc_e8m0.argtypes = [u32]; L.orc_e8m0.restype = C.c_double
+        L.orc_global_bandwidth.argtypes = [i32, vp, u64, u64, vp]; L.orc_global_bandwidth.restype = None
+        L.orc_global_bandwidth_thread.argtypes = [i32, u64, u32, u64, u64, u64]
+        L.orc_global_bandwidth_thread.restype = C.c_float
+        L.orc_sum_u01.argtypes = [u64, u32, u64]; L.orc_sum_u01.restype = C.c_double
+        L.orc_compute_mad.argtypes = [i32, i32, u64, u64, u64, u32, vp]; L.orc_compute_mad.restype = i32
+        L.orc_mfma_dense.argtypes = [i32, vp, vp, vp, vp, vp, vp, u32, u32]; L.orc_mfma_dense.restype = i32
+        L.orc_smfmac.argtypes = [i32, vp, vp, vp, vp, vp, u32, u32]; L.orc_smfmac.restype = i32
+        L.orc_gemm_tile.argtypes = [i32, vp, vp, u32, u32, u32, u32, u32, u32, u32, C.c_double, vp]
+        L.orc_gemm_tile.restype = i32
+        _lib = L
+    return _lib
+
+
+def rng_word(seed, stream, i):
+    return lib().orc_rng_word(seed, stream, i)
+
+
+def fill_f32(n, seed, stream, dist, first=0):
+    out = np.empty(n, dtype=np.float32)
+    lib().orc_fill_f32(out.ctypes.data, n, seed, stream, dist, first)
+    return out
+
+
+def normal(n, seed, stream, first=0):
+    L = lib()
+    return np.array([L.orc_normal(seed, stream, first + i) for i in range(n)], dtype=np.float64)
+
+
+def decode(fmt, codes):
+    L = lib()
+    return np.array([L.orc_decode(fmt, int(c)) for c in np.asarray(codes).ravel()], dtype=np.float64).reshape(np.shape(codes))
+
+
+def encode(fmt, values):
+    L = lib()
+    return np.array([L.orc_encode(fmt, float(v)) for v in np.asarray(values).ravel()], dtype=np.uint32).reshape(np.shape(values))
+
+
+def global_bandwidth(width, data, T):
+    data = np.ascontiguousarray(data, dtype=np.float32)
+    out = np.empty(T, dtype=np.float32)
+    lib().orc_global_bandwidth(width, data.ctypes.data, data.size, T, out.ctypes.data)
+    return out
+
+
+def global_bandwidth_thread(width, seed, stream, n_floats, T, t):
+    return lib().orc_global_bandwidth_thread(width, seed, stream, n_floats, T, t)
+
+
+def sum_u01(seed, stream, n):
+    return lib().orc_sum_u01(seed, stream, n)
+
+
+_MAD_OUT = {0: np.float32, 1: np.uint16, 2: np.float64, 3: np.float32, 4: np.float32, 5: np.uint32, 6: np.int32}
+
+
+def compute_mad(kind, width, seed, first, n, steps):
+    out = np.empty(n, dtype=_MAD_OUT[kind])
+    rc = lib().orc_compute_mad(kind, width, seed, first, n, steps, out.ctypes.data)
+    assert rc == 0, rc
+    return out
+
+
+def mfma_dense(kind, A, B, scaleA, scaleB, waves, iters, out_elems, is_int=False):
+    """Returns (out[waves*4*out_elems], abs_scale) -- abs_scale = iters * sum|a*b| per element."""
+    out = np.empty(waves * 4 * out_elems, dtype=np.int32 if is_int else np.float32)
+    ab = np.empty(waves * 4 * out_elems, dtype=np.float64)
+    A = np.ascontiguousarray(A); B = np.ascontiguousarray(B)
+    sa = np.ascontiguousarray(scaleA) if scaleA is not None else None
+    sb = np.ascontiguousarray(scaleB) if scaleB is not None else None
+    rc = lib().orc_mfma_dense(kind, A.ctypes.data, B.ctypes.data, sa.ctypes.data if sa is not None else None,
+                              sb.ctypes.data if sb is not None else None, out.ctypes.data, ab.ctypes.data, waves, iters)
+    assert rc == 0, rc
+    return out, ab
+
+
+def smfmac(kind, Ac, meta, B, waves, iters, is_int=False):
+    out = np.empty(waves * 4 * 256, dtype=np.int32 if is_int else np.float32)
+    ab = np.empty(waves * 4 * 256, dtype=np.float64)
+    Ac = np.ascontiguousarray(Ac); meta = np.ascontiguousarray(meta, dtype=np.uint8); B = np.ascontiguousarray(B)
+    rc = lib().orc_smfmac(kind, Ac.ctypes.data, meta.ctypes.data, B.ctypes.data, out.ctypes.data, ab.ctypes.data, waves, iters)
+    assert rc == 0, rc
+    return out, ab
+
+
+def gemm_tile(fmt, A, B, K, lda, ldb, m0, n0, tm, tn, scale=1.0):
+    out = np.empty((tm, tn), dtype=np.float64)
+    rc = lib().orc_gemm_tile(fmt, A.ctypes.data, B.ctypes.data, K, lda, ldb, m0, n0, tm, tn, scale, out.ctypes.data)
+    assert rc == 0, rc
+    return out
+
+
+def _bind_builders():
+    L = lib()
+    if getattr(L, "_builders_bound", False):
+        return L
+    vp, u64, u32, i32 = C.c_void_p, C.c_uint64, C.c_uint32, C.c_int
+    L.orc_fill_normal_codes.argtypes = [i32, C.c_double, u64, u32, u64, u64, vp]; L.orc_fill_normal_codes.restype = None
+    L.orc_fill_int8.argtypes = [u64, u32, u64, u64, vp]; L.orc_fill_int8.restype = None
+    L.orc_fill_e8m0.argtypes = [u64, u32, u64, u64, vp]; L.orc_fill_e8m0.restype = None
+    L.orc_fill_sparse_meta.argtypes = [u64, u32, u64, u64, vp]; L.orc_fill_sparse_meta.restype = None
+    L.orc_pack_bits.argtypes = [vp, u64, i32, vp]; L.orc_pack_bits.restype = None
+    L.orc_fill_bf16.argtypes = [vp, u64, u64, u32, i32, u64]; L.orc_fill_bf16.restype = None
+    L.orc_fill_e4m3.argtypes = [vp, u64, u64, u32, i32, C.c_float, u64]; L.orc_fill_e4m3.restype = None
+    L._builders_bound = True
+    return L
+
+
+def fill_normal_codes(fmt, sigma, seed, stream, n, first=0):
+    out = np.empty(n, dtype=np.uint16 if fmt <= FMT_BF16 else np.uint8)
+    _bind_builders().orc_fill_normal_codes(fmt, sigma, seed, stream, first, n, out.ctypes.data)
+    return out
+
+
+def fill_int8(seed, stream, n, first=0):
+    out = np.empty(n, dtype=np.int8)
+    _bind_builders().orc_fill_int8(seed, stream, first, n, out.ctypes.data)
+    return out
+
+
+def fill_e8m0(seed, stream, n, first=0):
+    out = np.empty(n, dtype=np.uint8)
+    _bind_builders().orc_fill_e8m0(seed, stream, first, n, out.ctypes.data)
+    return out
+
+
+def fill_sparse_meta(seed, stream, n, first=0):
+    out = np.empty(n, dtype=np.uint8)
+    _bind_builders().orc_fill_sparse_meta(seed, stream, first, n, out.ctypes.data)
+    return out
+
+
+def pack_bits(codes, bits):
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    out = np.empty((codes.size * bits + 7) // 8, dtype=np.uint8)
+    _bind_builders().orc_pack_bits(codes.ctypes.data, codes.size, bits, out.ctypes.data)
+    return out
+
+
+def fill_bf16(n, seed, stream, dist, first=0):
+    out = np.empty(n, dtype=np.uint16)
+    _bind_builders().orc_fill_bf16(out.ctypes.data, n, seed, stream, dist, first)
+    return out
+
+
+def fill_e4m3(n, seed, stream, dist, scale, first=0):
+    out = np.empty(n, dtype=np.uint8)
+    _bind_builders().orc_fill_e4m3(out.ctypes.data, n, seed, stream, dist, scale, first)
+    return out

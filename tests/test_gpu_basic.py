@@ -1,0 +1,145 @@
+"""GPU parity: device facts, seeded fills, global bandwidth, MAD chains, launch latency.
+Everything goes through the C ABI (clpeak_amd.capi) and is compared with the CPU oracle."""
+import numpy as np
+import pytest
+
+from clpeak_amd import capi
+from oracle import pyoracle as orc
+from oracle import workloads as wl
+
+pytestmark = pytest.mark.gpu
+SEED = wl.DEFAULT_SEED
+
+
+def test_device_props(dev):
+    p = dev.props
+    assert p.arch.decode().startswith("gfx950")
+    assert p.num_cus >= 64 and p.wave_size == 64 and p.total_mem > (64 << 30)
+    assert p.name and p.driver_version.count(b".") == 2 and p.runtime_version.count(b".") == 2
+
+
+def test_argument_errors_are_reported_not_launched(dev):
+    out = dev.alloc(1024)
+    with pytest.raises(capi.Mi355Error) as e:
+        dev.global_bandwidth(3, out, 256, out, 1, 256)
+    assert e.value.code == capi.ERR_ARG and "width" in str(e.value)
+    with pytest.raises(capi.Mi355Error) as e:
+        dev.global_bandwidth(4, out, 256, out, 1, 100)
+    assert "block_size" in str(e.value)
+    with pytest.raises(capi.Mi355Error) as e:
+        dev.compute_mad(capi.MAD_F16, 4, 1, 64, 1, out)
+    assert e.value.code == capi.ERR_ARG
+    with pytest.raises(capi.Mi355Error) as e:
+        dev.mfma_dense(0, out, out, None, None, out, 3, 1)
+    assert "multiple of 4" in str(e.value)
+    with pytest.raises(capi.Mi355Error) as e:
+        dev.mfma_dense(capi.MFMA_MXFP4_E2M1, out, out, None, None, out, 4, 1)
+    assert "scale" in str(e.value)
+    with pytest.raises(capi.Mi355Error) as e:
+        dev.gemm_bf16(out, out, out, 100, 256, 64)
+    assert "multiples of 256" in str(e.value)
+    out.free()
+
+
+@pytest.mark.parametrize("dist", [capi.DIST_U01, capi.DIST_UPM1])
+def test_fill_f32_bit_exact(dev, dist):
+    n = (1 << 20) + 77
+    buf = dev.alloc(n * 4)
+    dev.fill_f32(buf, n, SEED, 3, dist)
+    got = buf.download(np.float32, n)
+    assert np.array_equal(got, orc.fill_f32(n, SEED, 3, dist))
+    buf.free()
+
+
+def test_fill_bf16_and_fp8_bit_exact(dev):
+    n = (1 << 18) + 5
+    b16 = dev.alloc(n * 2)
+    dev.fill_bf16(b16, n, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1)
+    assert np.array_equal(b16.download(np.uint16, n), orc.fill_bf16(n, SEED, wl.STREAM_GEMM_A, 1))
+    b8 = dev.alloc(n)
+    for scale in (1.0, 64.0, 448.0, 1000.0):  # the last one exercises saturation
+        dev.fill_fp8_e4m3(b8, n, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, scale)
+        assert np.array_equal(b8.download(np.uint8, n), orc.fill_e4m3(n, SEED, wl.STREAM_GEMM_B, 1, scale)), scale
+    b16.free(); b8.free()
+
+
+@pytest.mark.parametrize("width", [1, 2, 4])
+@pytest.mark.parametrize("n,blocks,bs", [
+    (1 << 22, 64, 256),            # many full unrolled groups
+    ((1 << 20) + 4 * 999, 37, 256),  # ragged tail, odd grid
+    (4 * 100, 8, 64),              # fewer vectors than threads: most partials are 0
+    (1 << 16, 2, 1024),
+])
+def test_global_bandwidth_bit_exact(dev, width, n, blocks, bs):
+    data = orc.fill_f32(n, SEED, wl.STREAM_BW, 0)
+    src = dev.from_host(data)
+    T = blocks * bs
+    out = dev.alloc(T * 4)
+    dev.global_bandwidth(width, src, n, out, blocks, bs)
+    got = out.download(np.float32, T)
+    assert np.array_equal(got, orc.global_bandwidth(width, data, T))
+    src.free(); out.free()
+
+
+def test_global_bandwidth_full_size_4GiB(dev):
+    """The 4 GiB buffer of the HBM configuration: device-filled, every width; sampled
+    threads bit-exact against the oracle regenerating their elements, grand total within
+    1e-5 relative of the CPU reference sum, and equal across widths within tolerance."""
+    n = 1 << 30
+    src = dev.alloc(n * 4)
+    dev.fill_f32(src, n, SEED, wl.STREAM_BW, capi.DIST_U01)
+    blocks, bs = dev.props.num_cus * 8, 256
+    T = blocks * bs
+    out = dev.alloc(T * 4)
+    ref_total = orc.sum_u01(SEED, wl.STREAM_BW, n)
+    rng = np.random.default_rng(0)
+    for width in (1, 2, 4):
+        dev.global_bandwidth(width, src, n, out, blocks, bs)
+        got = out.download(np.float32, T)
+        for t in [0, 1, T - 1] + list(rng.integers(0, T, 13)):
+            assert got[t] == orc.global_bandwidth_thread(width, SEED, wl.STREAM_BW, n, T, int(t)), (width, t)
+        total = float(got.astype(np.float64).sum())
+        assert abs(total - ref_total) <= 1e-5 * ref_total, (width, total, ref_total)
+    src.free(); out.free()
+
+
+MAD_CASES = [
+    (capi.MAD_F32, 1, 4096, np.float32), (capi.MAD_F32, 2, 100, np.float32), (capi.MAD_F32, 4, 4096, np.float32),
+    (capi.MAD_F64, 1, 4096, np.float64), (capi.MAD_F64, 2, 33, np.float64), (capi.MAD_F64, 4, 512, np.float64),
+    (capi.MAD_F16, 1, 300, np.uint16), (capi.MAD_F16, 2, 300, np.uint16), (capi.MAD_F16, 2, 7, np.uint16),
+    (capi.MAD_MP, 1, 4096, np.float32), (capi.MAD_BF16, 1, 4096, np.float32),
+    (capi.MAD_I32, 1, 2048, np.uint32), (capi.MAD_I32, 2, 5, np.uint32), (capi.MAD_I32, 4, 2048, np.uint32),
+    (capi.MAD_I8DP, 1, 1024, np.int32), (capi.MAD_I8DP, 2, 1024, np.int32), (capi.MAD_I8DP, 4, 99, np.int32),
+    (capi.MAD_I8DP, 8, 1024, np.int32),
+]
+
+
+@pytest.mark.parametrize("kind,width,steps,dtype", MAD_CASES)
+def test_compute_mad_bit_exact(dev, kind, width, steps, dtype):
+    n = 1000 if kind != capi.MAD_F16 else 200   # ragged: not a multiple of the block size
+    out = dev.alloc(n * np.dtype(dtype).itemsize)
+    dev.compute_mad(kind, width, SEED, n, steps, out, 256)
+    got = out.download(dtype, n)
+    ref = orc.compute_mad(kind, width, SEED, 0, n, steps)
+    assert np.array_equal(got.view(np.uint8), ref.view(np.uint8)), (got[:4], ref[:4])
+    out.free()
+
+
+def test_compute_mad_f32_full_size_sampled(dev):
+    """2^20 work-items x 16 accumulators x 4096 steps; slices of the output against the oracle."""
+    n, steps = 1 << 20, 4096
+    out = dev.alloc(n * 4)
+    dev.compute_mad(capi.MAD_F32, 4, SEED, n, steps, out, 256)
+    got = out.download(np.float32, n)
+    for first in (0, 123457, n - 64):
+        assert np.array_equal(got[first:first + 64], orc.compute_mad(0, 4, SEED, first, 64, steps)), first
+    assert np.all(np.isfinite(got))
+    out.free()
+
+
+def test_launch_roundtrip(dev):
+    us = dev.launch_roundtrip(2, 1000)
+    assert 0.5 < us < 1000.0
+    # the HIP-event timer sees the same order of magnitude for a batch of empty launches
+    t = dev.time_launches(lambda: dev.launch_roundtrip(0, 1), 10)
+    assert t > 0

@@ -1,0 +1,82 @@
+"""GPU parity of the hand-written GEMM against the oracle's float64 tiles.
+
+Tolerance (from the workload definition): 2e-2 relative.  Stated precisely: for every
+checked element |gpu - ref| <= 2e-2*|ref| + 2e-2*rms(ref tile); the observed error is far
+smaller (bf16 output rounding, 2^-9 relative) and is asserted at 1e-2 as well."""
+import numpy as np
+import pytest
+
+from clpeak_amd import capi
+from oracle import pyoracle as orc
+from oracle import workloads as wl
+
+pytestmark = pytest.mark.gpu
+SEED = wl.DEFAULT_SEED
+FP8_SCALE = 448.0   # per-tensor scale: uniform [-1,1) * 448 fills the e4m3 range
+
+
+def _operands(dev, fp8, M, N, K):
+    eb = 1 if fp8 else 2
+    dA, dB = dev.alloc(M * K * eb), dev.alloc(N * K * eb)
+    if fp8:
+        dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, FP8_SCALE)
+        dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, FP8_SCALE)
+    else:
+        dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1)
+        dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+    return dA, dB
+
+
+def _rows(buf, fp8, row0, rows, K):
+    """Rows [row0, row0+rows) of a device operand (the fills themselves are checked bit-exact
+    against the oracle in test_gpu_basic.py)."""
+    eb = 1 if fp8 else 2
+    return buf.download(np.uint8 if fp8 else np.uint16, rows * K, offset_bytes=row0 * K * eb)
+
+
+def _check_tiles(dev, fp8, M, N, K, tiles, tile=128):
+    dA, dB = _operands(dev, fp8, M, N, K)
+    dC = dev.alloc(M * N * 2)
+    dev._check(dev.lib.mi355_memset(dev.h, dC.ptr, 0xff, M * N * 2))   # NaN pattern: unwritten output shows
+    if fp8:
+        dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1.0 / FP8_SCALE, 1.0 / FP8_SCALE)
+    else:
+        dev.gemm_bf16(dA, dB, dC, M, N, K)
+    fmt = orc.FMT_E4M3 if fp8 else orc.FMT_BF16
+    scale = 1.0 / (FP8_SCALE * FP8_SCALE) if fp8 else 1.0
+    worst = 0.0
+    for (m0, n0) in tiles:
+        a = _rows(dA, fp8, m0, tile, K)
+        b = _rows(dB, fp8, n0, tile, K)
+        ref = orc.gemm_tile(fmt, a, b, K, K, K, 0, 0, tile, tile, scale)
+        got = np.empty((tile, tile), dtype=np.float64)
+        for i in range(tile):
+            row = dC.download(np.uint16, tile, offset_bytes=((m0 + i) * N + n0) * 2)
+            got[i] = (row.astype(np.uint32) << 16).view(np.float32)
+        rms = float(np.sqrt((ref ** 2).mean()))
+        err = np.abs(got - ref)
+        assert np.all(np.isfinite(got)), (m0, n0)
+        assert np.all(err <= 2e-2 * np.abs(ref) + 2e-2 * rms), (m0, n0, float(err.max()), rms)
+        assert np.all(err <= 1e-2 * np.abs(ref) + 1e-2 * rms), (m0, n0, float(err.max()), rms)
+        worst = max(worst, float((err / (np.abs(ref) + rms)).max()))
+    for b in (dA, dB, dC):
+        b.free()
+    return worst
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (512, 768, 384), (2048, 2048, 1024)])
+def test_gemm_small_all_tiles(dev, fp8, M, N, K):
+    tiles = [(m, n) for m in range(0, M, 128) for n in range(0, N, 128)]
+    if len(tiles) > 24:
+        rng = np.random.default_rng(1)
+        tiles = [tiles[i] for i in rng.choice(len(tiles), 24, replace=False)]
+    _check_tiles(dev, fp8, M, N, K, tiles)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_gemm_8192_sampled_tiles(dev, fp8):
+    """M=N=K=8192, 64 randomly sampled 128x128 output tiles against the CPU GEMM."""
+    rng = np.random.default_rng(2)
+    tiles = [(int(m) * 128, int(n) * 128) for m, n in zip(rng.integers(0, 64, 64), rng.integers(0, 64, 64))]
+    _check_tiles(dev, fp8, 8192, 8192, 8192, tiles)

@@ -1,0 +1,294 @@
+"""Pins the oracle's kernels (CPU only) against what the mathematics fixes: closed forms
+of the affine recurrence, numpy restatements written from the definitions in
+include/clpeak_mi355.h, exact integer arithmetic in Python, special cases."""
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+from oracle import workloads as wl
+
+
+# ---- global bandwidth --------------------------------------------------------------
+@pytest.mark.parametrize("width", [1, 2, 4])
+@pytest.mark.parametrize("n,T", [(4096, 64), (4096 + 64, 128), (1000 * 4, 192), (64, 256)])
+def test_bandwidth_partials_brute_force(width, n, T):
+    data = orc.fill_f32(n, 3, wl.STREAM_BW, 0)
+    got = orc.global_bandwidth(width, data, T)
+    vec = data.reshape(-1, width)
+    ref = np.zeros(T, dtype=np.float32)
+    for t in range(T):
+        acc = np.zeros(width, dtype=np.float32)
+        for v in vec[t::T]:                      # thread t owns vectors t, t+T, ...
+            acc = (acc + v).astype(np.float32)
+        s = acc[0]
+        for c in range(1, width):
+            s = np.float32(s + acc[c])
+        ref[t] = s
+    assert np.array_equal(got, ref)
+    # invariant: the grand total does not depend on the vector width (up to fp32 rounding)
+    assert abs(float(got.astype(np.float64).sum()) - float(data.astype(np.float64).sum())) < 1e-5 * n
+
+
+def test_bandwidth_seeded_thread_matches_buffer_version():
+    n, T = 1 << 16, 512
+    data = orc.fill_f32(n, 77, wl.STREAM_BW, 0)
+    for width in (1, 2, 4):
+        full = orc.global_bandwidth(width, data, T)
+        for t in (0, 1, 255, 511):
+            assert orc.global_bandwidth_thread(width, 77, wl.STREAM_BW, n, T, t) == full[t]
+
+
+# ---- MAD chains ----------------------------------------------------------------------
+def _seeds(seed, first, n, per=16, stream=wl.STREAM_MAD):
+    return orc.fill_f32(n * per, seed, stream, 1, first=first * per).reshape(n, per).astype(np.float64)
+
+
+def test_mad_f64_closed_form():
+    """x_n = a^n x0 + x0 (a^n - 1)/(a - 1); the double chain tracks it to ~1e-12."""
+    n, steps, a = 32, 4096, 1.0001
+    got = orc.compute_mad(2, 1, 99, 5, n, steps)
+    x0 = _seeds(99, 5, n)
+    xn = a ** steps * x0 + x0 * (a ** steps - 1) / (a - 1)
+    assert abs(a ** steps - 1.5063) < 1e-3
+    assert np.allclose(got, xn.sum(axis=1), rtol=1e-10, atol=1e-9)
+
+
+def test_mad_f32_closed_form_and_bit_exact_numpy():
+    n, steps = 16, 4096
+    got = orc.compute_mad(0, 1, 99, 0, n, steps)
+    x0 = _seeds(99, 0, n)
+    a = float(np.float32(1.0001))
+    xn = a ** steps * x0 + x0 * (a ** steps - 1) / (a - 1)
+    assert np.allclose(got, xn.sum(axis=1), rtol=2e-3)
+    # bit-exact restatement: fp32 FMA = exact product-sum in float64 (24+24 bit product, one
+    # add) rounded once to fp32 -- float64 holds a*x exactly, the sum's double rounding cannot
+    # bite because the fp64 result keeps >= 29 bits beyond the fp32 mantissa except on exact ties
+    # that the 24-bit lattice of a*x + x0 rules out for these magnitudes; checked on short chains.
+    steps = 64
+    got = orc.compute_mad(0, 1, 99, 0, n, steps)
+    x0f = x0.astype(np.float32)
+    x = x0f.copy()
+    from fractions import Fraction
+    for _ in range(steps):
+        nxt = np.empty_like(x)
+        for idx in np.ndindex(x.shape):
+            exact = Fraction(float(x[idx])) * Fraction(float(np.float32(1.0001))) + Fraction(float(x0f[idx]))
+            nxt[idx] = _round_fraction_to_f32(exact)
+        x = nxt
+    ref = np.zeros(n, dtype=np.float32)
+    for j in range(16):
+        ref = (ref + x[:, j]).astype(np.float32)
+    assert np.array_equal(got, ref)
+
+
+def _round_fraction_to_f32(q):
+    """Correctly rounded (nearest even) fp32 of an exact rational."""
+    from fractions import Fraction
+    if q == 0:
+        return np.float32(0.0)
+    f = float(q)                       # float(Fraction) is correctly rounded to double
+    c = np.float32(f)
+    # repair a possible double rounding: compare the neighbours exactly
+    cands = [np.nextafter(c, np.float32(-np.inf)), c, np.nextafter(c, np.float32(np.inf))]
+    best = min(cands, key=lambda v: (abs(Fraction(float(v)) - q), int(np.float32(v).view(np.uint32)) & 1))
+    return np.float32(best)
+
+
+def test_mad_widths_do_not_change_results():
+    for kind in (0, 2, 5):
+        ref = orc.compute_mad(kind, 1, 5, 0, 8, 100)
+        for w in (2, 4):
+            assert np.array_equal(orc.compute_mad(kind, w, 5, 0, 8, 100), ref)
+
+
+def test_mad_f16_against_numpy_float16():
+    """numpy float16 arithmetic through exact float64 intermediates: fma = round16(x*a + x0)."""
+    n, steps = 8, 300
+    got = orc.compute_mad(1, 1, 21, 0, n, steps)
+    x0 = _seeds(21, 0, n).astype(np.float16)
+    a = np.float16(1 - 2.0 ** -10)
+    x = x0.copy()
+    for _ in range(steps):
+        x = (x.astype(np.float64) * float(a) + x0.astype(np.float64)).astype(np.float16)  # exact in f64, one rounding
+    s = np.zeros(n, dtype=np.float16)
+    for j in range(16):
+        s = (s.astype(np.float64) + x[:, j].astype(np.float64)).astype(np.float16)
+    assert np.array_equal(got, s.view(np.uint16))
+
+
+def test_mad_mixed_closed_form():
+    """acc_n = xh + n * (xh*a) up to fp32 rounding; operands really are rounded through half / bf16."""
+    n, steps = 8, 1000
+    for kind, a in ((3, 1 - 2.0 ** -10), (4, 1 - 2.0 ** -8)):
+        got = orc.compute_mad(kind, 1, 8, 0, n, steps)
+        u = _seeds(8, 0, n)
+        if kind == 3:
+            xn = u.astype(np.float16).astype(np.float64)
+        else:
+            xn = orc.decode(orc.FMT_BF16, orc.encode(orc.FMT_BF16, u))
+        ref = (xn + steps * xn * a).sum(axis=1)
+        assert np.allclose(got, ref, rtol=1e-4, atol=1e-3)
+        assert not np.allclose(got, (u + steps * u * a).sum(axis=1), rtol=1e-6, atol=0)  # rounding of operands is visible
+
+
+def test_mad_i32_exact():
+    n, steps = 8, 257
+    got = orc.compute_mad(5, 1, 4, 3, n, steps)
+    for q in range(n):
+        total = 0
+        for j in range(16):
+            x0 = orc.rng_word(4, wl.STREAM_MAD, (3 + q) * 16 + j) >> 32
+            # closed form mod 2^32: x_n = x0 * (3^(n+1) - 1) / 2
+            xn = (x0 * ((3 ** (steps + 1) - 1) // 2)) % (1 << 32)
+            total = (total + xn) % (1 << 32)
+        assert int(got[q]) == total
+
+
+def test_mad_i8dp_exact():
+    def sdot4(x, y, acc):
+        for b in range(4):
+            xb = ((x >> (8 * b)) & 0xff); xb -= 256 * (xb > 127)
+            yb = ((y >> (8 * b)) & 0xff); yb -= 256 * (yb > 127)
+            acc += xb * yb
+        return acc & 0xffffffff
+    n, steps = 4, 50
+    for chains in (1, 2, 4, 8):
+        got = orc.compute_mad(6, chains, 12, 0, n, steps)
+        for q in range(n):
+            total = 0
+            for c in range(chains):
+                x = orc.rng_word(12, wl.STREAM_MAD, q * 8 + c) >> 32
+                y = orc.rng_word(12, wl.STREAM_MAD_Y, q * 8 + c) >> 32
+                acc = 0
+                for _ in range(steps):
+                    acc = sdot4(x, y, acc)
+                    y ^= acc
+                total = (total + acc) & 0xffffffff
+            assert int(got[q]) & 0xffffffff == total
+
+
+# ---- matrix instructions ------------------------------------------------------------------
+def _unpack(packed, bits, n):
+    if bits == 16:
+        return packed.view(np.uint16)[:n].astype(np.uint32)
+    if bits == 8:
+        return packed[:n].astype(np.uint32)
+    b = np.unpackbits(packed, bitorder="little")[: n * bits].reshape(n, bits)
+    return (b.astype(np.uint32) << np.arange(bits, dtype=np.uint32)).sum(axis=1)
+
+
+def _dense_reference(kind, A, B, sA, sB, waves, iters):
+    """float64 A.B^T per (wave, chain) from the definitions in the C header."""
+    s = wl.DENSE[kind]
+    M, N, K, units = s["M"], s["N"], s["K"], waves * 4
+    if s["fmt"] is None:
+        a = A.view(np.int8).astype(np.int64).reshape(units, M, K)
+        b = B.view(np.int8).astype(np.int64).reshape(units, N, K)
+        return np.einsum("umk,unk->umn", a, b) * iters
+    a = orc.decode(s["fmt"], _unpack(A, s["bits"], units * M * K)).reshape(units, M, K)
+    b = orc.decode(s["fmt"], _unpack(B, s["bits"], units * N * K)).reshape(units, N, K)
+    if s["scaled"]:
+        a = a * np.repeat(2.0 ** (sA.astype(np.float64) - 127), 32).reshape(units, M, K)
+        b = b * np.repeat(2.0 ** (sB.astype(np.float64) - 127), 32).reshape(units, N, K)
+    return np.einsum("umk,unk->umn", a, b) * iters
+
+
+@pytest.mark.parametrize("kind", sorted(wl.DENSE))
+def test_mfma_dense_oracle_against_numpy(kind):
+    s = wl.DENSE[kind]
+    waves, iters = 4, 1
+    A, B, sA, sB = wl.dense_inputs(kind, waves, seed=1234)
+    out, ab = orc.mfma_dense(kind, A, B, sA, sB, waves, iters, s["M"] * s["N"], is_int=s["fmt"] is None)
+    ref = _dense_reference(kind, A, B, sA, sB, waves, iters).reshape(-1)
+    if s["fmt"] is None:
+        assert np.array_equal(out.astype(np.int64), ref)
+    else:
+        assert np.all(np.abs(out - ref) <= 1e-6 * np.abs(ref) + 1e-30)  # one fp32 rounding of an exact sum
+        assert np.all(ab >= np.abs(ref) * (1 - 1e-12))
+
+
+def test_mfma_iterations_accumulate_linearly_for_int8():
+    A, B, _, _ = wl.dense_inputs(4, 4, seed=9)
+    one, _ = orc.mfma_dense(4, A, B, None, None, 4, 1, 256, is_int=True)
+    many, _ = orc.mfma_dense(4, A, B, None, None, 4, 4096, 256, is_int=True)
+    assert np.array_equal(many.astype(np.int64), one.astype(np.int64) * 4096)   # no overflow in the seeded range
+    assert np.abs(many).max() < 2 ** 31 / 4
+
+
+def test_mfma_fp32_chain_is_sequential_rounding():
+    """acc after n steps is the n-fold fp32 running sum of one product, not n*P rounded once."""
+    A, B, _, _ = wl.dense_inputs(0, 4, seed=5)
+    one, _ = orc.mfma_dense(0, A, B, None, None, 4, 1, 256)
+    n = 1000
+    many, _ = orc.mfma_dense(0, A, B, None, None, 4, n, 256)
+    exact1 = _dense_reference(0, A, B, None, None, 4, 1).reshape(-1)
+    acc = np.zeros_like(one)
+    for _ in range(n):
+        acc = (acc.astype(np.float64) + exact1).astype(np.float32)
+    assert np.array_equal(many, acc)
+    assert np.allclose(many, exact1 * n, rtol=1e-4)
+
+
+def test_mfma_identity_b_reproduces_a():
+    """B = identity block (N x K with ones on the diagonal): out[m][n] = A[m][n]."""
+    s = wl.DENSE[0]
+    A, _, _, _ = wl.dense_inputs(0, 4, seed=3)
+    eye = np.zeros((16, 16, 32), dtype=np.float16)  # 16 units
+    for n in range(16):
+        eye[:, n, n] = 1.0
+    out, _ = orc.mfma_dense(0, A, eye.view(np.uint8).reshape(-1), None, None, 4, 1, 256)
+    a = A.view(np.float16).reshape(16, 16, 32)[:, :, :16].astype(np.float32)
+    assert np.array_equal(out.reshape(16, 16, 16), a)
+
+
+@pytest.mark.parametrize("kind", sorted(wl.SPARSE))
+def test_smfmac_oracle_is_dense_on_decompressed_a(kind):
+    s = wl.SPARSE[kind]
+    waves, K, eb = 4, s["K"], s["bits"] // 8
+    Ac, meta, B = wl.sparse_inputs(kind, waves, seed=77)
+    out, _ = orc.smfmac(kind, Ac, meta, B, waves, 3, is_int=s["fmt"] is None)
+    # decompress in numpy from the metadata definition
+    units = waves * 4
+    dt = np.uint16 if eb == 2 else np.uint8
+    ac = Ac.view(dt).reshape(units, 16, K // 4, 2)
+    md = meta.reshape(units, 16, K // 4)
+    dense = np.zeros((units, 16, K // 4, 4), dtype=dt)
+    u, m, g = np.indices(md.shape)
+    dense[u, m, g, md & 3] = ac[..., 0]
+    dense[u, m, g, (md >> 2) & 3] = ac[..., 1]
+    dense = dense.reshape(units, 16, K)
+    b = B.view(dt).reshape(units, 16, K)
+    if s["fmt"] is None:
+        ref = np.einsum("umk,unk->umn", dense.view(np.int8).astype(np.int64), b.view(np.int8).astype(np.int64)) * 3
+        assert np.array_equal(out.astype(np.int64), ref.reshape(-1))
+    else:
+        ref = np.einsum("umk,unk->umn", orc.decode(s["fmt"], dense), orc.decode(s["fmt"], b)) * 3
+        assert np.allclose(out, ref.reshape(-1), rtol=1e-5, atol=1e-12)
+    # exactly half of A is kept
+    assert np.count_nonzero(md & 3 == (md >> 2) & 3) == 0
+
+
+def test_smfmac_rejects_repeated_positions():
+    Ac, meta, B = wl.sparse_inputs(4, 4, seed=1)
+    meta = meta.copy(); meta[0] = 0b0101  # both kept values claim slot 1
+    out = np.empty(4 * 4 * 256, dtype=np.int32); ab = np.empty(4 * 4 * 256)
+    rc = orc.lib().orc_smfmac(4, Ac.ctypes.data, meta.ctypes.data, B.ctypes.data, out.ctypes.data, ab.ctypes.data, 4, 1)
+    assert rc == -2
+
+
+# ---- GEMM tiles -------------------------------------------------------------------------------
+@pytest.mark.parametrize("fmt", [orc.FMT_BF16, orc.FMT_E4M3])
+def test_gemm_tile_against_numpy_and_special_cases(fmt):
+    M = N = 64; K = 256
+    if fmt == orc.FMT_BF16:
+        A = orc.fill_bf16(M * K, 1, wl.STREAM_GEMM_A, 1); B = orc.fill_bf16(N * K, 1, wl.STREAM_GEMM_B, 1)
+    else:
+        A = orc.fill_e4m3(M * K, 1, wl.STREAM_GEMM_A, 1, 64.0); B = orc.fill_e4m3(N * K, 1, wl.STREAM_GEMM_B, 1, 64.0)
+    a = orc.decode(fmt, A).reshape(M, K); b = orc.decode(fmt, B).reshape(N, K)
+    got = orc.gemm_tile(fmt, A, B, K, K, K, 16, 32, 32, 16, scale=0.5)
+    assert np.allclose(got, 0.5 * (a[16:48] @ b[32:48].T), rtol=1e-12, atol=1e-12)
+    # A = I (as codes): C = B^T
+    one = int(orc.encode(fmt, [1.0])[0])
+    I = np.zeros((M, K), dtype=A.dtype); I[np.arange(M), np.arange(M)] = one
+    got = orc.gemm_tile(fmt, I, B, K, K, K, 0, 0, M, N)
+    assert np.array_equal(got, b[:, :M].T)
