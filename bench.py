@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark driver of the MI355X clpeak backend.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+Prints ONE JSON line.  A "step" is one launch of the headline kernel: the float4
+streaming read-reduce over a 4 GiB fp32 buffer resident in HBM (the HBM configuration
+of the workload list).  `value` is its throughput in GB/s.  The same line carries
+
+  roofline      the headline kernel against the 8 TB/s HBM3E peak, from HIP events on
+                the stream the kernel runs on;
+  cpu_baseline  the CPU oracle's float4 read-reduce timed on this host (bounded sample);
+  rows          every other kernel of the backend (float/float2 reads, MAD chains, launch
+                latency, dense MFMA, 2:4 SMFMAC, GEMM) with its absolute figure, the
+                MI355X datasheet peak it is compared with and the fraction reached.
+
+One GPU only: the path has no exchange step, every unit of work is independent, so more
+GPUs would simply run the same kernels side by side.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+# MI355X dense peaks (TFLOP/s or TOP/s); 2:4 sparse peaks are twice the dense ones.
+PEAK = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "fp6": 10100.0, "fp4": 10100.0,
+        "fp32_vec": 157.3, "fp64_vec": 78.6}
+SEED = 0x5EEDC1BEA4D355
+
+
+def timed(dev, launch, min_us=300e3, warm_us=300e3, max_iters=10000):
+    """Reference discipline (warm-up, probe, batch sized to a time budget), with the warm-up
+    long enough for the clocks to settle under this kernel's load.  Returns us per launch."""
+    launch(); dev.sync()
+    probe = max(dev.time_launches(launch, 1), 1.0)
+    dev.time_launches(launch, int(min(max(warm_us / probe, 2), max_iters)))
+    n = int(min(max(min_us / probe, 1), max_iters))
+    return dev.time_launches(launch, n) / n, n
+
+
+def bench_rows(dev, quick):
+    from clpeak_amd import capi
+    from oracle import workloads as wl
+    rows = []
+    budget = dict(min_us=100e3, warm_us=100e3) if quick else {}
+
+    def add(test, metric, value, unit, us, peak=None, **extra):
+        r = {"test": test, "metric": metric, "value": round(value, 2), "unit": unit, "us_per_launch": round(us, 2)}
+        if peak:
+            r["peak"] = peak
+            r["frac"] = round(value / peak, 4)
+        r.update(extra)
+        rows.append(r)
+
+    # --- vector MAD chains: 2^20 work-items x 16 accumulators x 4096 steps -------------
+    n_items, steps = 1 << 20, 4096
+    out = dev.alloc(n_items * 8)
+    mad = [("single_precision_compute", capi.MAD_F32, [(1, "float"), (2, "float2"), (4, "float4")], 2, "gflops", PEAK["fp32_vec"] * 1e3),
+           ("half_precision_compute", capi.MAD_F16, [(1, "half"), (2, "half2")], 2, "gflops", None),
+           ("double_precision_compute", capi.MAD_F64, [(1, "double"), (2, "double2"), (4, "double4")], 2, "gflops", PEAK["fp64_vec"] * 1e3),
+           ("mixed_precision_compute", capi.MAD_MP, [(1, "mp")], 2, "gflops", None),
+           ("bfloat16_compute", capi.MAD_BF16, [(1, "bf16")], 2, "gflops", None),
+           ("integer_compute", capi.MAD_I32, [(1, "int"), (2, "int2"), (4, "int4")], 2, "gops", None)]
+    for test, kind, variants, ops, unit, peak in mad:
+        for width, metric in variants:
+            us, _ = timed(dev, lambda: dev.compute_mad(kind, width, SEED, n_items, steps, out), **budget)
+            add(test, metric, n_items * 16 * steps * ops / us / 1e3, unit, us, peak)
+    for chains, metric in ((1, "int8_dp"), (2, "int8_dp2"), (4, "int8_dp4"), (8, "int8_dp8")):
+        us, _ = timed(dev, lambda: dev.compute_mad(capi.MAD_I8DP, chains, SEED, n_items, steps, out), **budget)
+        add("integer_compute_int8_dp", metric, n_items * chains * steps * 8 / us / 1e3, "gops", us)
+    out.free()
+
+    # --- launch latency ------------------------------------------------------------------
+    us = dev.launch_roundtrip(2, 10000)
+    add("kernel_launch_latency", "roundtrip", us, "us", us)
+
+    # --- dense MFMA / SMFMAC: 2048 waves x 4 chains x 4096 iterations ------------------------
+    waves, iters = 2048, 4096
+    clk = dev.alloc(16)
+    peaks = {0: "f16", 1: "bf16", 2: "f16", 3: "bf16", 4: "int8", 5: "fp8", 6: "fp8", 7: "fp6", 8: "fp6", 9: "fp4"}
+    for kind in sorted(wl.DENSE):
+        s = wl.DENSE[kind]
+        A, B, sA, sB = wl.dense_inputs(kind, waves, SEED)
+        bufs = [dev.from_host(A), dev.from_host(B), dev.from_host(sA) if sA is not None else None,
+                dev.from_host(sB) if sB is not None else None]
+        o = dev.alloc(waves * 4 * s["M"] * s["N"] * 4)
+        us, _ = timed(dev, lambda: dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], o, waves, iters, clk), **budget)
+        c = clk.download(np.uint64, 2)
+        unit = "tops" if s["fmt"] is None else "tflops"
+        add(s["name"], s["name"], wl.dense_flops(kind, waves, iters) / us / 1e6, unit, us, PEAK[peaks[kind]],
+            shape=s["shape"], sclk_mhz=round(float(c[0]) / max(float(c[1]), 1.0) * 100.0, 0))
+        for b in bufs + [o]:
+            if b is not None:
+                b.free()
+    speaks = {0: "f16", 1: "bf16", 2: "fp8", 3: "fp8", 4: "int8"}
+    for kind in sorted(wl.SPARSE):
+        s = wl.SPARSE[kind]
+        Ac, meta, B = wl.sparse_inputs(kind, waves, SEED)
+        bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
+        o = dev.alloc(waves * 4 * 256 * 4)
+        us, _ = timed(dev, lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk), **budget)
+        c = clk.download(np.uint64, 2)
+        unit = "tops" if s["fmt"] is None else "tflops"
+        add(s["name"], s["name"], wl.sparse_flops(kind, waves, iters) / us / 1e6, unit, us, 2 * PEAK[speaks[kind]],
+            shape=s["shape"], sclk_mhz=round(float(c[0]) / max(float(c[1]), 1.0) * 100.0, 0))
+        for b in bufs + [o]:
+            b.free()
+    clk.free()
+
+    # --- GEMM 8192^3 ---------------------------------------------------------------------------
+    M = N = K = 8192
+    for fp8 in (False, True):
+        eb = 1 if fp8 else 2
+        dA, dB, dC = dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * 2)
+        if fp8:
+            dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, 448.0)
+            dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, 448.0)
+            fn = lambda: dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1 / 448.0, 1 / 448.0)
+        else:
+            dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1)
+            dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            fn = lambda: dev.gemm_bf16(dA, dB, dC, M, N, K)
+        us, _ = timed(dev, fn, **budget)
+        add("hipblaslt-fp8" if fp8 else "rocblas-fp", "fp8_e4m3" if fp8 else "bf16", 2.0 * M * N * K / us / 1e6, "tflops", us,
+            PEAK["fp8" if fp8 else "bf16"], shape="8192x8192x8192")
+        for b in (dA, dB, dC):
+            b.free()
+    return rows
+
+
+def cpu_baseline(seconds=12.0):
+    """The oracle's float4 read-reduce (scalar C, one core) over a 256 MiB buffer, repeated
+    for about `seconds` of CPU time."""
+    from oracle import pyoracle as orc
+    from oracle import workloads as wl
+    n = 1 << 26
+    data = orc.fill_f32(n, SEED, wl.STREAM_BW, 0)
+    T = 1 << 20
+    orc.global_bandwidth(4, data, T)  # warm-up / page-in
+    t0 = time.perf_counter()
+    passes = 0
+    while time.perf_counter() - t0 < seconds:
+        orc.global_bandwidth(4, data, T)
+        passes += 1
+    dt = time.perf_counter() - t0
+    return {"value": round(passes * n * 4 / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{passes} passes of the float4 read-reduce over a 256 MiB (2^26 float) seeded buffer, "
+                      f"2^20 partial sums, scalar C oracle on one core, {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--no-rows", action="store_true", help="headline kernel only")
+    ap.add_argument("--quick", action="store_true", help="shorter time budget per extra row")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; the hot path has no multi-GPU step "
+                 "(every kernel is independent per device), run with --gpus 1")
+
+    from clpeak_amd import capi
+    from oracle import workloads as wl
+    dev = capi.Device(0)
+
+    n = 1 << 30                                   # 4 GiB of fp32, far past the 256 MB Infinity Cache
+    src = dev.alloc(n * 4)
+    dev.fill_f32(src, n, SEED, wl.STREAM_BW, capi.DIST_U01)
+    blocks, bs = dev.props.num_cus * HEADLINE_BLOCKS_PER_CU, 256
+    out = dev.alloc(blocks * bs * 4)
+    step = lambda: dev.global_bandwidth(4, src, n, out, blocks, bs)
+
+    for _ in range(args.warmup):
+        step()
+    dev.sync()
+    t0 = time.perf_counter()
+    ev_us = dev.time_launches(step, args.steps)   # HIP events on the kernel's stream; ends synchronised
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    kernel_us = ev_us / args.steps
+    gbps = n * 4 / (wall / args.steps) / 1e9
+
+    rows = []
+    # the other two widths of the same test, same discipline
+    for width, metric in ((1, "float"), (2, "float2")):
+        fn = lambda: dev.global_bandwidth(width, src, n, out, blocks, bs)
+        for _ in range(max(args.warmup // 4, 2)):
+            fn()
+        us = dev.time_launches(fn, max(args.steps // 4, 1)) / max(args.steps // 4, 1)
+        rows.append({"test": "global_memory_bandwidth", "metric": metric, "value": round(n * 4 / us / 1e3, 2), "unit": "gbps",
+                     "us_per_launch": round(us, 2), "peak": HBM_PEAK_GBPS, "frac": round(n * 4 / us / 1e3 / HBM_PEAK_GBPS, 4)})
+    src.free(); out.free()
+    if not args.no_rows:
+        rows += bench_rows(dev, args.quick)
+    dev.close()
+
+    achieved = n * 4 / kernel_us / 1e3
+    line = {
+        "metric": "MFMA TFLOPS/TOPS per dtype (dense, 2:4) + HBM GB/s, as % of MI355X peak",
+        "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "HBM streaming read: float4 grid-stride read-reduce over a 4 GiB fp32 buffer "
+                               "(uniform[0,1) seeded on device), one fp32 partial sum per thread",
+                   "buffer_bytes": n * 4, "threads": blocks * bs, "pct_of_peak": round(100 * gbps / HBM_PEAK_GBPS, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel_us": round(kernel_us, 2), "algorithmic_bytes": n * 4},
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(),
+        "rows": rows,
+    }
+    print(json.dumps(line))
+
+
+# Workgroups per CU of the headline launch (256 threads each).
+HEADLINE_BLOCKS_PER_CU = 8
+# HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (see profiles/), or None until measured.
+TRAFFIC_BYTES_PER_LAUNCH = None
+
+if __name__ == "__main__":
+    main()

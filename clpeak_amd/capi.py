@@ -74,8 +74,8 @@ def load_library(path=LIB_PATH):
     lib.mi355_global_bandwidth.argtypes = [vp, i32, vp, u64, vp, u32, u32]
     lib.mi355_compute_mad.argtypes = [vp, i32, i32, u64, u64, u32, vp, u32]
     lib.mi355_launch_roundtrip.argtypes = [vp, u32, u32, C.POINTER(C.c_double)]
-    lib.mi355_mfma_dense.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, u32]
-    lib.mi355_smfmac.argtypes = [vp, i32, vp, vp, vp, vp, u32, u32]
+    lib.mi355_mfma_dense.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, u32, vp]
+    lib.mi355_smfmac.argtypes = [vp, i32, vp, vp, vp, vp, u32, u32, vp]
     lib.mi355_mfma_raw.argtypes = [vp, i32, i32, vp, vp, vp, vp, vp, i32, i32, vp]
     lib.mi355_gemm_bf16.argtypes = [vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_gemm_fp8_e4m3.argtypes = [vp, vp, vp, vp, u32, u32, u32, C.c_float, C.c_float]
@@ -187,12 +187,14 @@ class Device:
         self._check(self.lib.mi355_launch_roundtrip(self.h, warmup, launches, C.byref(us)))
         return us.value
 
-    def mfma_dense(self, kind, A, B, scaleA, scaleB, out, waves, iters):
+    def mfma_dense(self, kind, A, B, scaleA, scaleB, out, waves, iters, clocks=None):
         self._check(self.lib.mi355_mfma_dense(self.h, kind, A.ptr, B.ptr, scaleA.ptr if scaleA else None,
-                                              scaleB.ptr if scaleB else None, out.ptr, waves, iters))
+                                              scaleB.ptr if scaleB else None, out.ptr, waves, iters,
+                                              clocks.ptr if clocks else None))
 
-    def smfmac(self, kind, Ac, meta, B, out, waves, iters):
-        self._check(self.lib.mi355_smfmac(self.h, kind, Ac.ptr, meta.ptr, B.ptr, out.ptr, waves, iters))
+    def smfmac(self, kind, Ac, meta, B, out, waves, iters, clocks=None):
+        self._check(self.lib.mi355_smfmac(self.h, kind, Ac.ptr, meta.ptr, B.ptr, out.ptr, waves, iters,
+                                          clocks.ptr if clocks else None))
 
     def mfma_raw(self, sparse, kind, a, b, c, aux0, aux1, sel0, sel1, d):
         self._check(self.lib.mi355_mfma_raw(self.h, int(sparse), kind, a.ptr, b.ptr, c.ptr, aux0.ptr, aux1.ptr,

@@ -58,7 +58,9 @@ extern "C" int mi355_open(int ordinal, mi355_dev **out) {
 
   mi355_dev *d = new mi355_dev();
   d->ordinal = ordinal;
-  snprintf(d->props.name, sizeof(d->props.name), "%s", p.name);
+  // Some driver stacks report an empty marketing name; rows need a device string.
+  if (p.name[0]) snprintf(d->props.name, sizeof(d->props.name), "%s", p.name);
+  else snprintf(d->props.name, sizeof(d->props.name), "AMD GPU %.6s", p.gcnArchName);
   snprintf(d->props.arch, sizeof(d->props.arch), "%s", p.gcnArchName);
   int drv = 0, rt = 0;
   (void)hipDriverGetVersion(&drv);

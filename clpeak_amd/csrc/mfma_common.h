@@ -11,14 +11,23 @@
 //   B operand: lane l holds column (l % 32), same K range.
 //   C/D:       register r (0..15) of lane l is element
 //              (row 8*(r/4) + 4*(l/32) + r%4, column l % 32).
-// Scaled f8f6f4, 16x16x128: lane l carries the E8M0 scale of its own 32-element K
-//   block (row/column l % 16, block l/16) in the byte of the scale register that
-//   op_sel names.
-// SMFMAC 16x16xK (K = 64 for 16-bit, 128 for 8-bit data): A holds the K/2 kept values
-//   of row (l % 16): lane l has kept values [ (l/16)*K/8, (l/16+1)*K/8 ), which belong
-//   to dense K range [ (l/16)*K/4, (l/16+1)*K/4 ) -- the range of B that lane l/16
-//   group holds.  The index register carries two 2-bit positions per group of four,
-//   first kept value in the lower bits, groups in K order from bit 0.
+// f8f6f4, 16x16x128.  6-bit and 4-bit codes follow the rule above (lane l holds the 32
+//   consecutive K elements of block l/16).  8-bit codes do not: the 32 bytes of lane l
+//   are K elements [ 16*(l/16), +16 ) followed by [ 64 + 16*(l/16), +16 ), i.e. two
+//   K=64 operands back to back.  In every case the E8M0 scale of 32-element block b of
+//   row/column r is taken from lane (r + 16*b), from the byte of the scale register
+//   that op_sel names.
+// SMFMAC 16x16xK (K = 64 for 16-bit, 128 for 8-bit data):
+//   A holds the K/2 kept values of row (l % 16): lane l has kept values
+//     [ (l/16)*K/8, (l/16+1)*K/8 ), i.e. the kept values of dense K range
+//     [ (l/16)*K/4, (l/16+1)*K/4 ).
+//   B is laid out as two dense half-K operands back to back: the first half of lane
+//     l's registers holds K elements [ (l/16)*K/8, (l/16+1)*K/8 ) of column (l % 16), the
+//     second half holds [ K/2 + (l/16)*K/8, K/2 + (l/16+1)*K/8 ).  In bytes both kinds
+//     read 16 bytes at row offset 16*(l/16) and 16 bytes at 64 + 16*(l/16).
+//   The index register carries two 2-bit positions per group of four, the first kept
+//     value in the lower bits, groups in K order from bit 0 (16 index bits for 16-bit
+//     data, ABID picks the half of the register; 32 bits for 8-bit data).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>

@@ -104,7 +104,16 @@ MI355_DENSE_TRAIT(I8_16x16x64, 16, 16, 64, 64, i32x4v, i32x4v, int32_t, "v_mfma_
     static constexpr bool scaled = SCALED;                                                         \
     using Frag = FRAG; using Acc = f32x4v; using Out = float;                                      \
     __device__ static Frag load(const uint8_t *rows, int lane) {                                   \
-      return load_fragment<Frag, 16, row_bytes, BITS * 4>(rows, lane);                             \
+      if constexpr (BITS == 8) { /* K elements [16g,+16) then [64+16g,+16), g = lane/16 */         \
+        const uint8_t *p = rows + (lane % 16) * row_bytes + (lane / 16) * 16;                      \
+        const i32x4v lo = load_bytes<i32x4v>(p), hi = load_bytes<i32x4v>(p + 64);                  \
+        const i32x8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};              \
+        Frag f;                                                                                    \
+        __builtin_memcpy(&f, &both, sizeof(f)); /* Frag is i32x8v on this branch */                \
+        return f;                                                                                  \
+      } else {                                                                                     \
+        return load_fragment<Frag, 16, row_bytes, BITS * 4>(rows, lane);                           \
+      }                                                                                            \
     }                                                                                              \
     MI355_DEFINE_STEPS_SCALED("v_mfma_scale_f32_16x16x128_f8f6f4", TAIL)                           \
   };
@@ -119,7 +128,7 @@ template <typename Tr>
 __global__ void __launch_bounds__(256)
 mfma_dense_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B,
                   const uint8_t *__restrict__ sA, const uint8_t *__restrict__ sB,
-                  typename Tr::Out *__restrict__ out, uint32_t iters) {
+                  typename Tr::Out *__restrict__ out, uint32_t iters, uint64_t *__restrict__ clocks) {
   const int lane = threadIdx.x % 64;
   const uint64_t wave = (uint64_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
   constexpr size_t a_bytes = (size_t)Tr::M * Tr::row_bytes, b_bytes = (size_t)Tr::N * Tr::row_bytes;
@@ -145,6 +154,7 @@ mfma_dense_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B,
   }
 
   const uint32_t blocks = iters / kBlock, rest = iters % kBlock;
+  const uint64_t t0 = clock64(), r0 = wall_clock64();
 #pragma unroll 1
   for (uint32_t it = 0; it < blocks; it++) Tr::block(acc, a, b, sa, sb);
 #pragma unroll 1
@@ -153,6 +163,10 @@ mfma_dense_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B,
   // not insert the wait states a VALU/VMEM read of their results needs: cover the
   // longest case (a 16-pass MFMA result read by a store) by hand.
   asm volatile("s_nop 15\n s_nop 15" ::: "memory");
+  if (clocks != nullptr && wave == 0 && lane == 0) {
+    clocks[0] = clock64() - t0;
+    clocks[1] = wall_clock64() - r0;
+  }
 
 #pragma unroll
   for (int c = 0; c < kChains; c++) {
@@ -169,10 +183,10 @@ mfma_dense_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B,
 
 template <typename Tr>
 int launch(mi355_dev *dev, const void *A, const void *B, const uint8_t *sA, const uint8_t *sB, void *out,
-           uint32_t waves, uint32_t iters) {
+           uint32_t waves, uint32_t iters, uint64_t *clocks) {
   if (Tr::scaled && (!sA || !sB)) return mi355_fail(dev, MI355_ERR_ARG, "mfma_dense: scaled kind needs scaleA and scaleB");
   mfma_dense_kernel<Tr><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)A, (const uint8_t *)B, sA, sB,
-                                                           (typename Tr::Out *)out, iters);
+                                                           (typename Tr::Out *)out, iters, clocks);
   MI355_LAUNCH_CHECK(dev, "mfma_dense");
   return MI355_OK;
 }
@@ -180,22 +194,22 @@ int launch(mi355_dev *dev, const void *A, const void *B, const uint8_t *sA, cons
 }  // namespace
 
 extern "C" int mi355_mfma_dense(mi355_dev *dev, int kind, const void *A, const void *B, const uint8_t *scaleA,
-                                const uint8_t *scaleB, void *out, uint32_t waves, uint32_t iters) {
+                                const uint8_t *scaleB, void *out, uint32_t waves, uint32_t iters, uint64_t *clocks) {
   MI355_ENTER(dev);
   MI355_REQUIRE(dev, A && B && out, "mfma_dense: null buffer");
   MI355_REQUIRE(dev, waves > 0 && waves % 4 == 0, "mfma_dense: waves (%u) must be a positive multiple of 4", waves);
   MI355_REQUIRE(dev, (((uintptr_t)A | (uintptr_t)B | (uintptr_t)out) & 15u) == 0, "mfma_dense: buffers must be 16-byte aligned");
   switch (kind) {
-    case MI355_MFMA_F16_16x16x32:  return launch<F16_16x16x32>(dev, A, B, scaleA, scaleB, out, waves, iters);
-    case MI355_MFMA_BF16_16x16x32: return launch<BF16_16x16x32>(dev, A, B, scaleA, scaleB, out, waves, iters);
-    case MI355_MFMA_F16_32x32x16:  return launch<F16_32x32x16>(dev, A, B, scaleA, scaleB, out, waves, iters);
-    case MI355_MFMA_BF16_32x32x16: return launch<BF16_32x32x16>(dev, A, B, scaleA, scaleB, out, waves, iters);
-    case MI355_MFMA_I8_16x16x64:   return launch<I8_16x16x64>(dev, A, B, scaleA, scaleB, out, waves, iters);
-    case MI355_MFMA_FP8_16x16x128: return launch<FP8_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
-    case MI355_MFMA_BF8_16x16x128: return launch<BF8_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
-    case MI355_MFMA_MXFP6_E2M3:    return launch<FP6_E2M3_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
-    case MI355_MFMA_MXFP6_E3M2:    return launch<FP6_E3M2_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
-    case MI355_MFMA_MXFP4_E2M1:    return launch<FP4_E2M1_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters);
+    case MI355_MFMA_F16_16x16x32:  return launch<F16_16x16x32>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_BF16_16x16x32: return launch<BF16_16x16x32>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_F16_32x32x16:  return launch<F16_32x32x16>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_BF16_32x32x16: return launch<BF16_32x32x16>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_I8_16x16x64:   return launch<I8_16x16x64>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_FP8_16x16x128: return launch<FP8_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_BF8_16x16x128: return launch<BF8_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_MXFP6_E2M3:    return launch<FP6_E2M3_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_MXFP6_E3M2:    return launch<FP6_E3M2_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_MXFP4_E2M1:    return launch<FP4_E2M1_16x16x128>(dev, A, B, scaleA, scaleB, out, waves, iters, clocks);
     default: return mi355_fail(dev, MI355_ERR_ARG, "mfma_dense: unknown kind %d", kind);
   }
 }

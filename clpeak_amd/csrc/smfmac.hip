@@ -53,7 +53,7 @@ MI355_SPARSE_TRAIT(SP_I8, 128, 1, i32x4v, i32x8v, i32x4v, int32_t, "v_smfmac_i32
 template <typename Tr>
 __global__ void __launch_bounds__(256)
 smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, const uint8_t *__restrict__ B,
-              typename Tr::Out *__restrict__ out, uint32_t iters) {
+              typename Tr::Out *__restrict__ out, uint32_t iters, uint64_t *__restrict__ clocks) {
   const int lane = threadIdx.x % 64;
   const uint64_t wave = (uint64_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
   constexpr int K = Tr::K;
@@ -68,7 +68,12 @@ smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, 
   for (int c = 0; c < kChains; c++) {
     const uint64_t u = wave * kChains + c;
     a[c] = load_bytes<typename Tr::FragA>(Ac + u * 16 * ac_row + (lane % 16) * ac_row + (lane / 16) * (ac_row / 4));
-    b[c] = load_bytes<typename Tr::FragB>(B + u * 16 * b_row + (lane % 16) * b_row + (lane / 16) * (b_row / 4));
+    {  // B: 16 bytes of the first K half and 16 bytes of the second (b_row is 128 for every kind)
+      const uint8_t *brow = B + u * 16 * b_row + (lane % 16) * b_row + (lane / 16) * 16;
+      const i32x4v lo = load_bytes<i32x4v>(brow), hi = load_bytes<i32x4v>(brow + b_row / 2);
+      const i32x8v both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      __builtin_memcpy(&b[c], &both, sizeof(both));
+    }
     const uint8_t *m = meta + u * 16 * m_row + (lane % 16) * m_row + (lane / 16) * groups;
     uint32_t packed = 0;
 #pragma unroll
@@ -79,12 +84,17 @@ smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, 
   }
 
   const uint32_t blocks = iters / kBlock, rest = iters % kBlock;
+  const uint64_t t0 = clock64(), r0 = wall_clock64();
 #pragma unroll 1
   for (uint32_t it = 0; it < blocks; it++) Tr::block(acc, a, b, idx);
 #pragma unroll 1
   for (uint32_t it = 0; it < rest; it++) Tr::single(acc, a, b, idx);
   // Wait states the compiler cannot know are needed before the results are read.
   asm volatile("s_nop 15\n s_nop 15" ::: "memory");
+  if (clocks != nullptr && wave == 0 && lane == 0) {
+    clocks[0] = clock64() - t0;
+    clocks[1] = wall_clock64() - r0;
+  }
 
 #pragma unroll
   for (int c = 0; c < kChains; c++) {
@@ -96,9 +106,9 @@ smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, 
 
 template <typename Tr>
 int launch(mi355_dev *dev, const void *Ac, const uint8_t *meta, const void *B, void *out, uint32_t waves,
-           uint32_t iters) {
+           uint32_t iters, uint64_t *clocks) {
   smfmac_kernel<Tr><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)Ac, meta, (const uint8_t *)B,
-                                                       (typename Tr::Out *)out, iters);
+                                                       (typename Tr::Out *)out, iters, clocks);
   MI355_LAUNCH_CHECK(dev, "smfmac");
   return MI355_OK;
 }
@@ -106,17 +116,17 @@ int launch(mi355_dev *dev, const void *Ac, const uint8_t *meta, const void *B, v
 }  // namespace
 
 extern "C" int mi355_smfmac(mi355_dev *dev, int kind, const void *Ac, const uint8_t *meta, const void *B,
-                            void *out, uint32_t waves, uint32_t iters) {
+                            void *out, uint32_t waves, uint32_t iters, uint64_t *clocks) {
   MI355_ENTER(dev);
   MI355_REQUIRE(dev, Ac && meta && B && out, "smfmac: null buffer");
   MI355_REQUIRE(dev, waves > 0 && waves % 4 == 0, "smfmac: waves (%u) must be a positive multiple of 4", waves);
   MI355_REQUIRE(dev, (((uintptr_t)Ac | (uintptr_t)B | (uintptr_t)out) & 15u) == 0, "smfmac: buffers must be 16-byte aligned");
   switch (kind) {
-    case MI355_SMFMAC_F16_16x16x64:  return launch<SP_F16>(dev, Ac, meta, B, out, waves, iters);
-    case MI355_SMFMAC_BF16_16x16x64: return launch<SP_BF16>(dev, Ac, meta, B, out, waves, iters);
-    case MI355_SMFMAC_FP8_16x16x128: return launch<SP_FP8>(dev, Ac, meta, B, out, waves, iters);
-    case MI355_SMFMAC_BF8_16x16x128: return launch<SP_BF8>(dev, Ac, meta, B, out, waves, iters);
-    case MI355_SMFMAC_I8_16x16x128:  return launch<SP_I8>(dev, Ac, meta, B, out, waves, iters);
+    case MI355_SMFMAC_F16_16x16x64:  return launch<SP_F16>(dev, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_BF16_16x16x64: return launch<SP_BF16>(dev, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_FP8_16x16x128: return launch<SP_FP8>(dev, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_BF8_16x16x128: return launch<SP_BF8>(dev, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_I8_16x16x128:  return launch<SP_I8>(dev, Ac, meta, B, out, waves, iters, clocks);
     default: return mi355_fail(dev, MI355_ERR_ARG, "smfmac: unknown kind %d", kind);
   }
 }

@@ -114,13 +114,17 @@ int mi355_global_bandwidth(mi355_dev *dev, int width, const float *in, uint64_t 
  * accumulators (as 16/width vectors of `width` lanes) seeded from stream
  * `MI355_STREAM_MAD` element item*16+j, `steps` dependent steps, out[item] = sum of
  * the 16 accumulators in index order (one element of the kernel's type). */
-#define MI355_MAD_F32      0  /* x = fma(x, a, x0), a = 1.0001f; x0 uniform[-1,1)           */
-#define MI355_MAD_F16      1  /* same in IEEE half (width 1: v_fma_f16, 2: v_pk_fma_f16)    */
-#define MI355_MAD_F64      2  /* same in double, a = 1.0001                                  */
-#define MI355_MAD_MP       3  /* fp32 accumulator, operands rounded through half each step   */
-#define MI355_MAD_BF16     4  /* fp32 accumulator, operands rounded through bf16 each step   */
-#define MI355_MAD_I32      5  /* x = x*a + x0 (wrapping), a = 3                              */
-#define MI355_MAD_I8DP     6  /* acc = sdot4(x, y, acc); y ^= acc; `width` = number of chains */
+#define MI355_MAD_F32      0  /* x = fma(x, a, x0), a = 1.0001f, x0 uniform[-1,1); widths 1,2,4          */
+#define MI355_MAD_F16      1  /* same in IEEE half, a = 1-2^-10 (1.0001 is 1.0 in half), x0 = half(u);
+                                 width 1: scalar half FMA, 2: packed half2 FMA; out is half bits        */
+#define MI355_MAD_F64      2  /* same in double, a = 1.0001; widths 1,2,4                               */
+#define MI355_MAD_MP       3  /* acc = fma(float(xh), float(ah), acc) in fp32, xh = half(u), acc0 = xh,
+                                 ah = 1-2^-10: half x half + float; width 1                             */
+#define MI355_MAD_BF16     4  /* same with bf16 operands, ab = 1-2^-8; width 1                          */
+#define MI355_MAD_I32      5  /* x = x*3 + x0 (wrapping), x0 = high 32 bits of the word; widths 1,2,4   */
+#define MI355_MAD_I8DP     6  /* acc = sdot4(x, y, acc); y ^= acc; `width` in {1,2,4,8} = number of
+                                 independent chains (x, y from element item*8+chain of streams
+                                 MI355_STREAM_MAD / MI355_STREAM_MAD_Y), out = sum of the chains' acc    */
 int mi355_compute_mad(mi355_dev *dev, int kind, int width, uint64_t seed,
                       uint64_t n_items, uint32_t steps, void *out, uint32_t block_size);
 
@@ -143,7 +147,10 @@ int mi355_launch_roundtrip(mi355_dev *dev, uint32_t warmup, uint32_t launches, d
  * 3 bytes and fp4 2 codes per byte, little-endian bit order along K.
  * Scaled kinds take scaleA[wave][chain][M][K/32] and scaleB[wave][chain][N][K/32]
  * E8M0 bytes (value 2^(byte-127)); other kinds pass NULL.
- * waves must be a multiple of 4 (a workgroup is 4 waves). */
+ * waves must be a multiple of 4 (a workgroup is 4 waves).
+ * clocks (may be NULL): two uint64 in device memory; wave 0 stores the shader-clock
+ * ticks and the 100 MHz reference-clock ticks its MFMA loop took, from which the
+ * caller derives the clock the chip actually held under this load. */
 #define MI355_MFMA_F16_16x16x32     0
 #define MI355_MFMA_BF16_16x16x32    1
 #define MI355_MFMA_F16_32x32x16     2
@@ -157,7 +164,7 @@ int mi355_launch_roundtrip(mi355_dev *dev, uint32_t warmup, uint32_t launches, d
 #define MI355_MFMA_KIND_COUNT      10
 int mi355_mfma_dense(mi355_dev *dev, int kind, const void *A, const void *B,
                      const uint8_t *scaleA, const uint8_t *scaleB,
-                     void *out, uint32_t waves, uint32_t iters);
+                     void *out, uint32_t waves, uint32_t iters, uint64_t *clocks);
 
 /* ---- 2:4 structured-sparse SMFMAC --------------------------------------------- */
 /* Takes over smfmac_fp16/bf16/fp8/int8 (src/rocm/rocm_kernels/smfmac_*.hip) and their
@@ -166,7 +173,8 @@ int mi355_mfma_dense(mi355_dev *dev, int kind, const void *A, const void *B,
  *   meta[wave][chain][M][K/4] one byte per group: bits[1:0] = position (0..3) of the
  *                             first kept value, bits[3:2] = position of the second
  *   B[wave][chain][N][K]      dense, K contiguous;  out as for mi355_mfma_dense.
- * K is the dense-equivalent depth (64 for 16-bit kinds, 128 for 8-bit kinds). */
+ * K is the dense-equivalent depth (64 for 16-bit kinds, 128 for 8-bit kinds).
+ * clocks: as for mi355_mfma_dense. */
 #define MI355_SMFMAC_F16_16x16x64    0
 #define MI355_SMFMAC_BF16_16x16x64   1
 #define MI355_SMFMAC_FP8_16x16x128   2
@@ -174,7 +182,7 @@ int mi355_mfma_dense(mi355_dev *dev, int kind, const void *A, const void *B,
 #define MI355_SMFMAC_I8_16x16x128    4
 #define MI355_SMFMAC_KIND_COUNT      5
 int mi355_smfmac(mi355_dev *dev, int kind, const void *Ac, const uint8_t *meta, const void *B,
-                 void *out, uint32_t waves, uint32_t iters);
+                 void *out, uint32_t waves, uint32_t iters, uint64_t *clocks);
 
 /* One matrix instruction on raw per-lane register images (no reference counterpart:
  * the reference never checks a result, so it never needed to know the operand

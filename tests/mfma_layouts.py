@@ -30,6 +30,19 @@ def operand_regs(rows_bytes, rows_mod, dwords):
     return regs.view("<u4").reshape(64, dwords)
 
 
+def split_k_regs(rows_bytes):
+    """rows_bytes[16][128] -> regs[64][8]: lane l holds bytes [16g, 16g+16) and
+    [64+16g, 64+16g+16) of row l % 16, g = l // 16 (two half-K operands back to back).
+    This is the B operand of every SMFMAC and both operands of the 8-bit f8f6f4 MFMA."""
+    assert rows_bytes.shape == (16, 128)
+    regs = np.zeros((64, 32), dtype=np.uint8)
+    for l in range(64):
+        g = l // 16
+        regs[l, :16] = rows_bytes[l % 16, 16 * g:16 * g + 16]
+        regs[l, 16:] = rows_bytes[l % 16, 64 + 16 * g:64 + 16 * g + 16]
+    return regs.view("<u4").reshape(64, 8)
+
+
 def c_regs_from_matrix(Cm):
     """C[M][N] (4-byte elements) -> regs[64][16]."""
     M, N = Cm.shape

@@ -1,9 +1,18 @@
 """GPU parity of the matrix-instruction kernels against the CPU oracle.
 
-Integer kinds are bit-exact.  Floating kinds: |gpu - oracle| <= TOL * iters*sum|a*b| per
-element (the oracle accumulates the exact dot product in fp32 once per iteration; the
-matrix pipe rounds inside the dot product too, so a relative-to-magnitude bound is the
-honest statement)."""
+Integer kinds are bit-exact.  Floating kinds cannot be: measured on gfx950, the matrix
+pipe neither forms the K-long dot product exactly (f16/bf16 and, much more so, fp8/bf8
+align the products with a limited number of bits; fp6/fp4 are exact) nor rounds the
+running fp32 accumulator to nearest every time.  The oracle accumulates the exact dot
+product with one fp32 round-to-nearest per iteration, and the stated tolerance is, per
+element,
+
+    |gpu - oracle| <= (DOT_TOL + iters * 2^-23) * iters * sum_k |a_k * b_k|
+
+i.e. 2^-14.6 of the product magnitudes for the dot product plus at most one unit in the
+last place of the accumulator per iteration, all in the same direction (the accumulator
+never exceeds iters * sum|a*b|).  At 4096 iterations this is 5.3e-4; the observed worst
+case is 1.4e-4."""
 import numpy as np
 import pytest
 
@@ -13,7 +22,7 @@ from oracle import workloads as wl
 
 pytestmark = pytest.mark.gpu
 SEED = wl.DEFAULT_SEED
-TOL = 1e-5   # relative to iters * sum|a_k * b_k|
+DOT_TOL = 4e-5   # relative to sum|a_k * b_k|, one instruction
 
 
 def _run_dense(dev, kind, waves, iters, seed=SEED):
@@ -34,12 +43,12 @@ def _run_dense(dev, kind, waves, iters, seed=SEED):
     return got, ref, ab, is_int
 
 
-def _check(got, ref, ab, is_int, what):
+def _check(got, ref, ab, is_int, what, iters):
     if is_int:
         assert np.array_equal(got, ref), what
     else:
         err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
-        bound = TOL * ab + 1e-30
+        bound = (DOT_TOL + iters * 2.0 ** -23) * ab + 1e-30
         worst = float((err / bound).max())
         assert worst <= 1.0, (what, worst, float(err.max()))
         assert np.count_nonzero(got) > got.size * 0.9, what   # a kernel that wrote nothing must not pass
@@ -49,7 +58,7 @@ def _check(got, ref, ab, is_int, what):
 @pytest.mark.parametrize("iters", [1, 13, 4096])
 def test_mfma_dense_parity(dev, kind, iters):
     got, ref, ab, is_int = _run_dense(dev, kind, 8, iters)
-    _check(got, ref, ab, is_int, (wl.DENSE[kind]["name"], iters))
+    _check(got, ref, ab, is_int, (wl.DENSE[kind]["name"], iters), iters)
 
 
 @pytest.mark.parametrize("kind", sorted(wl.DENSE))
@@ -57,7 +66,7 @@ def test_mfma_dense_full_launch_sampled(dev, kind):
     """The configured launch: 2048 waves x 4 chains x 4096 iterations.  The oracle replays
     every wave (seconds) and the whole output is compared."""
     got, ref, ab, is_int = _run_dense(dev, kind, 2048, 4096)
-    _check(got, ref, ab, is_int, wl.DENSE[kind]["name"])
+    _check(got, ref, ab, is_int, wl.DENSE[kind]["name"], 4096)
 
 
 def test_mfma_int8_linearity(dev):
@@ -86,10 +95,10 @@ def _run_sparse(dev, kind, waves, iters, seed=SEED):
 @pytest.mark.parametrize("iters", [1, 13, 4096])
 def test_smfmac_parity(dev, kind, iters):
     got, ref, ab, is_int = _run_sparse(dev, kind, 8, iters)
-    _check(got, ref, ab, is_int, (wl.SPARSE[kind]["name"], iters))
+    _check(got, ref, ab, is_int, (wl.SPARSE[kind]["name"], iters), iters)
 
 
 @pytest.mark.parametrize("kind", sorted(wl.SPARSE))
 def test_smfmac_full_launch(dev, kind):
     got, ref, ab, is_int = _run_sparse(dev, kind, 2048, 4096)
-    _check(got, ref, ab, is_int, wl.SPARSE[kind]["name"])
+    _check(got, ref, ab, is_int, wl.SPARSE[kind]["name"], 4096)
