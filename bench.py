@@ -221,8 +221,9 @@ def main():
     print(json.dumps(line))
 
 
-# Workgroups per CU of the headline launch (256 threads each).
-HEADLINE_BLOCKS_PER_CU = 8
+# Workgroups per CU of the headline launch (256 threads each); one per CU measured best (a
+# small grid keeps the strided loads of one unrolled group inside a few 2 MiB pages).
+HEADLINE_BLOCKS_PER_CU = 1
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (see profiles/), or None until measured.
 TRAFFIC_BYTES_PER_LAUNCH = None
 

@@ -49,7 +49,8 @@ mad_fp_kernel(uint64_t seed, T a, uint32_t steps, uint64_t n_items, T *__restric
   for (uint32_t s = 0; s < steps; s++) {
 #pragma unroll
     for (int v = 0; v < NV; v++) {
-      if constexpr (W == 1) x[v] = __builtin_fma(x[v], a, x0[v]);
+      // elementwise_fma is typed by its operands (the plain fma builtin is always double)
+      if constexpr (W == 1) x[v] = __builtin_elementwise_fma(x[v], a, x0[v]);
       else x[v] = __builtin_elementwise_fma(x[v], (Vec)(a), x0[v]);
     }
   }

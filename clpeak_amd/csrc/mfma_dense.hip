@@ -20,10 +20,14 @@ constexpr int kChains = 4;
 // copy next to an MFMA costs wait states.  One block = kBlock rounds over the 4
 // chains, accumulating in place (vDst == SrcC), which the matrix pipe executes
 // back to back with no software wait states: the next MFMA that touches the same
-// accumulator is 3 independent MFMAs away.
-constexpr int kBlock = 8;
+// accumulator is 3 independent MFMAs away.  A block is 128 instructions because the
+// loop branch costs the issuing wave about 20 cycles in which the pipe idles (waves of
+// one SIMD run one after the other here: the oldest always has an MFMA ready and wins
+// arbitration), 4 % at 32 instructions per trip and 1 % at 128.
+constexpr int kBlock = 32;
 
 #define MI355_REP8(x) x x x x x x x x
+#define MI355_REP32(x) MI355_REP8(x) MI355_REP8(x) MI355_REP8(x) MI355_REP8(x)
 // %0-%3 accumulators, %4-%7 A fragments, %8-%11 B fragments
 #define MI355_ROUND(INSN, TAIL)                \
   INSN " %0, %4, %8, %0" TAIL "\n"             \
@@ -40,7 +44,7 @@ constexpr int kBlock = 8;
 #define MI355_DEFINE_STEPS(INSN, TAIL)                                                             \
   __device__ static void block(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&)[4], \
                                const int (&)[4]) {                                                 \
-    asm volatile(MI355_REP8(MI355_ROUND(INSN, TAIL))                                               \
+    asm volatile(MI355_REP32(MI355_ROUND(INSN, TAIL))                                               \
                  : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
                  : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3])); \
   }                                                                                                \
@@ -54,7 +58,7 @@ constexpr int kBlock = 8;
 #define MI355_DEFINE_STEPS_SCALED(INSN, TAIL)                                                      \
   __device__ static void block(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&sa)[4], \
                                const int (&sb)[4]) {                                               \
-    asm volatile(MI355_REP8(MI355_ROUND_SCALED(INSN, TAIL))                                        \
+    asm volatile(MI355_REP32(MI355_ROUND_SCALED(INSN, TAIL))                                        \
                  : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
                  : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), \
                    "v"(sa[0]), "v"(sa[1]), "v"(sa[2]), "v"(sa[3]), "v"(sb[0]), "v"(sb[1]), "v"(sb[2]), "v"(sb[3])); \

@@ -16,8 +16,9 @@ constexpr int kChains = 4;
 // The hot loop is inline assembly for the reason given in mfma_dense.hip: accumulate
 // in place, 4 independent chains, no copies between matrix instructions.  SMFMAC takes
 // its accumulator from the destination registers: D = A*B + D.
-constexpr int kBlock = 8;
+constexpr int kBlock = 32;
 #define MI355_REP8(x) x x x x x x x x
+#define MI355_REP32(x) MI355_REP8(x) MI355_REP8(x) MI355_REP8(x) MI355_REP8(x)
 // %0-%3 accumulators, %4-%7 compressed A, %8-%11 B, %12-%15 index registers
 #define MI355_SP_ROUND(INSN)       \
   INSN " %0, %4, %8, %12\n"        \
@@ -37,7 +38,7 @@ constexpr int kBlock = 8;
     static constexpr int K = K_, elem = ELEM;                                                      \
     using FragA = FRAGA; using FragB = FRAGB; using Acc = ACC; using Out = OUT;                    \
     __device__ static void block(Acc (&acc)[4], const FragA (&a)[4], const FragB (&b)[4], const int (&idx)[4]) { \
-      asm volatile(MI355_REP8(MI355_SP_ROUND(INSN)) MI355_SP_OPERANDS);                            \
+      asm volatile(MI355_REP32(MI355_SP_ROUND(INSN)) MI355_SP_OPERANDS);                            \
     }                                                                                              \
     __device__ static void single(Acc (&acc)[4], const FragA (&a)[4], const FragB (&b)[4], const int (&idx)[4]) { \
       asm volatile(MI355_SP_ROUND(INSN) MI355_SP_OPERANDS);                                        \
