@@ -45,7 +45,7 @@ def timed(dev, launch, min_us=300e3, warm_us=300e3, max_iters=10000):
     return dev.time_launches(launch, n) / n, n
 
 
-def bench_rows(dev, quick):
+def bench_rows(dev, quick, only):
     from clpeak_amd import capi
     from oracle import workloads as wl
     rows = []
@@ -59,6 +59,19 @@ def bench_rows(dev, quick):
         r.update(extra)
         rows.append(r)
 
+    if "mad" in only:
+        _mad_rows(dev, capi, add, budget)
+    if "latency" in only:
+        us = dev.launch_roundtrip(2, 10000)
+        add("kernel_launch_latency", "roundtrip", us, "us", us)
+    if "mfma" in only or "smfmac" in only:
+        _matrix_rows(dev, wl, add, budget, only)
+    if "gemm" in only:
+        _gemm_rows(dev, capi, wl, add, budget)
+    return rows
+
+
+def _mad_rows(dev, capi, add, budget):
     # --- vector MAD chains: 2^20 work-items x 16 accumulators x 4096 steps -------------
     n_items, steps = 1 << 20, 4096
     out = dev.alloc(n_items * 8)
@@ -77,15 +90,13 @@ def bench_rows(dev, quick):
         add("integer_compute_int8_dp", metric, n_items * chains * steps * 8 / us / 1e3, "gops", us)
     out.free()
 
-    # --- launch latency ------------------------------------------------------------------
-    us = dev.launch_roundtrip(2, 10000)
-    add("kernel_launch_latency", "roundtrip", us, "us", us)
 
+def _matrix_rows(dev, wl, add, budget, only):
     # --- dense MFMA / SMFMAC: 2048 waves x 4 chains x 4096 iterations ------------------------
     waves, iters = 2048, 4096
     clk = dev.alloc(16)
     peaks = {0: "f16", 1: "bf16", 2: "f16", 3: "bf16", 4: "int8", 5: "fp8", 6: "fp8", 7: "fp6", 8: "fp6", 9: "fp4"}
-    for kind in sorted(wl.DENSE):
+    for kind in sorted(wl.DENSE) if "mfma" in only else []:
         s = wl.DENSE[kind]
         A, B, sA, sB = wl.dense_inputs(kind, waves, SEED)
         bufs = [dev.from_host(A), dev.from_host(B), dev.from_host(sA) if sA is not None else None,
@@ -100,7 +111,7 @@ def bench_rows(dev, quick):
             if b is not None:
                 b.free()
     speaks = {0: "f16", 1: "bf16", 2: "fp8", 3: "fp8", 4: "int8"}
-    for kind in sorted(wl.SPARSE):
+    for kind in sorted(wl.SPARSE) if "smfmac" in only else []:
         s = wl.SPARSE[kind]
         Ac, meta, B = wl.sparse_inputs(kind, waves, SEED)
         bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
@@ -114,6 +125,8 @@ def bench_rows(dev, quick):
             b.free()
     clk.free()
 
+
+def _gemm_rows(dev, capi, wl, add, budget):
     # --- GEMM 8192^3 ---------------------------------------------------------------------------
     M = N = K = 8192
     for fp8 in (False, True):
@@ -132,7 +145,6 @@ def bench_rows(dev, quick):
             PEAK["fp8" if fp8 else "bf16"], shape="8192x8192x8192")
         for b in (dA, dB, dC):
             b.free()
-    return rows
 
 
 def cpu_baseline(seconds=12.0):
@@ -163,6 +175,11 @@ def main():
     ap.add_argument("--no-rows", action="store_true", help="headline kernel only")
     ap.add_argument("--quick", action="store_true", help="shorter time budget per extra row")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only the plain copy kernel over 1 GiB (20 launches): under rocprofv3 --pmc this "
+                         "gives what FETCH_SIZE / WRITE_SIZE read for a transfer of known size")
+    ap.add_argument("--only", default="mad,latency,mfma,smfmac,gemm",
+                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,gemm")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; the hot path has no multi-GPU step "
@@ -171,6 +188,16 @@ def main():
     from clpeak_amd import capi
     from oracle import workloads as wl
     dev = capi.Device(0)
+
+    if args.calibrate_copy:
+        nbytes = 1 << 30
+        a, b = dev.alloc(nbytes), dev.alloc(nbytes)
+        dev.fill_f32(a, nbytes // 4, SEED, wl.STREAM_BW, capi.DIST_U01)
+        for _ in range(20):
+            dev.copy(b, a, nbytes)
+        dev.sync()
+        print(json.dumps({"calibrate_copy_bytes": nbytes, "launches": 20}))
+        return
 
     n = 1 << 30                                   # 4 GiB of fp32, far past the 256 MB Infinity Cache
     src = dev.alloc(n * 4)
@@ -200,7 +227,7 @@ def main():
                      "us_per_launch": round(us, 2), "peak": HBM_PEAK_GBPS, "frac": round(n * 4 / us / 1e3 / HBM_PEAK_GBPS, 4)})
     src.free(); out.free()
     if not args.no_rows:
-        rows += bench_rows(dev, args.quick)
+        rows += bench_rows(dev, args.quick, set(args.only.split(",")))
     dev.close()
 
     achieved = n * 4 / kernel_us / 1e3
@@ -224,8 +251,10 @@ def main():
 # Workgroups per CU of the headline launch (256 threads each); one per CU measured best (a
 # small grid keeps the strided loads of one unrolled group inside a few 2 MiB pages).
 HEADLINE_BLOCKS_PER_CU = 1
-# HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (see profiles/), or None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in
+# KiB per dispatch), each scaled by what the counter reads for the plain copy kernel of known size
+# (FETCH_SIZE x 2.0000, WRITE_SIZE x 1.0000): profiles/hbm_float4_read_4GiB_traffic.md.
+TRAFFIC_BYTES_PER_LAUNCH = 4295155713
 
 if __name__ == "__main__":
     main()

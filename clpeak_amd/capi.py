@@ -16,7 +16,7 @@ SYMBOLS = [
     "mi355_device_count", "mi355_open", "mi355_close", "mi355_get_props", "mi355_last_error",
     "mi355_alloc", "mi355_free", "mi355_upload", "mi355_download", "mi355_memset", "mi355_sync",
     "mi355_timer_start", "mi355_timer_stop",
-    "mi355_fill_f32", "mi355_fill_bf16", "mi355_fill_fp8_e4m3",
+    "mi355_fill_f32", "mi355_fill_bf16", "mi355_fill_fp8_e4m3", "mi355_copy",
     "mi355_global_bandwidth", "mi355_compute_mad", "mi355_launch_roundtrip",
     "mi355_mfma_dense", "mi355_smfmac", "mi355_mfma_raw",
     "mi355_gemm_bf16", "mi355_gemm_fp8_e4m3",
@@ -71,6 +71,7 @@ def load_library(path=LIB_PATH):
     lib.mi355_fill_f32.argtypes = [vp, vp, u64, u64, u32, i32]
     lib.mi355_fill_bf16.argtypes = [vp, vp, u64, u64, u32, i32]
     lib.mi355_fill_fp8_e4m3.argtypes = [vp, vp, u64, u64, u32, i32, C.c_float]
+    lib.mi355_copy.argtypes = [vp, vp, vp, C.c_size_t]
     lib.mi355_global_bandwidth.argtypes = [vp, i32, vp, u64, vp, u32, u32]
     lib.mi355_compute_mad.argtypes = [vp, i32, i32, u64, u64, u32, vp, u32]
     lib.mi355_launch_roundtrip.argtypes = [vp, u32, u32, C.POINTER(C.c_double)]
@@ -175,6 +176,9 @@ class Device:
 
     def fill_fp8_e4m3(self, buf, n, seed, stream, dist, scale):
         self._check(self.lib.mi355_fill_fp8_e4m3(self.h, buf.ptr, n, seed, stream, dist, scale))
+
+    def copy(self, dst, src, nbytes):
+        self._check(self.lib.mi355_copy(self.h, dst.ptr, src.ptr, nbytes))
 
     def global_bandwidth(self, width, inbuf, n_floats, outbuf, blocks, block_size=256):
         self._check(self.lib.mi355_global_bandwidth(self.h, width, inbuf.ptr, n_floats, outbuf.ptr, blocks, block_size))

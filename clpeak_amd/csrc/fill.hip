@@ -32,6 +32,12 @@ __global__ void fill_fp8_kernel(uint8_t *dst, uint64_t n, uint64_t seed, uint32_
     dst[i] = mi355_f32_to_e4m3(draw(seed, stream, i, dist) * scale);
 }
 
+typedef int copy_vec __attribute__((ext_vector_type(4)));
+__global__ void copy_kernel(copy_vec *__restrict__ dst, const copy_vec *__restrict__ src, uint64_t n) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
 uint32_t fill_grid(uint64_t n) {
   uint64_t blocks = (n + kFillBlock - 1) / kFillBlock;
   const uint64_t cap = 256u * 32u;  // 32 workgroups per CU is plenty for a store-bound fill
@@ -71,5 +77,15 @@ extern "C" int mi355_fill_fp8_e4m3(mi355_dev *dev, uint8_t *dst, uint64_t n, uin
   if (int rc = check_fill(dev, dst, n, dist)) return rc;
   fill_fp8_kernel<<<fill_grid(n), kFillBlock, 0, dev->stream>>>(dst, n, seed, stream, dist, scale);
   MI355_LAUNCH_CHECK(dev, "fill_fp8_e4m3");
+  return MI355_OK;
+}
+
+extern "C" int mi355_copy(mi355_dev *dev, void *dst, const void *src, size_t bytes) {
+  MI355_ENTER(dev);
+  MI355_REQUIRE(dev, dst && src, "copy: null pointer");
+  MI355_REQUIRE(dev, bytes > 0 && bytes % 16 == 0, "copy: size must be a positive multiple of 16");
+  MI355_REQUIRE(dev, (((uintptr_t)dst | (uintptr_t)src) & 15u) == 0, "copy: pointers must be 16-byte aligned");
+  copy_kernel<<<fill_grid(bytes / 16), kFillBlock, 0, dev->stream>>>((copy_vec *)dst, (const copy_vec *)src, bytes / 16);
+  MI355_LAUNCH_CHECK(dev, "copy");
   return MI355_OK;
 }

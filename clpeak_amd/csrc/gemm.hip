@@ -21,14 +21,13 @@
 // 1 KiB destination, so lane i fetches the global chunk that belongs there.
 //
 // Schedule of one step (bf16: two K=32 halves, fragment sets F0 and F1):
-//     issue the 12 LDS reads of F1          | F0 was read during the previous step
-//     32 MFMAs on F0
+//     32 MFMAs on F0, the 12 LDS reads of F1 slipped between the first 20
 //     wait F1; wait own global loads; barrier      <- slab s+1 complete, slab s free
-//     issue global->LDS loads of slab s+2 into the freed buffer
-//     issue the 12 LDS reads of the next step's F0
-//     32 MFMAs on F1
-// One barrier per step, and no MFMA waits on an LDS read issued less than 32 MFMAs
-// earlier.  The loop body is inline assembly so that this order is the order issued;
+//     32 MFMAs on F1; between them the 12 LDS reads of the next step's F0 and the 8
+//     global->LDS loads of slab s+2 into the freed buffer
+// One barrier per step; an MFMA is always the first thing a wave issues after the barrier
+// (its operands are already in registers), memory instructions are spread out so that a
+// wave never sits on a full memory queue with MFMAs waiting behind it.  The loop body is inline assembly so that this order is the order issued;
 // the compiler knows neither the LDS reads nor the MFMAs and therefore inserts no wait
 // states of its own: every s_waitcnt below is part of the schedule.
 //
@@ -83,13 +82,10 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
 #define MI355_MFMA_BF16(acc, fb, fa) \
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(fb), "v"(fa))
 
-template <typename Frag>
-__device__ inline void mfma_block_bf16(f32x4v (&acc)[8][4], const Frag (&fa)[8], const Frag (&fb)[4]) {
-#pragma unroll
-  for (int i = 0; i < 8; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) MI355_MFMA_BF16(acc[i][j], fb[j], fa[i]);
-}
+// One row of MFMAs: the 4 tiles that share A fragment i.
+#define MI355_MFMA_ROW(acc, fa, fb, i)                                                             \
+  MI355_MFMA_BF16(acc[i][0], fb[0], fa[i]); MI355_MFMA_BF16(acc[i][1], fb[1], fa[i]);              \
+  MI355_MFMA_BF16(acc[i][2], fb[2], fa[i]); MI355_MFMA_BF16(acc[i][3], fb[3], fa[i])
 
 __device__ inline void tile_of_block(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn) {
   const uint32_t bid = blockIdx.x, total = tiles_m * tiles_n;
@@ -151,20 +147,57 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, u
   MI355_READ_FRAGS(fa0, fb0, a_cur, b_cur);
   MI355_WAIT_FRAGS(fa0, fb0);
 
+  // Per-lane global pointers of the next slab to fetch (advanced by one step per trip) and
+  // the wave's LDS destination for it.
+  const uint8_t *ga_next = ga + 2 * (size_t)kRowBytes, *gb_next = gb + 2 * (size_t)kRowBytes;
+  const size_t row8 = 8 * (size_t)k_bytes;
+
   for (uint32_t s = 0; s < steps; s++) {
     const uint32_t buf = s & 1u;
-    {  // second K half of this step
-      const uint32_t a1 = a_cur ^ 64u, b1 = b_cur ^ 64u;
-      MI355_READ_FRAGS(fa1, fb1, a1, b1);
-    }
-    mfma_block_bf16(acc, fa0, fb0);
+    const uint32_t a1 = a_cur ^ 64u, b1 = b_cur ^ 64u;   // second K half of this step
+    // ---- first half: MFMAs on F0, the reads of F1 slipped in between ---------------------------
+    MI355_DS_READ(fb1[0], b1, 0);     MI355_DS_READ(fb1[1], b1, 2048);
+    MI355_MFMA_ROW(acc, fa0, fb0, 0);
+    MI355_DS_READ(fb1[2], b1, 4096);  MI355_DS_READ(fb1[3], b1, 6144);
+    MI355_DS_READ(fa1[0], a1, 0);     MI355_DS_READ(fa1[1], a1, 2048);
+    MI355_MFMA_ROW(acc, fa0, fb0, 1);
+    MI355_DS_READ(fa1[2], a1, 4096);  MI355_DS_READ(fa1[3], a1, 6144);
+    MI355_MFMA_ROW(acc, fa0, fb0, 2);
+    MI355_DS_READ(fa1[4], a1, 8192);  MI355_DS_READ(fa1[5], a1, 10240);
+    MI355_MFMA_ROW(acc, fa0, fb0, 3);
+    MI355_DS_READ(fa1[6], a1, 12288); MI355_DS_READ(fa1[7], a1, 14336);
+    MI355_MFMA_ROW(acc, fa0, fb0, 4);
+    MI355_MFMA_ROW(acc, fa0, fb0, 5);
+    MI355_MFMA_ROW(acc, fa0, fb0, 6);
+    MI355_MFMA_ROW(acc, fa0, fb0, 7);
     MI355_WAIT_FRAGS(fa1, fb1);
     // every wave is done reading slab s; every wave's share of slab s+1 has landed
     asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-    if (s + 2 < steps) fetch_slab(s + 2, buf);
-    if (s + 1 < steps) { MI355_READ_FRAGS(fa0, fb0, a_nxt, b_nxt); }
-    mfma_block_bf16(acc, fa1, fb1);
+    // ---- second half: MFMAs on F1 first (they are ready), next F0 reads and the global loads
+    //      of slab s+2 spread between them so that no wave sits on the memory queues ------------
+    const bool more_reads = s + 1 < steps, more_loads = s + 2 < steps;
+    const uint32_t dst = dst_wave + buf * kBufBytes;
+    MI355_MFMA_ROW(acc, fa1, fb1, 0);
+    if (more_reads) { MI355_DS_READ(fb0[0], b_nxt, 0);    MI355_DS_READ(fb0[1], b_nxt, 2048);
+                      MI355_DS_READ(fb0[2], b_nxt, 4096); MI355_DS_READ(fb0[3], b_nxt, 6144); }
+    MI355_MFMA_ROW(acc, fa1, fb1, 1);
+    if (more_reads) { MI355_DS_READ(fa0[0], a_nxt, 0);    MI355_DS_READ(fa0[1], a_nxt, 2048);
+                      MI355_DS_READ(fa0[2], a_nxt, 4096); MI355_DS_READ(fa0[3], a_nxt, 6144); }
+    MI355_MFMA_ROW(acc, fa1, fb1, 2);
+    if (more_reads) { MI355_DS_READ(fa0[4], a_nxt, 8192);  MI355_DS_READ(fa0[5], a_nxt, 10240);
+                      MI355_DS_READ(fa0[6], a_nxt, 12288); MI355_DS_READ(fa0[7], a_nxt, 14336); }
+    MI355_MFMA_ROW(acc, fa1, fb1, 3);
+    if (more_loads) { load_to_lds(ga_next, dst);                  load_to_lds(gb_next, dst + kSlabBytes); }
+    MI355_MFMA_ROW(acc, fa1, fb1, 4);
+    if (more_loads) { load_to_lds(ga_next + row8, dst + 1024u);   load_to_lds(gb_next + row8, dst + kSlabBytes + 1024u); }
+    MI355_MFMA_ROW(acc, fa1, fb1, 5);
+    if (more_loads) { load_to_lds(ga_next + 2 * row8, dst + 2048u); load_to_lds(gb_next + 2 * row8, dst + kSlabBytes + 2048u); }
+    MI355_MFMA_ROW(acc, fa1, fb1, 6);
+    if (more_loads) { load_to_lds(ga_next + 3 * row8, dst + 3072u); load_to_lds(gb_next + 3 * row8, dst + kSlabBytes + 3072u); }
+    MI355_MFMA_ROW(acc, fa1, fb1, 7);
     MI355_WAIT_FRAGS(fa0, fb0);
+    ga_next += kRowBytes;
+    gb_next += kRowBytes;
     uint32_t t = a_cur; a_cur = a_nxt; a_nxt = t;
     t = b_cur; b_cur = b_nxt; b_nxt = t;
   }

@@ -95,6 +95,12 @@ int mi355_fill_bf16(mi355_dev *dev, uint16_t *dst, uint64_t n, uint64_t seed, ui
  * e4m3fn with saturation to +-448 (fp8 GEMM operands). */
 int mi355_fill_fp8_e4m3(mi355_dev *dev, uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist, float scale);
 
+/* Plain device-to-device copy kernel (16 bytes per lane, grid-stride).  No counterpart in
+ * the reference; it exists so that the HBM byte counters (FETCH_SIZE / WRITE_SIZE) can be
+ * calibrated against a transfer of known size.  bytes must be a multiple of 16 and both
+ * pointers 16-byte aligned. */
+int mi355_copy(mi355_dev *dev, void *dst, const void *src, size_t bytes);
+
 /* ---- global memory bandwidth -------------------------------------------------- */
 /* Takes over global_bandwidth_v1/v2/v4 (src/rocm/rocm_kernels/global_bandwidth.hip:10-67)
  * and their launch in runGlobalBandwidth (src/rocm/global_bandwidth.cpp:6-110).

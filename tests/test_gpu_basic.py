@@ -63,6 +63,17 @@ def test_fill_bf16_and_fp8_bit_exact(dev):
     b16.free(); b8.free()
 
 
+def test_copy_kernel(dev):
+    n = (1 << 20) + 16
+    src = dev.from_host(orc.fill_f32(n, SEED, 3, 0))
+    dst = dev.alloc(n * 4)
+    dev.copy(dst, src, n * 4)
+    assert np.array_equal(dst.download(np.float32, n), orc.fill_f32(n, SEED, 3, 0))
+    with pytest.raises(capi.Mi355Error):
+        dev.copy(dst, src, 10)
+    src.free(); dst.free()
+
+
 @pytest.mark.parametrize("width", [1, 2, 4])
 @pytest.mark.parametrize("n,blocks,bs", [
     (1 << 22, 64, 256),            # many full unrolled groups
