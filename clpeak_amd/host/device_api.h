@@ -1,0 +1,34 @@
+// The C ABI of libclpeak_mi355.so as a table of function pointers.  The backend class talks
+// to the GPU only through such a table: the real one binds the library's entry points, the
+// fake one (fake_device.cpp) stands in for a GPU so that the row set, ordering, gating and
+// file output can be exercised on a machine without one.
+#pragma once
+#include "../../include/clpeak_mi355.h"
+
+struct Mi355Api {
+  decltype(&mi355_device_count) device_count;
+  decltype(&mi355_open) open;
+  decltype(&mi355_close) close;
+  decltype(&mi355_get_props) get_props;
+  decltype(&mi355_last_error) last_error;
+  decltype(&mi355_alloc) alloc;
+  decltype(&mi355_free) free;
+  decltype(&mi355_upload) upload;
+  decltype(&mi355_download) download;
+  decltype(&mi355_sync) sync;
+  decltype(&mi355_timer_start) timer_start;
+  decltype(&mi355_timer_stop) timer_stop;
+  decltype(&mi355_fill_f32) fill_f32;
+  decltype(&mi355_fill_bf16) fill_bf16;
+  decltype(&mi355_fill_fp8_e4m3) fill_fp8_e4m3;
+  decltype(&mi355_global_bandwidth) global_bandwidth;
+  decltype(&mi355_compute_mad) compute_mad;
+  decltype(&mi355_launch_roundtrip) launch_roundtrip;
+  decltype(&mi355_mfma_dense) mfma_dense;
+  decltype(&mi355_smfmac) smfmac;
+  decltype(&mi355_gemm_bf16) gemm_bf16;
+  decltype(&mi355_gemm_fp8_e4m3) gemm_fp8_e4m3;
+};
+
+const Mi355Api &mi355_real_api();   // the entry points of libclpeak_mi355.so
+const Mi355Api &mi355_fake_api();   // one pretend gfx950 device, host memory, fixed timings

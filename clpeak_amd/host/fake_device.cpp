@@ -1,0 +1,81 @@
+// A pretend device behind the Mi355Api table: no GPU, no arithmetic.  Allocations are sizes
+// only (nothing is dereferenced), every launch "takes" a fixed time, and environment
+// variables can inject failures so that the backend's degrade paths can be tested:
+//   CLPEAK_FAKE_DEVICES=n          number of devices (default 1)
+//   CLPEAK_FAKE_FAIL=<entry>       that entry point fails (alloc, mfma_dense, gemm_bf16, ...)
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include "device_api.h"
+
+struct mi355_dev {
+  std::string error;
+  unsigned launches = 0;
+};
+
+namespace {
+bool fails(const char *what) {
+  const char *f = getenv("CLPEAK_FAKE_FAIL");
+  return f && strcmp(f, what) == 0;
+}
+int fail(mi355_dev *d, const char *what) {
+  d->error = std::string("fake device: injected failure in ") + what;
+  return MI355_ERR_HIP;
+}
+#define FAKE_ENTRY(dev, name) do { if (fails(name)) return fail(dev, name); (dev)->launches++; } while (0)
+
+int f_device_count(int *n) {
+  const char *e = getenv("CLPEAK_FAKE_DEVICES");
+  *n = e ? atoi(e) : 1;
+  return MI355_OK;
+}
+int f_open(int ordinal, mi355_dev **out) {
+  int n = 0;
+  f_device_count(&n);
+  if (ordinal < 0 || ordinal >= n) return MI355_ERR_NODEV;
+  *out = new mi355_dev();
+  return MI355_OK;
+}
+int f_close(mi355_dev *d) { delete d; return MI355_OK; }
+int f_get_props(mi355_dev *, mi355_props_t *p) {
+  memset(p, 0, sizeof(*p));
+  strcpy(p->name, "Fake MI355X");
+  strcpy(p->arch, "gfx950:sramecc+:xnack-");
+  strcpy(p->driver_version, "7.2.0");
+  strcpy(p->runtime_version, "7.2.26015");
+  p->num_cus = 256; p->wave_size = 64; p->max_threads_per_block = 1024; p->clock_khz = 2400000;
+  p->total_mem = 288ull << 30;
+  return MI355_OK;
+}
+const char *f_last_error(mi355_dev *d) { return d ? d->error.c_str() : "fake device: no such device"; }
+int f_alloc(mi355_dev *d, size_t bytes, void **p) {
+  FAKE_ENTRY(d, "alloc");
+  *p = (void *)(uintptr_t)(0x1000 + bytes % 4096 * 0);   // never dereferenced
+  *p = (void *)(uintptr_t)0x100000;
+  return MI355_OK;
+}
+int f_free(mi355_dev *, void *) { return MI355_OK; }
+int f_upload(mi355_dev *d, void *, const void *, size_t) { FAKE_ENTRY(d, "upload"); return MI355_OK; }
+int f_download(mi355_dev *d, void *dst, const void *, size_t n) { FAKE_ENTRY(d, "download"); memset(dst, 0, n); return MI355_OK; }
+int f_sync(mi355_dev *) { return MI355_OK; }
+int f_timer_start(mi355_dev *d) { d->launches = 0; return MI355_OK; }
+int f_timer_stop(mi355_dev *d, float *us) { *us = 100.0f * (float)(d->launches ? d->launches : 1); return MI355_OK; }
+int f_fill_f32(mi355_dev *d, float *, uint64_t, uint64_t, uint32_t, int) { FAKE_ENTRY(d, "fill_f32"); return MI355_OK; }
+int f_fill_bf16(mi355_dev *d, uint16_t *, uint64_t, uint64_t, uint32_t, int) { FAKE_ENTRY(d, "fill_bf16"); return MI355_OK; }
+int f_fill_fp8(mi355_dev *d, uint8_t *, uint64_t, uint64_t, uint32_t, int, float) { FAKE_ENTRY(d, "fill_fp8_e4m3"); return MI355_OK; }
+int f_global_bandwidth(mi355_dev *d, int, const float *, uint64_t, float *, uint32_t, uint32_t) { FAKE_ENTRY(d, "global_bandwidth"); return MI355_OK; }
+int f_compute_mad(mi355_dev *d, int, int, uint64_t, uint64_t, uint32_t, void *, uint32_t) { FAKE_ENTRY(d, "compute_mad"); return MI355_OK; }
+int f_launch_roundtrip(mi355_dev *d, uint32_t, uint32_t, double *us) { FAKE_ENTRY(d, "launch_roundtrip"); *us = 9.5; return MI355_OK; }
+int f_mfma_dense(mi355_dev *d, int, const void *, const void *, const uint8_t *, const uint8_t *, void *, uint32_t, uint32_t, uint64_t *) { FAKE_ENTRY(d, "mfma_dense"); return MI355_OK; }
+int f_smfmac(mi355_dev *d, int, const void *, const uint8_t *, const void *, void *, uint32_t, uint32_t, uint64_t *) { FAKE_ENTRY(d, "smfmac"); return MI355_OK; }
+int f_gemm_bf16(mi355_dev *d, const uint16_t *, const uint16_t *, uint16_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_bf16"); return MI355_OK; }
+int f_gemm_fp8(mi355_dev *d, const uint8_t *, const uint8_t *, uint16_t *, uint32_t, uint32_t, uint32_t, float, float) { FAKE_ENTRY(d, "gemm_fp8_e4m3"); return MI355_OK; }
+}  // namespace
+
+const Mi355Api &mi355_fake_api() {
+  static const Mi355Api api = {
+      f_device_count, f_open, f_close, f_get_props, f_last_error, f_alloc, f_free, f_upload, f_download, f_sync,
+      f_timer_start, f_timer_stop, f_fill_f32, f_fill_bf16, f_fill_fp8, f_global_bandwidth, f_compute_mad,
+      f_launch_roundtrip, f_mfma_dense, f_smfmac, f_gemm_bf16, f_gemm_fp8};
+  return api;
+}

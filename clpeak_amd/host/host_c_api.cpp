@@ -1,0 +1,33 @@
+// A few C entry points into the host layer so that tests can reach it with ctypes: the seeded
+// operand generator, pickIters, and a whole run against the stand-in device.
+#include <cstring>
+#include <sstream>
+#include "mi355_peak.h"
+#include "seeded_inputs.h"
+
+extern "C" {
+
+unsigned clpeak_host_pick_iters(double per_iter_us, unsigned target_us, unsigned forced, unsigned max_iters) {
+  return pickIters(per_iter_us, target_us, forced, max_iters);
+}
+
+unsigned long long clpeak_host_target_global_threads(unsigned num_cus) { return targetGlobalThreads(num_cus); }
+
+// fmt: 0 f16, 1 bf16, 2 e4m3, 3 e5m2, 4 e2m3, 5 e3m2, 6 e2m1, 7 int8.  Returns the number of bytes written.
+size_t clpeak_host_seeded_operand(int fmt, double sigma, unsigned long long seed, unsigned stream, unsigned long long n,
+                                  unsigned char *out, size_t cap) {
+  const std::vector<uint8_t> v = seeded_operand((OperandFormat)fmt, sigma, seed, stream, n);
+  if (v.size() > cap) return 0;
+  memcpy(out, v.data(), v.size());
+  return v.size();
+}
+
+size_t clpeak_host_seeded_bytes(int what, unsigned long long seed, unsigned stream, unsigned long long n, unsigned char *out) {
+  const std::vector<uint8_t> v = what == 0 ? seeded_e8m0(seed, stream, n) : seeded_sparse_meta(seed, stream, n);
+  memcpy(out, v.data(), v.size());
+  return v.size();
+}
+
+void clpeak_host_request_cancel(void) { clpeak::requestCancel(); }
+void clpeak_host_reset_cancel(void) { clpeak::resetCancel(); }
+}

@@ -1,0 +1,456 @@
+#include "mi355_peak.h"
+#include <algorithm>
+#include <cstdio>
+#include <ostream>
+#include "../csrc/seeded_rng.h"
+#include "seeded_inputs.h"
+
+// ---- small helpers ----------------------------------------------------------------------------
+struct Mi355Peak::Buffer {
+  const Mi355Api &api;
+  mi355_dev *dev;
+  void *ptr = nullptr;
+  Buffer(const Mi355Api &a, mi355_dev *d, size_t bytes) : api(a), dev(d) {
+    if (api.alloc(dev, bytes, &ptr) != MI355_OK) ptr = nullptr;
+  }
+  ~Buffer() { if (ptr) api.free(dev, ptr); }
+  Buffer(const Buffer &) = delete;
+  Buffer &operator=(const Buffer &) = delete;
+  explicit operator bool() const { return ptr != nullptr; }
+  bool upload(const std::vector<uint8_t> &host) { return ptr && api.upload(dev, ptr, host.data(), host.size()) == MI355_OK; }
+};
+
+static const char *widthNote(int width) {
+  switch (width) {
+    case 1: return "One value per lane at a time.";
+    case 2: return "The 16 accumulators of a work-item grouped as 2-wide vectors.";
+    case 4: return "The 16 accumulators of a work-item grouped as 4-wide vectors.";
+    default: return "";
+  }
+}
+
+Mi355Peak::Mi355Peak(const Mi355Api &api) : api_(api) {}
+
+void Mi355Peak::applyOptions(const CliOptions &opts) {
+  Peak::applyOptions(opts);
+  deviceIndices = opts.rocmDeviceIndices;
+}
+
+int Mi355Peak::listDevices(const Mi355Api &api, std::ostream &os) {
+  int n = 0;
+  if (api.device_count(&n) != MI355_OK) return -1;
+  for (int i = 0; i < n; i++) {
+    mi355_dev *d = nullptr;
+    if (api.open(i, &d) != MI355_OK) {
+      os << "ROCm device " << i << ": not usable by this backend (" << api.last_error(nullptr) << ")\n";
+      continue;
+    }
+    mi355_props_t p;
+    api.get_props(d, &p);
+    os << "ROCm device " << i << ": " << p.name << " (" << p.arch << ", " << p.num_cus << " CUs, "
+       << (p.total_mem >> 20) << " MB)\n";
+    api.close(d);
+  }
+  return n;
+}
+
+float Mi355Peak::runKernel(const std::function<int()> &launch, unsigned targetUs, unsigned forcedIters) {
+  for (unsigned w = 0; w < warmupCount; w++)
+    if (launch() != MI355_OK || api_.sync(dev_) != MI355_OK) return -1.0f;
+  auto batch = [&](unsigned n) -> float {
+    if (api_.timer_start(dev_) != MI355_OK) return -1.0f;
+    for (unsigned i = 0; i < n; i++)
+      if (launch() != MI355_OK) {
+        if (clpeak::verboseEnabled()) fprintf(stderr, "launch failed: %s\n", api_.last_error(dev_));
+        return -1.0f;
+      }
+    float us = 0.0f;
+    if (api_.timer_stop(dev_, &us) != MI355_OK) return -1.0f;
+    return us;
+  };
+  const float probe = batch(1);
+  if (probe <= 0.0f) return -1.0f;
+  const unsigned iters = pickIters(probe, targetUs, forcedIters);
+  const float total = batch(iters);
+  return total > 0.0f ? total / (float)iters : -1.0f;
+}
+
+// ---- run order ------------------------------------------------------------------------------------
+int Mi355Peak::runAll() {
+  int count = 0;
+  if (api_.device_count(&count) != MI355_OK) {
+    log->note("ROCm: runtime init failed\n");
+    return -1;
+  }
+  if (count == 0) {
+    log->note("ROCm: no devices found\n");
+    return 0;
+  }
+  auto backend = log->beginBackend("ROCm");
+  for (int i = 0; i < count; i++) {
+    if (clpeak::cancelRequested()) break;
+    if (!deviceIndices.empty() && std::find(deviceIndices.begin(), deviceIndices.end(), i) == deviceIndices.end()) continue;
+    runDevice(i, backend);
+  }
+  return 0;
+}
+
+struct MadTest {
+  Benchmark bench;
+  const char *tag, *display, *unit, *description;
+  int kind, elemBytes;
+  int opsPerStep;   // operations one accumulator step counts for
+  struct Variant { const char *metric; int width; const char *note; } variants[4];
+};
+
+void Mi355Peak::runDevice(int ordinal, logger::BackendScope &backend) {
+  if (api_.open(ordinal, &dev_) != MI355_OK) {
+    log->note("ROCm: failed to init device " + std::to_string(ordinal) + ": " + api_.last_error(nullptr) + "\n");
+    dev_ = nullptr;
+    return;
+  }
+  api_.get_props(dev_, &props_);
+  benchmark_config_t cfg = benchmark_config_t::forDevice(DeviceType::Gpu);
+  cfg.targetTimeUs = targetTimeUs;
+  cfg.kernelLatencyIters = forceIters ? specifiedIters : workload.latencyLaunches;
+
+  auto device = backend.beginDevice({props_.name, "", props_.driver_version,
+                                     {{"Arch", props_.arch},
+                                      {"HIP", props_.runtime_version},
+                                      {"CUs", std::to_string(props_.num_cus)},
+                                      {"Wave", std::to_string(props_.wave_size)},
+                                      {"VRAM", std::to_string(props_.total_mem / (1024 * 1024)) + " MB"}},
+                                     -1, ordinal});
+  device_ = &device;
+
+  static const MadTest sp = {Benchmark::ComputeSP, "single_precision_compute", "Single-precision compute", "gflops",
+      "Vector-ALU rate on 32-bit floats: 2^20 work-items, each advancing 16 independent fused multiply-add chains, "
+      "nothing but registers involved.", MI355_MAD_F32, 4, 2,
+      {{"float", 1, widthNote(1)}, {"float2", 2, widthNote(2)}, {"float4", 4, widthNote(4)}, {nullptr, 0, nullptr}}};
+  static const MadTest hp = {Benchmark::ComputeHP, "half_precision_compute", "Half-precision compute", "gflops",
+      "The same chains in IEEE half precision; the packed form does two lanes per instruction.", MI355_MAD_F16, 2, 2,
+      {{"half", 1, "Scalar half FMA."}, {"half2", 2, "Packed half2 FMA."}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
+  static const MadTest dp = {Benchmark::ComputeDP, "double_precision_compute", "Double-precision compute", "gflops",
+      "The same chains on 64-bit floats.", MI355_MAD_F64, 8, 2,
+      {{"double", 1, widthNote(1)}, {"double2", 2, widthNote(2)}, {"double4", 4, widthNote(4)}, {nullptr, 0, nullptr}}};
+  static const MadTest mp = {Benchmark::ComputeMP, "mixed_precision_compute", "Mixed-precision compute fp16xfp16+fp32", "gflops",
+      "Half-precision operands multiplied into a 32-bit running total.", MI355_MAD_MP, 4, 2,
+      {{"mp", 1, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
+  static const MadTest bf = {Benchmark::ComputeBF16, "bfloat16_compute", "BF16 compute bf16xbf16+fp32", "gflops",
+      "bfloat16 operands multiplied into a 32-bit running total.", MI355_MAD_BF16, 4, 2,
+      {{"bf16", 1, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
+  static const MadTest i32 = {Benchmark::ComputeInt, "integer_compute", "Integer compute (32-bit IMAD)", "gops",
+      "The same chains on 32-bit integers (multiply-add, wrapping).", MI355_MAD_I32, 4, 2,
+      {{"int", 1, widthNote(1)}, {"int2", 2, widthNote(2)}, {"int4", 4, widthNote(4)}, {nullptr, 0, nullptr}}};
+  static const MadTest i8 = {Benchmark::ComputeInt8DP, "integer_compute_int8_dp", "INT8 dot-product compute (DP4a)", "gops",
+      "Four 8-bit multiply-adds per instruction, each result fed back into the next operand.", MI355_MAD_I8DP, 4, 8,
+      {{"int8_dp", 1, "One dependent chain."}, {"int8_dp2", 2, "Two independent chains."},
+       {"int8_dp4", 4, "Four independent chains."}, {"int8_dp8", 8, "Eight independent chains."}}};
+
+  // fp phase
+  if (isAllowed(Benchmark::ComputeSP)) runComputeMad(sp);
+  if (isAllowed(Benchmark::ComputeHP)) runComputeMad(hp);
+  if (isAllowed(Benchmark::ComputeDP)) runComputeMad(dp);
+  if (isAllowed(Benchmark::ComputeMP)) runComputeMad(mp);
+  if (isAllowed(Benchmark::ComputeBF16)) runComputeMad(bf);
+  if (isAllowedAs(Benchmark::Wmma, Category::FpCompute)) runUnsupportedMatrixRows(Category::FpCompute, true);
+  if (isAllowedAs(Benchmark::Rocwmma, Category::FpCompute)) runUnsupportedMatrixRows(Category::FpCompute, false);
+  if (isAllowedAs(Benchmark::Mfma, Category::FpCompute)) runMfma(Category::FpCompute);
+  if (isAllowedAs(Benchmark::Mfma, Category::FpCompute)) runSparseMfma(Category::FpCompute);
+  if (isAllowedAs(Benchmark::Rocblas, Category::FpCompute)) runGemmFp();
+  if (isAllowedAs(Benchmark::Rocblas, Category::FpCompute)) runGemmFp8();
+  // int phase
+  if (isAllowed(Benchmark::ComputeInt)) runComputeMad(i32);
+  if (isAllowed(Benchmark::ComputeInt8DP)) runComputeMad(i8);
+  if (isAllowedAs(Benchmark::Wmma, Category::IntCompute)) runUnsupportedMatrixRows(Category::IntCompute, true);
+  if (isAllowedAs(Benchmark::Rocwmma, Category::IntCompute)) runUnsupportedMatrixRows(Category::IntCompute, false);
+  if (isAllowedAs(Benchmark::Mfma, Category::IntCompute)) runMfma(Category::IntCompute);
+  if (isAllowedAs(Benchmark::Mfma, Category::IntCompute)) runSparseMfma(Category::IntCompute);
+  if (isAllowedAs(Benchmark::Rocblas, Category::IntCompute)) runGemmInt();
+  // bandwidth and latency
+  if (isAllowed(Benchmark::GlobalBW)) runGlobalBandwidth();
+  if (isAllowed(Benchmark::LocalBW))
+    runNotBuilt("local_memory_bandwidth", "Local memory bandwidth", {"float", "float2", "float4"},
+                "Not built in the MI355X backend yet", ResultStatus::Skipped);
+  if (isAllowed(Benchmark::ImageBW))
+    runNotBuilt("image_memory_bandwidth", "Image memory bandwidth", {"float4"},
+                "Device has no image/texture support", ResultStatus::Unsupported);
+  if (isAllowed(Benchmark::TransferBW))
+    runNotBuilt("transfer_bandwidth", "Transfer bandwidth", {"h2d_pinned", "d2h_pinned"},
+                "Not built in the MI355X backend yet", ResultStatus::Skipped);
+  if (isAllowed(Benchmark::KernelLatency)) runKernelLatency(cfg);
+
+  device_ = nullptr;
+  device.end();
+  api_.close(dev_);
+  dev_ = nullptr;
+}
+
+// ---- vector MAD -----------------------------------------------------------------------------------------
+void Mi355Peak::runComputeMad(const MadTest &t) {
+  auto test = device_->beginTest({t.tag, t.display, t.unit, Category::Unknown, t.description});
+  Buffer out(api_, dev_, workload.madItems * (size_t)t.elemBytes);
+  for (const auto &v : t.variants) {
+    if (!v.metric) break;
+    const std::string note = v.note ? v.note : "";
+    if (!out) {
+      test.skip(v.metric, ResultStatus::Error, "Failed to allocate output buffer", note);
+      continue;
+    }
+    const float us = runKernel(
+        [&] { return api_.compute_mad(dev_, t.kind, v.width, workload.seed, workload.madItems, workload.madSteps, out.ptr, 256); },
+        targetTimeUs, forceIters ? specifiedIters : 0);
+    if (us <= 0.0f) {
+      test.skip(v.metric, ResultStatus::Error, "kernel launch failed", note);
+      continue;
+    }
+    // 16 accumulators per item (or `width` chains for the dot-product test)
+    const double chains = t.kind == MI355_MAD_I8DP ? (double)v.width : 16.0;
+    const double ops = (double)workload.madItems * chains * (double)workload.madSteps * (double)t.opsPerStep;
+    test.emit(v.metric, (float)(ops * 1e6 / us / 1e9), {false, note});
+  }
+}
+
+// ---- rows that exist only on other AMD families ----------------------------------------------------------------
+void Mi355Peak::runUnsupportedMatrixRows(Category phase, bool wmma) {
+  struct Row { const char *tag, *display, *unit; };
+  static const Row wmmaFp[] = {{"wmma_fp16", "WMMA fp16xfp16+fp32 16x16x16", "tflops"},
+                               {"wmma_bf16", "WMMA bf16xbf16+fp32 16x16x16", "tflops"},
+                               {"wmma_fp8_e4m3", "WMMA fp8(E4M3)xfp8(E4M3)+fp32 16x16x16", "tflops"},
+                               {"wmma_fp8_e5m2", "WMMA fp8(E5M2)xfp8(E5M2)+fp32 16x16x16", "tflops"}};
+  static const Row wmmaInt[] = {{"wmma_int8", "WMMA int8xint8+int32 16x16x16", "tops"}};
+  const bool isInt = phase == Category::IntCompute;
+  if (wmma) {
+    const Row *rows = isInt ? wmmaInt : wmmaFp;
+    const size_t n = isInt ? 1 : 4;
+    for (size_t i = 0; i < n; i++) {
+      auto test = device_->beginTest({rows[i].tag, rows[i].display, rows[i].unit, Category::Unknown, ""});
+      test.skip(rows[i].tag, ResultStatus::Unsupported,
+                "WMMA is an RDNA3+/RDNA4 (gfx11/gfx12) matrix-core feature; absent on this architecture");
+    }
+  } else {
+    auto test = isInt ? device_->beginTest({"rocwmma-int", "rocWMMA int8xint8+int32 16x16x16", "tops", Category::Unknown, ""})
+                      : device_->beginTest({"rocwmma-fp", "rocWMMA fp16xfp16+fp32 16x16x16", "tflops", Category::Unknown, ""});
+    test.skip(isInt ? "rocwmma_int8" : "rocwmma_fp16", ResultStatus::Unsupported,
+              "rocWMMA does not support this GPU architecture");
+  }
+}
+
+// ---- dense MFMA ----------------------------------------------------------------------------------------------
+namespace {
+struct MfmaRow {
+  const char *tag, *display, *unit, *description;
+  int kind, M, N, K;
+  OperandFormat fmt;
+  double sigma;
+  bool scaled;
+};
+const MfmaRow kMfmaFp[] = {
+    {"mfma_fp16", "MFMA fp16xfp16+fp32 16x16x32", "tflops", "Matrix-core rate on half-precision inputs with a 32-bit accumulator.",
+     MI355_MFMA_F16_16x16x32, 16, 16, 32, OperandFormat::F16, 0.01, false},
+    {"mfma_fp16_32x32x16", "MFMA fp16xfp16+fp32 32x32x16", "tflops", "The same on the 32x32 tile shape.",
+     MI355_MFMA_F16_32x32x16, 32, 32, 16, OperandFormat::F16, 0.01, false},
+    {"mfma_bf16", "MFMA bf16xbf16+fp32 16x16x32", "tflops", "Matrix-core rate on bfloat16 inputs with a 32-bit accumulator.",
+     MI355_MFMA_BF16_16x16x32, 16, 16, 32, OperandFormat::BF16, 0.01, false},
+    {"mfma_bf16_32x32x16", "MFMA bf16xbf16+fp32 32x32x16", "tflops", "The same on the 32x32 tile shape.",
+     MI355_MFMA_BF16_32x32x16, 32, 32, 16, OperandFormat::BF16, 0.01, false},
+    {"mfma_fp8", "MFMA fp8xfp8+fp32 16x16x128", "tflops", "Matrix-core rate on OCP fp8 (E4M3) inputs.",
+     MI355_MFMA_FP8_16x16x128, 16, 16, 128, OperandFormat::E4M3, 1.0, false},
+    {"mfma_bf8", "MFMA bf8xbf8+fp32 16x16x128", "tflops", "Matrix-core rate on OCP fp8 (E5M2) inputs.",
+     MI355_MFMA_BF8_16x16x128, 16, 16, 128, OperandFormat::E5M2, 1.0, false},
+    {"mfma_mxfp6_e2m3", "MFMA mxfp6(e2m3)+fp32 16x16x128", "tflops", "6-bit MX inputs with one E8M0 scale per 32 elements.",
+     MI355_MFMA_MXFP6_E2M3, 16, 16, 128, OperandFormat::E2M3, 1.0, true},
+    {"mfma_mxfp6_e3m2", "MFMA mxfp6(e3m2)+fp32 16x16x128", "tflops", "6-bit MX inputs, the wider-range variant.",
+     MI355_MFMA_MXFP6_E3M2, 16, 16, 128, OperandFormat::E3M2, 1.0, true},
+    {"mfma_mxfp4", "MFMA mxfp4(e2m1)+fp32 16x16x128", "tflops", "4-bit MX inputs with one E8M0 scale per 32 elements.",
+     MI355_MFMA_MXFP4_E2M1, 16, 16, 128, OperandFormat::E2M1, 1.0, true},
+};
+const MfmaRow kMfmaInt[] = {
+    {"mfma_int8", "MFMA int8xint8+int32 16x16x64", "tops", "Matrix-core rate on 8-bit integers with a 32-bit accumulator.",
+     MI355_MFMA_I8_16x16x64, 16, 16, 64, OperandFormat::I8, 0.0, false},
+};
+struct SparseRow {
+  const char *tag, *display, *unit, *description;
+  int kind, K;
+  OperandFormat fmt;
+  double sigma;
+};
+const SparseRow kSparseFp[] = {
+    {"smfmac_fp16", "Sparse MFMA fp16 2:4 16x16x64 (TFLOPS)", "tflops", "2:4 structured-sparse matrix-core rate, half-precision inputs.",
+     MI355_SMFMAC_F16_16x16x64, 64, OperandFormat::F16, 0.01},
+    {"smfmac_bf16", "Sparse MFMA bf16 2:4 16x16x64 (TFLOPS)", "tflops", "2:4 structured-sparse matrix-core rate, bfloat16 inputs.",
+     MI355_SMFMAC_BF16_16x16x64, 64, OperandFormat::BF16, 0.01},
+    {"smfmac_fp8", "Sparse MFMA fp8 2:4 16x16x128 (TFLOPS)", "tflops", "2:4 structured-sparse matrix-core rate, fp8 (E4M3) inputs.",
+     MI355_SMFMAC_FP8_16x16x128, 128, OperandFormat::E4M3, 1.0},
+    {"smfmac_bf8", "Sparse MFMA bf8 2:4 16x16x128 (TFLOPS)", "tflops", "2:4 structured-sparse matrix-core rate, fp8 (E5M2) inputs.",
+     MI355_SMFMAC_BF8_16x16x128, 128, OperandFormat::E5M2, 1.0},
+};
+const SparseRow kSparseInt[] = {
+    {"smfmac_int8", "Sparse MFMA int8 2:4 16x16x128 (TOPS)", "tops", "2:4 structured-sparse matrix-core rate, 8-bit integers.",
+     MI355_SMFMAC_I8_16x16x128, 128, OperandFormat::I8, 0.0},
+};
+}  // namespace
+
+void Mi355Peak::runMfma(Category phase) {
+  const bool isInt = phase == Category::IntCompute;
+  const MfmaRow *rows = isInt ? kMfmaInt : kMfmaFp;
+  const size_t n = isInt ? sizeof(kMfmaInt) / sizeof(kMfmaInt[0]) : sizeof(kMfmaFp) / sizeof(kMfmaFp[0]);
+  const uint32_t waves = (uint32_t)props_.num_cus * workload.mfmaWavesPerCU;
+  const uint64_t units = (uint64_t)waves * 4;
+  for (size_t r = 0; r < n; r++) {
+    const MfmaRow &m = rows[r];
+    auto test = device_->beginTest({m.tag, m.display, m.unit, Category::Unknown, m.description});
+    const std::vector<uint8_t> A = seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_A, units * m.M * m.K);
+    const std::vector<uint8_t> B = seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_B, units * m.N * m.K);
+    Buffer dA(api_, dev_, A.size()), dB(api_, dev_, B.size()), out(api_, dev_, units * m.M * m.N * 4);
+    Buffer sA(api_, dev_, m.scaled ? units * m.M * (m.K / 32) : 16), sB(api_, dev_, m.scaled ? units * m.N * (m.K / 32) : 16);
+    bool ok = dA && dB && out && sA && sB && dA.upload(A) && dB.upload(B);
+    if (ok && m.scaled)
+      ok = sA.upload(seeded_e8m0(workload.seed, MI355_STREAM_SCALE_A, units * m.M * (m.K / 32))) &&
+           sB.upload(seeded_e8m0(workload.seed, MI355_STREAM_SCALE_B, units * m.N * (m.K / 32)));
+    if (!ok) {
+      test.skip(m.tag, ResultStatus::Error, "Failed to allocate or upload operand buffers");
+      continue;
+    }
+    const float us = runKernel(
+        [&] {
+          return api_.mfma_dense(dev_, m.kind, dA.ptr, dB.ptr, m.scaled ? (const uint8_t *)sA.ptr : nullptr,
+                                 m.scaled ? (const uint8_t *)sB.ptr : nullptr, out.ptr, waves, workload.mfmaIters, nullptr);
+        },
+        targetTimeUs, forceIters ? specifiedIters : 0);
+    if (us <= 0.0f) {
+      test.skip(m.tag, ResultStatus::Error, "kernel launch failed");
+      continue;
+    }
+    // every wave issues 4 * iters instructions of 2*M*N*K operations
+    const double ops = (double)units * workload.mfmaIters * 2.0 * m.M * m.N * m.K;
+    test.emit(m.tag, (float)(ops * 1e6 / us / 1e12));
+  }
+}
+
+void Mi355Peak::runSparseMfma(Category phase) {
+  const bool isInt = phase == Category::IntCompute;
+  const SparseRow *rows = isInt ? kSparseInt : kSparseFp;
+  const size_t n = isInt ? sizeof(kSparseInt) / sizeof(kSparseInt[0]) : sizeof(kSparseFp) / sizeof(kSparseFp[0]);
+  const uint32_t waves = (uint32_t)props_.num_cus * workload.mfmaWavesPerCU;
+  const uint64_t units = (uint64_t)waves * 4;
+  for (size_t r = 0; r < n; r++) {
+    const SparseRow &m = rows[r];
+    auto test = device_->beginTest({m.tag, m.display, m.unit, Category::Unknown, m.description});
+    const std::vector<uint8_t> Ac = seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_A, units * 16 * (m.K / 2));
+    const std::vector<uint8_t> B = seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_B, units * 16 * m.K);
+    const std::vector<uint8_t> meta = seeded_sparse_meta(workload.seed, MI355_STREAM_SPARSE, units * 16 * (m.K / 4));
+    Buffer dA(api_, dev_, Ac.size()), dB(api_, dev_, B.size()), dM(api_, dev_, meta.size()), out(api_, dev_, units * 256 * 4);
+    if (!(dA && dB && dM && out && dA.upload(Ac) && dB.upload(B) && dM.upload(meta))) {
+      test.skip(m.tag, ResultStatus::Error, "Failed to allocate or upload operand buffers");
+      continue;
+    }
+    const float us = runKernel(
+        [&] { return api_.smfmac(dev_, m.kind, dA.ptr, (const uint8_t *)dM.ptr, dB.ptr, out.ptr, waves, workload.mfmaIters, nullptr); },
+        targetTimeUs, forceIters ? specifiedIters : 0);
+    if (us <= 0.0f) {
+      test.skip(m.tag, ResultStatus::Error, "kernel launch failed");
+      continue;
+    }
+    // counted with the dense-equivalent K, as the datasheet's sparse column is
+    const double ops = (double)units * workload.mfmaIters * 2.0 * 16 * 16 * m.K;
+    test.emit(m.tag, (float)(ops * 1e6 / us / 1e12));
+  }
+}
+
+// ---- GEMM (the slots of the vendor-library tests) ------------------------------------------------------------------
+void Mi355Peak::runGemmFp() {
+  auto test = device_->beginTest({"rocblas-fp", "rocBLAS GEMM peak", "tflops", Category::Unknown,
+                                  "Square GEMM.  The bf16 row is this backend's hand-written MFMA kernel "
+                                  "(LDS double-buffered 256x256x64 tiles), not a vendor library."});
+  const char *notBuilt = "No hand-written kernel for this type in the MI355X backend (no vendor BLAS is used)";
+  test.skip("fp32", ResultStatus::Unsupported, notBuilt);
+  test.skip("fp64", ResultStatus::Unsupported, notBuilt);
+  test.skip("fp16", ResultStatus::Unsupported, notBuilt);
+  const uint32_t D = workload.gemmDim;
+  Buffer A(api_, dev_, (size_t)D * D * 2), B(api_, dev_, (size_t)D * D * 2), C(api_, dev_, (size_t)D * D * 2);
+  const bool ok = A && B && C &&
+                  api_.fill_bf16(dev_, (uint16_t *)A.ptr, (uint64_t)D * D, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1) == MI355_OK &&
+                  api_.fill_bf16(dev_, (uint16_t *)B.ptr, (uint64_t)D * D, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1) == MI355_OK;
+  if (!ok) {
+    test.skip("bf16", ResultStatus::Error, "Failed to allocate or fill GEMM buffers");
+    return;
+  }
+  const float us = runKernel([&] { return api_.gemm_bf16(dev_, (const uint16_t *)A.ptr, (const uint16_t *)B.ptr, (uint16_t *)C.ptr, D, D, D); },
+                             targetTimeUs, forceIters ? specifiedIters : 0);
+  if (us <= 0.0f) test.skip("bf16", ResultStatus::Error, "kernel launch failed");
+  else test.emit("bf16", (float)(2.0 * D * D * D * 1e6 / us / 1e12), "bf16 inputs, fp32 accumulation, bf16 output; A row-major, B column-major.");
+}
+
+void Mi355Peak::runGemmFp8() {
+  auto test = device_->beginTest({"hipblaslt-fp8", "hipBLASLt FP8 GEMM peak", "tflops", Category::Unknown,
+                                  "Square FP8 GEMM with per-tensor scales.  The e4m3 row is this backend's hand-written "
+                                  "MFMA kernel, not a vendor library."});
+  const uint32_t D = workload.gemmDim;
+  const float scale = 448.0f;   // uniform [-1,1) stretched over the e4m3 range
+  {
+    Buffer A(api_, dev_, (size_t)D * D), B(api_, dev_, (size_t)D * D), C(api_, dev_, (size_t)D * D * 2);
+    const bool ok = A && B && C &&
+                    api_.fill_fp8_e4m3(dev_, (uint8_t *)A.ptr, (uint64_t)D * D, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1, scale) == MI355_OK &&
+                    api_.fill_fp8_e4m3(dev_, (uint8_t *)B.ptr, (uint64_t)D * D, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1, scale) == MI355_OK;
+    float us = -1.0f;
+    if (ok)
+      us = runKernel([&] { return api_.gemm_fp8_e4m3(dev_, (const uint8_t *)A.ptr, (const uint8_t *)B.ptr, (uint16_t *)C.ptr, D, D, D, 1.0f / scale, 1.0f / scale); },
+                     targetTimeUs, forceIters ? specifiedIters : 0);
+    if (!ok) test.skip("fp8_e4m3", ResultStatus::Error, "Failed to allocate or fill GEMM buffers");
+    else if (us <= 0.0f) test.skip("fp8_e4m3", ResultStatus::Error, "kernel launch failed");
+    else test.emit("fp8_e4m3", (float)(2.0 * D * D * D * 1e6 / us / 1e12), "OCP e4m3 inputs, per-tensor fp32 scales, fp32 accumulation, bf16 output.");
+  }
+  const char *notBuilt = "No hand-written kernel for this type in the MI355X backend (no vendor BLAS is used)";
+  test.skip("fp8_e5m2", ResultStatus::Unsupported, notBuilt);
+  test.skip("mxf4_e2m1", ResultStatus::Unsupported, notBuilt);
+}
+
+void Mi355Peak::runGemmInt() {
+  auto test = device_->beginTest({"rocblas-int", "rocBLAS GEMM peak", "tops", Category::Unknown, ""});
+  test.skip("int8", ResultStatus::Unsupported, "No hand-written kernel for this type in the MI355X backend (no vendor BLAS is used)");
+}
+
+// ---- bandwidth, latency ---------------------------------------------------------------------------------------------
+void Mi355Peak::runGlobalBandwidth() {
+  auto test = device_->beginTest({"global_memory_bandwidth", "Global memory bandwidth", "gbps", Category::Unknown,
+                                  "Streaming read of a buffer far larger than every cache; each reading fetches a "
+                                  "different number of floats per load instruction."});
+  static const struct { const char *metric; int width; } variants[] = {{"float", 1}, {"float2", 2}, {"float4", 4}};
+  uint64_t n = workload.bwFloats;
+  const uint64_t cap = props_.total_mem / 4 / sizeof(float);   // never more than a quarter of VRAM
+  if (n > cap) n = cap & ~3ull;
+  const uint32_t blocks = (uint32_t)props_.num_cus * workload.bwBlocksPerCU, bs = 256;
+  Buffer in(api_, dev_, n * sizeof(float)), out(api_, dev_, (size_t)blocks * bs * sizeof(float));
+  const bool ok = in && out && api_.fill_f32(dev_, (float *)in.ptr, n, workload.seed, MI355_STREAM_BW, MI355_DIST_U01) == MI355_OK;
+  for (const auto &v : variants) {
+    if (!ok) {
+      test.skip(v.metric, ResultStatus::Error, "Failed to allocate buffers", widthNote(v.width));
+      continue;
+    }
+    const float us = runKernel([&] { return api_.global_bandwidth(dev_, v.width, (const float *)in.ptr, n, (float *)out.ptr, blocks, bs); },
+                               targetTimeUs, forceIters ? specifiedIters : 0);
+    if (us <= 0.0f) test.skip(v.metric, ResultStatus::Error, "kernel launch failed", widthNote(v.width));
+    else test.emit(v.metric, (float)((double)n * sizeof(float) / us / 1e3), widthNote(v.width));
+  }
+}
+
+void Mi355Peak::runNotBuilt(const char *tag, const char *display, std::initializer_list<std::string> metrics, const char *why,
+                            ResultStatus status) {
+  auto test = device_->beginTest({tag, display, "gbps", Category::Unknown, ""});
+  test.skipAll(metrics, status, why);
+}
+
+void Mi355Peak::runKernelLatency(const benchmark_config_t &cfg) {
+  auto test = device_->beginTest({"kernel_launch_latency", "Kernel launch latency", "us", Category::Unknown,
+                                  "What it costs to ask the GPU to do anything: an empty kernel, launched and waited for."});
+  const char *dispatchNote = "Submit to start of execution; the host and the GPU share no clock through HIP.";
+  const char *roundtripNote = "Submit, run, hear back: the mean wall-clock time of launch plus stream synchronisation.";
+  test.skip("dispatch", ResultStatus::Unsupported, "Not measurable via HIP runtime/module API", dispatchNote);
+  double us = 0.0;
+  const unsigned n = cfg.kernelLatencyIters ? cfg.kernelLatencyIters : 1000;
+  if (api_.launch_roundtrip(dev_, warmupCount, n, &us) != MI355_OK)
+    test.skip("roundtrip", ResultStatus::Error, "launch/synchronize failed", roundtripNote);
+  else
+    test.emit("roundtrip", (float)us, roundtripNote);
+}

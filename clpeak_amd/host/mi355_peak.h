@@ -1,0 +1,61 @@
+// The MI355X backend behind clpeak's Peak interface.
+//
+// Takes the place of the reference's RocmPeak (include/rocm/rocm_peak.h:119-169,
+// src/rocm/rocm_peak.cpp:117-229): same backend name ("ROCm"), same device properties, same
+// test tags / metric names / units in the same order, the same degrade-to-a-skip-row error
+// handling -- but every measured row runs a hand-written gfx950 kernel on seeded inputs
+// through the C ABI in include/clpeak_mi355.h, never HIP directly.
+#pragma once
+#include <functional>
+#include <vector>
+#include "device_api.h"
+#include "peak.h"
+
+class Mi355Peak : public Peak {
+ public:
+  std::vector<int> deviceIndices;   // empty = run every device
+
+  explicit Mi355Peak(const Mi355Api &api = mi355_real_api());
+  void applyOptions(const CliOptions &opts) override;
+  int runAll() override;
+
+  // One line per device: "ROCm device <i>: <name> (<arch>, <CUs> CUs, <VRAM> MB)".
+  static int listDevices(const Mi355Api &api, std::ostream &os);
+
+  // Shapes of the seeded workloads.  Defaults are the configured ones; tests shrink them.
+  struct Workload {
+    uint64_t seed = 0x5EEDC1BEA4D355ull;
+    uint64_t madItems = 1ull << 20;       // work-items of the MAD tests
+    uint32_t madSteps = 4096;             // dependent steps per accumulator
+    uint64_t bwFloats = 1ull << 30;       // 4 GiB bandwidth buffer
+    uint32_t bwBlocksPerCU = 1;           // 256-thread workgroups per CU
+    uint32_t mfmaWavesPerCU = 8;          // 2048 waves on 256 CUs
+    uint32_t mfmaIters = 4096;
+    uint32_t gemmDim = 8192;
+    uint32_t latencyLaunches = 10000;
+  } workload;
+
+ private:
+  const Mi355Api &api_;
+  mi355_dev *dev_ = nullptr;
+  mi355_props_t props_{};
+  logger::DeviceScope *device_ = nullptr;
+
+  // RocmPeak::runKernel (src/rocm/rocm_peak.cpp:51-115): warm-ups, one-launch probe, pickIters,
+  // timed batch between two events; microseconds per launch, or -1 on any failure.
+  float runKernel(const std::function<int()> &launch, unsigned targetTimeUs, unsigned forcedIters);
+
+  struct Buffer;   // RAII device allocation
+  void runDevice(int ordinal, logger::BackendScope &backend);
+  void runComputeMad(const struct MadTest &t);
+  void runUnsupportedMatrixRows(Category phase, bool wmma);
+  void runMfma(Category phase);
+  void runSparseMfma(Category phase);
+  void runGemmFp();
+  void runGemmFp8();
+  void runGemmInt();
+  void runGlobalBandwidth();
+  void runNotBuilt(const char *tag, const char *display, std::initializer_list<std::string> metrics, const char *why,
+                   ResultStatus status);
+  void runKernelLatency(const benchmark_config_t &cfg);
+};

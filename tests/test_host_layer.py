@@ -1,0 +1,243 @@
+"""Host layer (C++ Peak / logger / result store / CLI) on a machine without a GPU: the CLI runs
+against the stand-in device, so row set, order, gating, degrade paths and the dump formats are
+all exercised; no kernel runs."""
+import ctypes as C
+import os
+import re
+import subprocess
+import xml.etree.ElementTree as ET
+
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+from oracle import workloads as wl
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CLI = os.path.join(ROOT, "clpeak_amd", "clpeak-mi355")
+HOSTLIB = os.path.join(ROOT, "clpeak_amd", "libclpeak_host.so")
+
+
+def run_cli(*args, env=None):
+    e = dict(os.environ)
+    e.update(env or {})
+    return subprocess.run([CLI, "--fake-device", "--small-shapes", *args], capture_output=True, text=True, env=e, timeout=120)
+
+
+# The rows a ROCm device reports, in order: (test tag, unit, metrics).  Tags, units and metric
+# names are the reference's (src/rocm/*.cpp); the tags marked + are rows this backend adds.
+EXPECTED_ROWS = [
+    ("single_precision_compute", "gflops", ["float", "float2", "float4"]),
+    ("half_precision_compute", "gflops", ["half", "half2"]),
+    ("double_precision_compute", "gflops", ["double", "double2", "double4"]),
+    ("mixed_precision_compute", "gflops", ["mp"]),
+    ("bfloat16_compute", "gflops", ["bf16"]),
+    ("wmma_fp16", "tflops", ["wmma_fp16"]), ("wmma_bf16", "tflops", ["wmma_bf16"]),
+    ("wmma_fp8_e4m3", "tflops", ["wmma_fp8_e4m3"]), ("wmma_fp8_e5m2", "tflops", ["wmma_fp8_e5m2"]),
+    ("rocwmma-fp", "tflops", ["rocwmma_fp16"]),
+    ("mfma_fp16", "tflops", ["mfma_fp16"]), ("mfma_fp16_32x32x16", "tflops", ["mfma_fp16_32x32x16"]),  # +
+    ("mfma_bf16", "tflops", ["mfma_bf16"]), ("mfma_bf16_32x32x16", "tflops", ["mfma_bf16_32x32x16"]),  # +
+    ("mfma_fp8", "tflops", ["mfma_fp8"]), ("mfma_bf8", "tflops", ["mfma_bf8"]),                          # +
+    ("mfma_mxfp6_e2m3", "tflops", ["mfma_mxfp6_e2m3"]), ("mfma_mxfp6_e3m2", "tflops", ["mfma_mxfp6_e3m2"]),  # +
+    ("mfma_mxfp4", "tflops", ["mfma_mxfp4"]),
+    ("smfmac_fp16", "tflops", ["smfmac_fp16"]), ("smfmac_bf16", "tflops", ["smfmac_bf16"]),
+    ("smfmac_fp8", "tflops", ["smfmac_fp8"]), ("smfmac_bf8", "tflops", ["smfmac_bf8"]),                  # +
+    ("rocblas-fp", "tflops", ["fp32", "fp64", "fp16", "bf16"]),
+    ("hipblaslt-fp8", "tflops", ["fp8_e4m3", "fp8_e5m2", "mxf4_e2m1"]),
+    ("integer_compute", "gops", ["int", "int2", "int4"]),
+    ("integer_compute_int8_dp", "gops", ["int8_dp", "int8_dp2", "int8_dp4", "int8_dp8"]),
+    ("wmma_int8", "tops", ["wmma_int8"]), ("rocwmma-int", "tops", ["rocwmma_int8"]),
+    ("mfma_int8", "tops", ["mfma_int8"]), ("smfmac_int8", "tops", ["smfmac_int8"]),
+    ("rocblas-int", "tops", ["int8"]),
+    ("global_memory_bandwidth", "gbps", ["float", "float2", "float4"]),
+    ("local_memory_bandwidth", "gbps", ["float", "float2", "float4"]),
+    ("image_memory_bandwidth", "gbps", ["float4"]),
+    ("transfer_bandwidth", "gbps", ["h2d_pinned", "d2h_pinned"]),
+    ("kernel_launch_latency", "us", ["dispatch", "roundtrip"]),
+]
+CATEGORY_OF_UNIT = {"gflops": "fp_compute", "tflops": "fp_compute", "gops": "int_compute", "tops": "int_compute",
+                    "gbps": "bandwidth", "us": "latency"}
+
+
+def parse_xml(path):
+    root = ET.parse(path).getroot()
+    rows = []
+    for run in root.findall("run"):
+        for cat in run.findall("category"):
+            for test in cat.findall("test"):
+                rows.append((cat.get("name"), test.get("name"), test.get("unit"),
+                             [(m.get("name"), m.get("status"), m.text) for m in test.findall("metric")]))
+    return root, rows
+
+
+def test_full_run_row_contract_and_xml(tmp_path):
+    x = tmp_path / "out.xml"
+    r = run_cli("--xml-file", str(x))
+    assert r.returncode == 0, r.stderr
+    root, rows = parse_xml(x)
+    assert root.get("format_version") == "2" and root.get("os") == "Linux x64"
+    run = root.find("run")
+    assert run.get("backend") == "ROCm" and run.get("platform") == "ROCm" and run.get("device") == "Fake MI355X"
+    assert [p.get("name") for p in run.findall("prop")] == ["Arch", "HIP", "CUs", "Wave", "VRAM"]
+    assert [(t, u, [m[0] for m in ms]) for _, t, u, ms in rows] == EXPECTED_ROWS
+    for cat, _, unit, _ in rows:
+        assert cat == CATEGORY_OF_UNIT[unit]
+    # measured values carry exactly 4 decimals
+    vals = [m[2] for _, _, _, ms in rows for m in ms if m[1] is None]
+    assert len(vals) == 38 and all(re.fullmatch(r"-?\d+\.\d{4}", v) for v in vals)
+    # rows that are deliberate skips keep the reference's status
+    status = {(t, m[0]): m[1] for _, t, _, ms in rows for m in ms}
+    assert status[("kernel_launch_latency", "dispatch")] == "unsupported"
+    assert status[("image_memory_bandwidth", "float4")] == "unsupported"
+    assert status[("wmma_fp16", "wmma_fp16")] == "unsupported"
+    assert status[("rocblas-fp", "bf16")] is None and status[("rocblas-fp", "fp32")] == "unsupported"
+    assert status[("hipblaslt-fp8", "fp8_e4m3")] is None
+
+
+def test_text_table_format():
+    r = run_cli("--single-precision-compute", "--global-memory-bandwidth")
+    out = r.stdout
+    assert "Single-precision compute (GFLOPS)" in out and "Global memory bandwidth (GBPS)" in out
+    assert re.search(r"^\s+float    : \d+\.\d\d$", out, re.M) and re.search(r"^\s+float4   : \d+\.\d\d$", out, re.M)
+    assert "MFMA" not in out and "latency" not in out.lower()
+
+
+def test_allow_list_and_subtract_flags(tmp_path):
+    x = tmp_path / "o.xml"
+    run_cli("--mfma", "--xml-file", str(x))
+    _, rows = parse_xml(x)
+    tags = [t for _, t, _, _ in rows]
+    assert tags[0] == "mfma_fp16" and "smfmac_int8" in tags and "mfma_int8" in tags     # Mfma gates dense and sparse, fp and int
+    assert not any(t.startswith(("single", "rocblas", "global", "wmma")) for t in tags)
+    run_cli("--no-mfma", "--no-int-compute", "--xml-file", str(x))
+    _, rows = parse_xml(x)
+    tags = [t for _, t, _, _ in rows]
+    assert not any("mfma" in t for t in tags) and "integer_compute" not in tags and "rocblas-int" not in tags
+    assert "rocblas-fp" in tags and "global_memory_bandwidth" in tags
+    run_cli("--bandwidth", "--xml-file", str(x))
+    _, rows = parse_xml(x)
+    assert {c for c, _, _, _ in rows} == {"bandwidth"}
+
+
+def test_no_device_is_a_note_and_status_zero():
+    r = run_cli(env={"CLPEAK_FAKE_DEVICES": "0"})
+    assert r.returncode == 0 and "ROCm: no devices found" in r.stdout and "Backend:" not in r.stdout
+
+
+def test_device_selection(tmp_path):
+    x = tmp_path / "o.xml"
+    r = run_cli("--rocm-device", "1", "--kernel-launch-latency", "--xml-file", str(x), env={"CLPEAK_FAKE_DEVICES": "3"})
+    assert r.stdout.count("Device 1:") == 1 and "Device 0:" not in r.stdout and "Device 2:" not in r.stdout
+    r = run_cli("--rocm-device", "99", "--kernel-launch-latency")
+    assert r.returncode == 0 and "Device" not in r.stdout
+    assert run_cli("--rocm-device", "x").returncode == 1
+    assert run_cli("--no-such-flag").returncode == 1
+
+
+@pytest.mark.parametrize("entry,tag,metric", [("mfma_dense", "mfma_bf16", "mfma_bf16"), ("gemm_bf16", "rocblas-fp", "bf16"),
+                                              ("global_bandwidth", "global_memory_bandwidth", "float4"),
+                                              ("alloc", "single_precision_compute", "float"),
+                                              ("launch_roundtrip", "kernel_launch_latency", "roundtrip")])
+def test_failures_degrade_to_error_rows(tmp_path, entry, tag, metric):
+    """Any failing device call becomes an `error` row for the readings it affects; the run goes on."""
+    x = tmp_path / "o.xml"
+    r = run_cli("--xml-file", str(x), env={"CLPEAK_FAKE_FAIL": entry})
+    assert r.returncode == 0
+    _, rows = parse_xml(x)
+    assert [t for _, t, _, _ in rows] == [t for t, _, _ in EXPECTED_ROWS]      # same test set, same order
+    status = {(t, m[0]): m[1] for _, t, _, ms in rows for m in ms}
+    assert status[(tag, metric)] == "error"
+    assert status[("kernel_launch_latency", "dispatch")] == "unsupported"
+
+
+def test_dump_formats_round_trip(tmp_path):
+    x, j, c = tmp_path / "a.xml", tmp_path / "a.json", tmp_path / "a.csv"
+    r = run_cli("--xml-file", str(x), "--json-file", str(j), "--csv-file", str(c), env={"CLPEAK_FAKE_FAIL": "smfmac"})
+    assert r.returncode == 0
+    # JSON: one entry object per line, reference field names
+    import json
+    doc = json.loads(j.read_text())
+    assert doc["format_version"] == 2 and doc["devices"][0]["props"][0] == {"k": "Arch", "v": "gfx950:sramecc+:xnack-"}
+    _, rows = parse_xml(x)
+    n_metrics = sum(len(ms) for _, _, _, ms in rows)
+    assert len(doc["entries"]) == n_metrics
+    ok = [e for e in doc["entries"] if "value" in e]
+    bad = [e for e in doc["entries"] if "status" in e]
+    assert len(ok) + len(bad) == n_metrics and all("reason" in e for e in bad) and all("status" not in e for e in ok)
+    assert {e["status"] for e in bad} == {"unsupported", "skipped", "error"}
+    assert set(ok[0]) >= {"backend", "platform", "device", "driver", "category", "test", "metric", "unit", "display", "value"}
+    # CSV: header + one row per metric, format_version first, 15 columns
+    lines = c.read_text().strip().split("\n")
+    assert lines[0].startswith("format_version,backend,platform,device,driver,category,test,metric,unit,status,value,reason")
+    assert len(lines) == n_metrics + 1 and all(l.startswith("2,ROCm,ROCm,Fake MI355X,") for l in lines[1:])
+    # --compare against its own dump prints a zero delta on every measured row (loader round trip)
+    for f in (x, j, c):
+        r2 = run_cli("--compare", str(f), "--single-precision-compute")
+        assert r2.stdout.count("(was 83.89, ") == 3 and r2.stdout.count("0.0%)") == 3, f
+
+
+def test_reference_result_files_load(tmp_path):
+    """A result file in the reference's own XML grammar (written out here by hand from its
+    documented tree) loads through --compare and matches on the row key."""
+    ref = tmp_path / "ref.xml"
+    ref.write_text('<?xml version="1.0" encoding="utf-8"?>\n<clpeak format_version="2" clpeak_version="2.0.16" os="Linux x64">\n'
+                   '  <run backend="ROCm" platform="ROCm" device="Fake MI355X" driver="6.0.0">\n    <prop name="CUs" value="256"/>\n'
+                   '    <category name="fp_compute">\n      <test name="single_precision_compute" display="Single-precision compute" unit="gflops">\n'
+                   '        <metric name="float" info="x &amp; y">41.9431</metric>\n        <metric name="float2" status="unsupported" reason="n/a"/>\n'
+                   '      </test>\n    </category>\n  </run>\n</clpeak>\n')
+    r = run_cli("--compare", str(ref), "--single-precision-compute")
+    assert r.stdout.count("(was 41.94, +100.0%)") == 1 and r.stdout.count("(was ") == 1
+    old = tmp_path / "v1.xml"
+    old.write_text('<clpeak format_version="1">\n<run backend="ROCm" platform="ROCm" device="Fake MI355X" driver="1">\n</run></clpeak>\n')
+    assert "(was" not in run_cli("--compare", str(old), "--single-precision-compute").stdout
+
+
+# ---- pieces reached through the host library --------------------------------------------------------
+@pytest.fixture(scope="module")
+def host():
+    L = C.CDLL(HOSTLIB)
+    L.clpeak_host_pick_iters.argtypes = [C.c_double, C.c_uint, C.c_uint, C.c_uint]; L.clpeak_host_pick_iters.restype = C.c_uint
+    L.clpeak_host_target_global_threads.argtypes = [C.c_uint]; L.clpeak_host_target_global_threads.restype = C.c_ulonglong
+    L.clpeak_host_seeded_operand.argtypes = [C.c_int, C.c_double, C.c_ulonglong, C.c_uint, C.c_ulonglong, C.c_void_p, C.c_size_t]
+    L.clpeak_host_seeded_operand.restype = C.c_size_t
+    L.clpeak_host_seeded_bytes.argtypes = [C.c_int, C.c_ulonglong, C.c_uint, C.c_ulonglong, C.c_void_p]
+    L.clpeak_host_seeded_bytes.restype = C.c_size_t
+    return L
+
+
+def test_pick_iters_and_launch_width(host):
+    """Calibration rules of the reference (src/common/common.cpp:35-45, include/common/common.h:142-147)."""
+    p = host.clpeak_host_pick_iters
+    assert p(100.0, 500000, 0, 10000) == 5000
+    assert p(0.01, 500000, 0, 10000) == 10000            # sub-microsecond probes count as 1 us, then the cap
+    assert p(1e9, 500000, 0, 10000) == 1                 # one launch already over budget
+    assert p(100.0, 500000, 7, 10000) == 7               # --iters wins
+    assert p(1000.0, 0, 0, 10000) == 5000                # 0 = the legacy 5 s budget
+    assert p(1.0, 2000000, 0, 100000000) == 2000000      # the CPU harness' larger cap
+    assert host.clpeak_host_target_global_threads(256) == 256 * 2048 * 256
+    assert host.clpeak_host_target_global_threads(4) == 32 << 20
+
+
+@pytest.mark.parametrize("fmt,ofmt,sigma", [(0, orc.FMT_F16, 0.01), (1, orc.FMT_BF16, 0.01), (2, orc.FMT_E4M3, 1.0),
+                                            (3, orc.FMT_E5M2, 1.0), (4, orc.FMT_E2M3, 1.0), (5, orc.FMT_E3M2, 1.0),
+                                            (6, orc.FMT_E2M1, 1.0), (2, orc.FMT_E4M3, 300.0), (0, orc.FMT_F16, 3e4)])
+def test_host_operand_generator_matches_oracle(host, fmt, ofmt, sigma):
+    """The backend's own host-side generator and the oracle's produce the same operand bytes."""
+    n, seed, stream = 8192, wl.DEFAULT_SEED, wl.STREAM_MFMA_A
+    bits = {0: 16, 1: 16, 2: 8, 3: 8, 4: 6, 5: 6, 6: 4}[fmt]
+    buf = np.zeros(n * bits // 8, dtype=np.uint8)
+    assert host.clpeak_host_seeded_operand(fmt, sigma, seed, stream, n, buf.ctypes.data, buf.size) == buf.size
+    codes = orc.fill_normal_codes(ofmt, sigma, seed, stream, n)
+    ref = codes.view(np.uint8) if bits in (8, 16) else orc.pack_bits(codes, bits)
+    assert np.array_equal(buf, ref)
+
+
+def test_host_int8_scales_and_sparse_metadata_match_oracle(host):
+    n, seed = 4096, wl.DEFAULT_SEED
+    buf = np.zeros(n, dtype=np.uint8)
+    host.clpeak_host_seeded_operand(7, 0.0, seed, wl.STREAM_MFMA_B, n, buf.ctypes.data, n)
+    assert np.array_equal(buf.view(np.int8), orc.fill_int8(seed, wl.STREAM_MFMA_B, n))
+    host.clpeak_host_seeded_bytes(0, seed, wl.STREAM_SCALE_A, n, buf.ctypes.data)
+    assert np.array_equal(buf, orc.fill_e8m0(seed, wl.STREAM_SCALE_A, n))
+    host.clpeak_host_seeded_bytes(1, seed, wl.STREAM_SPARSE, n, buf.ctypes.data)
+    assert np.array_equal(buf, orc.fill_sparse_meta(seed, wl.STREAM_SPARSE, n))
