@@ -109,7 +109,10 @@ int main(int argc, char **argv) {
   }
 
   const Mi355Api &api = fake ? mi355_fake_api() : mi355_real_api();
-  if (opts.listDevices) return Mi355Peak::listDevices(api, std::cout) < 0 ? 1 : 0;
+  if (opts.listDevices) {
+    Mi355Peak::printInventory(Mi355Peak::enumerate(api), std::cout);
+    return 0;
+  }
 
   Mi355Peak peak(api);
   peak.workload = shape;

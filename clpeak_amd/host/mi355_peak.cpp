@@ -36,22 +36,48 @@ void Mi355Peak::applyOptions(const CliOptions &opts) {
   deviceIndices = opts.rocmDeviceIndices;
 }
 
-int Mi355Peak::listDevices(const Mi355Api &api, std::ostream &os) {
+BackendInventory Mi355Peak::enumerate(const Mi355Api &api) {
+  BackendInventory inv;
+  inv.backend = "ROCm";
   int n = 0;
-  if (api.device_count(&n) != MI355_OK) return -1;
+  if (api.device_count(&n) != MI355_OK || n == 0) return inv;
+  inv.available = true;
+  InventoryPlatform plat;
+  plat.index = 0;
+  plat.name = "ROCm/HIP";
   for (int i = 0; i < n; i++) {
     mi355_dev *d = nullptr;
-    if (api.open(i, &d) != MI355_OK) {
-      os << "ROCm device " << i << ": not usable by this backend (" << api.last_error(nullptr) << ")\n";
-      continue;
-    }
+    if (api.open(i, &d) != MI355_OK) continue;   // not a gfx950 part: not this backend's device
     mi355_props_t p;
     api.get_props(d, &p);
-    os << "ROCm device " << i << ": " << p.name << " (" << p.arch << ", " << p.num_cus << " CUs, "
-       << (p.total_mem >> 20) << " MB)\n";
     api.close(d);
+    InventoryDevice dev;
+    dev.index = i;
+    dev.name = p.name;
+    dev.typeStr = "GPU";
+    dev.driverVersion = p.driver_version;
+    dev.numComputeUnits = (unsigned)p.num_cus;
+    dev.maxClockMHz = (unsigned)(p.clock_khz / 1000);
+    dev.globalMemBytes = p.total_mem;
+    dev.hasFp16 = dev.hasFp64 = true;
+    plat.devices.push_back(dev);
   }
-  return n;
+  inv.platforms.push_back(plat);
+  return inv;
+}
+
+void Mi355Peak::printInventory(const BackendInventory &inv, std::ostream &os) {
+  os << "\n=== ROCm backend ===\n";
+  if (!inv.available) {
+    os << "ROCm: runtime init failed or no devices found\n";
+    return;
+  }
+  for (const InventoryPlatform &plat : inv.platforms)
+    for (const InventoryDevice &d : plat.devices) {
+      os << "  ROCm Device " << d.index << ": " << d.name;
+      if (!d.typeStr.empty()) os << " [" << d.typeStr << "]";
+      os << "\n";
+    }
 }
 
 float Mi355Peak::runKernel(const std::function<int()> &launch, unsigned targetUs, unsigned forcedIters) {

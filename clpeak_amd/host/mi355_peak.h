@@ -9,6 +9,7 @@
 #include <functional>
 #include <vector>
 #include "device_api.h"
+#include "inventory.h"
 #include "peak.h"
 
 class Mi355Peak : public Peak {
@@ -19,8 +20,10 @@ class Mi355Peak : public Peak {
   void applyOptions(const CliOptions &opts) override;
   int runAll() override;
 
-  // One line per device: "ROCm device <i>: <name> (<arch>, <CUs> CUs, <VRAM> MB)".
-  static int listDevices(const Mi355Api &api, std::ostream &os);
+  // What the front ends call for --list-devices and the backend catalog
+  // (RocmPeak::enumerate / printInventory, src/rocm/rocm_peak.cpp:231-278).
+  static BackendInventory enumerate(const Mi355Api &api = mi355_real_api());
+  static void printInventory(const BackendInventory &inv, std::ostream &os);
 
   // Shapes of the seeded workloads.  Defaults are the configured ones; tests shrink them.
   struct Workload {

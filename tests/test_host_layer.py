@@ -124,6 +124,13 @@ def test_no_device_is_a_note_and_status_zero():
     assert r.returncode == 0 and "ROCm: no devices found" in r.stdout and "Backend:" not in r.stdout
 
 
+def test_list_devices():
+    r = run_cli("--list-devices", env={"CLPEAK_FAKE_DEVICES": "2"})
+    assert r.returncode == 0 and "=== ROCm backend ===" in r.stdout
+    assert "ROCm Device 0: Fake MI355X [GPU]" in r.stdout and "ROCm Device 1: Fake MI355X [GPU]" in r.stdout
+    assert "no devices found" in run_cli("--list-devices", env={"CLPEAK_FAKE_DEVICES": "0"}).stdout
+
+
 def test_device_selection(tmp_path):
     x = tmp_path / "o.xml"
     r = run_cli("--rocm-device", "1", "--kernel-launch-latency", "--xml-file", str(x), env={"CLPEAK_FAKE_DEVICES": "3"})
