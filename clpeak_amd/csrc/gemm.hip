@@ -10,9 +10,8 @@
 //
 // Data movement.  Global memory goes straight into LDS (global_load_lds_dwordx4, 16
 // bytes per lane, no staging registers, no ds_write): one such instruction moves 8
-// rows x 128 B, a wave issues 4 for A and 4 for B per step.  The loads of slab s+2
-// are issued in the middle of step s, right after the barrier that frees their
-// buffer, so they have a whole step to land.
+// rows x 128 B.  The loads of slab s+2 are issued during step s, right after the barrier
+// that frees their buffer, so they have most of a step to land.
 //
 // LDS layout.  A row's 128 bytes are eight 16-byte chunks; chunk c of row r is stored
 // at chunk position c ^ (r & 7).  A fragment read (16 lanes = 16 consecutive rows,
@@ -20,14 +19,15 @@
 // one bank group 16 times.  The direct-to-LDS load writes lane i at position i of its
 // 1 KiB destination, so lane i fetches the global chunk that belongs there.
 //
-// Schedule of one step (bf16: two K=32 halves, fragment sets F0 and F1):
-//     32 MFMAs on F0, the 12 LDS reads of F1 slipped between the first 20
+// Schedule of one step: 64 MFMAs per wave, 32 on fragment set F0 (first K half of the slab) then
+// 32 on F1 (second half); never more than one memory instruction between two MFMAs:
+//     MFMA  0..12   one LDS read of F1 in each of the first 12 gaps
 //     wait F1; wait own global loads; barrier      <- slab s+1 complete, slab s free
-//     32 MFMAs on F1; between them the 12 LDS reads of the next step's F0 and the 8
-//     global->LDS loads of slab s+2 into the freed buffer
-// One barrier per step; an MFMA is always the first thing a wave issues after the barrier
-// (its operands are already in registers), memory instructions are spread out so that a
-// wave never sits on a full memory queue with MFMAs waiting behind it.  The loop body is inline assembly so that this order is the order issued;
+//     MFMA 13..39   the wave's 8 global->LDS loads of slab s+2, one every third MFMA
+//     MFMA 40..63   one LDS read of the next step's F0 in each of the first 12 gaps
+// One barrier per step, placed as early as the F1 reads allow so that the loads of slab s+2 have
+// the rest of this step and the start of the next to land.
+// The loop body is inline assembly so that this order is the order issued;
 // the compiler knows neither the LDS reads nor the MFMAs and therefore inserts no wait
 // states of its own: every s_waitcnt below is part of the schedule.
 //
@@ -59,6 +59,12 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
   __builtin_amdgcn_global_load_lds((global_void_ptr)gptr, (lds_void_ptr)(uintptr_t)lds_dst, 16, 0, 0);
 }
 
+// The same as instructions in the hand-scheduled loop: scalar base + per-lane 32-bit offset (no
+// vector ALU work per load), LDS destination through M0 (one wait state after writing it).
+#define MI355_LOAD_LDS(voff, sbase, m0val)                                                         \
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"                     \
+               :: "v"(voff), "s"(sbase), "s"(m0val) : "memory", "m0")
+
 #define MI355_DS_READ(dst, addr, off) \
   asm volatile("ds_read_b128 %0, %1 offset:" #off : "=v"(dst) : "v"(addr))
 
@@ -82,10 +88,88 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
 #define MI355_MFMA_BF16(acc, fb, fa) \
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(fb), "v"(fa))
 
-// One row of MFMAs: the 4 tiles that share A fragment i.
-#define MI355_MFMA_ROW(acc, fa, fb, i)                                                             \
-  MI355_MFMA_BF16(acc[i][0], fb[0], fa[i]); MI355_MFMA_BF16(acc[i][1], fb[1], fa[i]);              \
-  MI355_MFMA_BF16(acc[i][2], fb[2], fa[i]); MI355_MFMA_BF16(acc[i][3], fb[3], fa[i])
+// State of one wave's walk along K that the step function advances.
+struct GemmWalk {
+  uint32_t a_cur, b_cur, a_nxt, b_nxt;   // LDS byte addresses of this lane's first A / B fragment, both buffers
+  uint32_t dst;                          // LDS destination of the wave's 32 A rows in the buffer to refill
+  uint64_t ga, gb;                       // uniform global addresses of those A / B rows in the next slab to fetch
+  uint32_t voff;                         // this lane's byte offset from ga / gb within a group of 8 rows
+  uint32_t row8;                         // bytes between rows r and r+8 (load q reads from base + q*row8)
+};
+
+// One step of K: 64 MFMAs per wave, 32 on fragment set F0 (first K half of the slab) then 32 on
+// F1.  The order written here is the order issued; never more than one memory instruction between
+// two MFMAs, because a ds_read_b128 (about 11 cycles of issue) slips into the 16-cycle shadow of
+// the MFMA before it, while two in a row would stall the matrix pipe.
+// MAIN: a step of the steady state; otherwise `reads` / `loads` are run-time (wave-uniform)
+// switches for the last steps, which have nothing left to prefetch.
+template <bool MAIN>
+__device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8], bf16x8v (&fb0)[4],
+                                          bf16x8v (&fa1)[8], bf16x8v (&fb1)[4], const GemmWalk &w,
+                                          bool reads, bool loads) {
+  const bool READS = MAIN || reads, LOADS = MAIN || loads;
+  const uint32_t a1 = w.a_cur ^ 64u, b1 = w.b_cur ^ 64u;   // second K half of this step
+#define MM(F, i, j) MI355_MFMA_BF16(acc[i][j], F##b##_[j], F##a##_[i])
+#define LDA(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst + (q) * 1024u)
+#define LDB(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst + kSlabBytes + (q) * 1024u)
+  bf16x8v(&x0a_)[8] = fa0; bf16x8v(&x0b_)[4] = fb0; bf16x8v(&x1a_)[8] = fa1; bf16x8v(&x1b_)[4] = fb1;
+  // ---- MFMAs 0..12 (on F0); the 12 reads of F1 in the first 12 gaps -----------------------------
+  MM(x0, 0, 0); MI355_DS_READ(fb1[0], b1, 0);
+  MM(x0, 0, 1); MI355_DS_READ(fb1[1], b1, 2048);
+  MM(x0, 0, 2); MI355_DS_READ(fb1[2], b1, 4096);
+  MM(x0, 0, 3); MI355_DS_READ(fb1[3], b1, 6144);
+  MM(x0, 1, 0); MI355_DS_READ(fa1[0], a1, 0);
+  MM(x0, 1, 1); MI355_DS_READ(fa1[1], a1, 2048);
+  MM(x0, 1, 2); MI355_DS_READ(fa1[2], a1, 4096);
+  MM(x0, 1, 3); MI355_DS_READ(fa1[3], a1, 6144);
+  MM(x0, 2, 0); MI355_DS_READ(fa1[4], a1, 8192);
+  MM(x0, 2, 1); MI355_DS_READ(fa1[5], a1, 10240);
+  MM(x0, 2, 2); MI355_DS_READ(fa1[6], a1, 12288);
+  MM(x0, 2, 3); MI355_DS_READ(fa1[7], a1, 14336);
+  MM(x0, 3, 0);
+  MI355_WAIT_FRAGS(fa1, fb1);
+  // every wave holds all fragments of this step's slab (its buffer is free) and every wave's
+  // share of the next slab has landed
+  asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+  // ---- MFMAs 13..39: fetch the slab two steps ahead, one load every third MFMA -------------------
+  MM(x0, 3, 1); LDA(0);
+  MM(x0, 3, 2); MM(x0, 3, 3);
+  MM(x0, 4, 0); LDB(0);
+  MM(x0, 4, 1); MM(x0, 4, 2);
+  MM(x0, 4, 3); LDA(1);
+  MM(x0, 5, 0); MM(x0, 5, 1);
+  MM(x0, 5, 2); LDB(1);
+  MM(x0, 5, 3); MM(x0, 6, 0);
+  MM(x0, 6, 1); LDA(2);
+  MM(x0, 6, 2); MM(x0, 6, 3);
+  MM(x0, 7, 0); LDB(2);
+  MM(x0, 7, 1); MM(x0, 7, 2);
+  MM(x0, 7, 3); LDA(3);
+  MM(x1, 0, 0); MM(x1, 0, 1);
+  MM(x1, 0, 2); LDB(3);
+  MM(x1, 0, 3); MM(x1, 1, 0);
+  MM(x1, 1, 1); MM(x1, 1, 2); MM(x1, 1, 3);
+  // ---- MFMAs 40..63 (on F1); F0 is dead since MFMA 31: the next step's F0 reads, one per gap -----
+  MM(x1, 2, 0); if (READS) MI355_DS_READ(fb0[0], w.b_nxt, 0);
+  MM(x1, 2, 1); if (READS) MI355_DS_READ(fb0[1], w.b_nxt, 2048);
+  MM(x1, 2, 2); if (READS) MI355_DS_READ(fb0[2], w.b_nxt, 4096);
+  MM(x1, 2, 3); if (READS) MI355_DS_READ(fb0[3], w.b_nxt, 6144);
+  MM(x1, 3, 0); if (READS) MI355_DS_READ(fa0[0], w.a_nxt, 0);
+  MM(x1, 3, 1); if (READS) MI355_DS_READ(fa0[1], w.a_nxt, 2048);
+  MM(x1, 3, 2); if (READS) MI355_DS_READ(fa0[2], w.a_nxt, 4096);
+  MM(x1, 3, 3); if (READS) MI355_DS_READ(fa0[3], w.a_nxt, 6144);
+  MM(x1, 4, 0); if (READS) MI355_DS_READ(fa0[4], w.a_nxt, 8192);
+  MM(x1, 4, 1); if (READS) MI355_DS_READ(fa0[5], w.a_nxt, 10240);
+  MM(x1, 4, 2); if (READS) MI355_DS_READ(fa0[6], w.a_nxt, 12288);
+  MM(x1, 4, 3); if (READS) MI355_DS_READ(fa0[7], w.a_nxt, 14336);
+  MM(x1, 5, 0); MM(x1, 5, 1); MM(x1, 5, 2); MM(x1, 5, 3);
+  MM(x1, 6, 0); MM(x1, 6, 1); MM(x1, 6, 2); MM(x1, 6, 3);
+  MM(x1, 7, 0); MM(x1, 7, 1); MM(x1, 7, 2); MM(x1, 7, 3);
+  MI355_WAIT_FRAGS(fa0, fb0);
+#undef LDA
+#undef LDB
+#undef MM
+}
 
 __device__ inline void tile_of_block(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn) {
   const uint32_t bid = blockIdx.x, total = tiles_m * tiles_n;
@@ -102,7 +186,8 @@ __global__ void __launch_bounds__(kThreads)
 gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, uint16_t *__restrict__ C,
                  uint32_t N, uint32_t k_bytes, uint32_t tiles_m, uint32_t tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-  const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const uint32_t tid = threadIdx.x, lane = tid % 64;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);   // wave-uniform, and known to be
   const uint32_t wm = wave / 4, wn = wave % 4;
   uint32_t tm, tn;
   tile_of_block(tiles_m, tiles_n, tm, tn);
@@ -147,60 +232,25 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, u
   MI355_READ_FRAGS(fa0, fb0, a_cur, b_cur);
   MI355_WAIT_FRAGS(fa0, fb0);
 
-  // Per-lane global pointers of the next slab to fetch (advanced by one step per trip) and
-  // the wave's LDS destination for it.
-  const uint8_t *ga_next = ga + 2 * (size_t)kRowBytes, *gb_next = gb + 2 * (size_t)kRowBytes;
-  const size_t row8 = 8 * (size_t)k_bytes;
-
-  for (uint32_t s = 0; s < steps; s++) {
-    const uint32_t buf = s & 1u;
-    const uint32_t a1 = a_cur ^ 64u, b1 = b_cur ^ 64u;   // second K half of this step
-    // ---- first half: MFMAs on F0, the reads of F1 slipped in between ---------------------------
-    MI355_DS_READ(fb1[0], b1, 0);     MI355_DS_READ(fb1[1], b1, 2048);
-    MI355_MFMA_ROW(acc, fa0, fb0, 0);
-    MI355_DS_READ(fb1[2], b1, 4096);  MI355_DS_READ(fb1[3], b1, 6144);
-    MI355_DS_READ(fa1[0], a1, 0);     MI355_DS_READ(fa1[1], a1, 2048);
-    MI355_MFMA_ROW(acc, fa0, fb0, 1);
-    MI355_DS_READ(fa1[2], a1, 4096);  MI355_DS_READ(fa1[3], a1, 6144);
-    MI355_MFMA_ROW(acc, fa0, fb0, 2);
-    MI355_DS_READ(fa1[4], a1, 8192);  MI355_DS_READ(fa1[5], a1, 10240);
-    MI355_MFMA_ROW(acc, fa0, fb0, 3);
-    MI355_DS_READ(fa1[6], a1, 12288); MI355_DS_READ(fa1[7], a1, 14336);
-    MI355_MFMA_ROW(acc, fa0, fb0, 4);
-    MI355_MFMA_ROW(acc, fa0, fb0, 5);
-    MI355_MFMA_ROW(acc, fa0, fb0, 6);
-    MI355_MFMA_ROW(acc, fa0, fb0, 7);
-    MI355_WAIT_FRAGS(fa1, fb1);
-    // every wave is done reading slab s; every wave's share of slab s+1 has landed
-    asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-    // ---- second half: MFMAs on F1 first (they are ready), next F0 reads and the global loads
-    //      of slab s+2 spread between them so that no wave sits on the memory queues ------------
-    const bool more_reads = s + 1 < steps, more_loads = s + 2 < steps;
-    const uint32_t dst = dst_wave + buf * kBufBytes;
-    MI355_MFMA_ROW(acc, fa1, fb1, 0);
-    if (more_reads) { MI355_DS_READ(fb0[0], b_nxt, 0);    MI355_DS_READ(fb0[1], b_nxt, 2048);
-                      MI355_DS_READ(fb0[2], b_nxt, 4096); MI355_DS_READ(fb0[3], b_nxt, 6144); }
-    MI355_MFMA_ROW(acc, fa1, fb1, 1);
-    if (more_reads) { MI355_DS_READ(fa0[0], a_nxt, 0);    MI355_DS_READ(fa0[1], a_nxt, 2048);
-                      MI355_DS_READ(fa0[2], a_nxt, 4096); MI355_DS_READ(fa0[3], a_nxt, 6144); }
-    MI355_MFMA_ROW(acc, fa1, fb1, 2);
-    if (more_reads) { MI355_DS_READ(fa0[4], a_nxt, 8192);  MI355_DS_READ(fa0[5], a_nxt, 10240);
-                      MI355_DS_READ(fa0[6], a_nxt, 12288); MI355_DS_READ(fa0[7], a_nxt, 14336); }
-    MI355_MFMA_ROW(acc, fa1, fb1, 3);
-    if (more_loads) { load_to_lds(ga_next, dst);                  load_to_lds(gb_next, dst + kSlabBytes); }
-    MI355_MFMA_ROW(acc, fa1, fb1, 4);
-    if (more_loads) { load_to_lds(ga_next + row8, dst + 1024u);   load_to_lds(gb_next + row8, dst + kSlabBytes + 1024u); }
-    MI355_MFMA_ROW(acc, fa1, fb1, 5);
-    if (more_loads) { load_to_lds(ga_next + 2 * row8, dst + 2048u); load_to_lds(gb_next + 2 * row8, dst + kSlabBytes + 2048u); }
-    MI355_MFMA_ROW(acc, fa1, fb1, 6);
-    if (more_loads) { load_to_lds(ga_next + 3 * row8, dst + 3072u); load_to_lds(gb_next + 3 * row8, dst + kSlabBytes + 3072u); }
-    MI355_MFMA_ROW(acc, fa1, fb1, 7);
-    MI355_WAIT_FRAGS(fa0, fb0);
-    ga_next += kRowBytes;
-    gb_next += kRowBytes;
-    uint32_t t = a_cur; a_cur = a_nxt; a_nxt = t;
-    t = b_cur; b_cur = b_nxt; b_nxt = t;
-  }
+  // The loads inside the loop take the scalar-base form (uniform 64-bit base + this lane's 32-bit
+  // offset), which costs no vector ALU work: load q of the wave covers rows 8q..8q+7 of its 32.
+  GemmWalk w;
+  w.a_cur = a_cur; w.b_cur = b_cur; w.a_nxt = a_nxt; w.b_nxt = b_nxt;
+  w.voff = (lane / 8u) * k_bytes + lchunk * 16u;
+  w.row8 = 8u * k_bytes;
+  w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
+  w.gb = (uint64_t)(uintptr_t)(B + ((size_t)tn * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
+  w.dst = dst_wave;
+  auto advance = [&](uint32_t s) {
+    w.dst = dst_wave + ((s + 1) & 1u) * kBufBytes;
+    w.ga += kRowBytes;
+    w.gb += kRowBytes;
+    uint32_t t = w.a_cur; w.a_cur = w.a_nxt; w.a_nxt = t;
+    t = w.b_cur; w.b_cur = w.b_nxt; w.b_nxt = t;
+  };
+  uint32_t s = 0;
+  for (; s + 2 < steps; s++) { gemm_step<true>(acc, fa0, fb0, fa1, fb1, w, true, true); advance(s); }
+  for (; s < steps; s++) { gemm_step<false>(acc, fa0, fb0, fa1, fb1, w, s + 1 < steps, false); advance(s); }
   // wait states the compiler cannot know about, before the accumulators are read
   asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
@@ -317,7 +367,7 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
   return MI355_OK;
 }
 
-constexpr size_t kLdsBytes = 2 * (size_t)kBufBytes;  // 128 KiB
+constexpr size_t kLdsBytes = 2 * (size_t)kBufBytes;  // two 64 KiB buffers
 
 }  // namespace
 
