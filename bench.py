@@ -147,24 +147,34 @@ def _gemm_rows(dev, capi, wl, add, budget):
             b.free()
 
 
-def cpu_baseline(seconds=12.0):
-    """The oracle's float4 read-reduce (scalar C, one core) over a 256 MiB buffer, repeated
-    for about `seconds` of CPU time."""
+def cpu_baseline(target_us=2_000_000, extra_target_us=1_000_000):
+    """The oracle's kernels on this host's cores, timed with the reference's CPU discipline (pinned
+    persistent pool, warm-ups, settle phase before the all-core run, adaptive probe, one timed batch
+    sized to the budget): one thread (ST) and every logical core (MT).  The headline figure is the
+    float4 read-reduce in its CPU-sized form (2^26 floats, 2^20 partial sums); the other workloads are
+    listed under "others" on bounded samples."""
     from oracle import pyoracle as orc
-    from oracle import workloads as wl
-    n = 1 << 26
-    data = orc.fill_f32(n, SEED, wl.STREAM_BW, 0)
-    T = 1 << 20
-    orc.global_bandwidth(4, data, T)  # warm-up / page-in
+    cores = len(os.sched_getaffinity(0))
     t0 = time.perf_counter()
-    passes = 0
-    while time.perf_counter() - t0 < seconds:
-        orc.global_bandwidth(4, data, T)
-        passes += 1
+    with orc.CpuPool(cores) as pool:
+        r = pool.measure(orc.CPUH_READ_FLOAT4, SEED, 2, target_us)
+        others = {}
+        for name, kind, unit, what in (
+                ("single_precision_compute float", orc.CPUH_MAD_F32, "gflops",
+                 "8 work-items x 16 accumulators x 4096 fma per iteration"),
+                ("mfma_bf16", orc.CPUH_MFMA_BF16, "gflops", "4 emulated 16x16x32 bf16 products per iteration"),
+                ("mfma_int8", orc.CPUH_MFMA_I8, "gops", "4 emulated 16x16x64 int8 products per iteration"),
+                ("rocblas-fp bf16", orc.CPUH_GEMM_BF16, "gflops", "one 64x64 tile of the K=8192 bf16 GEMM per iteration")):
+            q = pool.measure(kind, SEED, 2, extra_target_us)
+            others[name] = {"ST": round(q.giga_st, 3), "MT": round(q.giga_mt, 3), "unit": unit, "threads": q.threads_mt,
+                            "iters_ST": q.iters_st, "iters_MT": q.iters_mt, "sample": what}
     dt = time.perf_counter() - t0
-    return {"value": round(passes * n * 4 / dt / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{passes} passes of the float4 read-reduce over a 256 MiB (2^26 float) seeded buffer, "
-                      f"2^20 partial sums, scalar C oracle on one core, {dt:.1f} s"}
+    return {"value": round(r.giga_mt, 2), "unit": "GB/s", "cores": r.threads_mt, "kind": "port",
+            "ST": round(r.giga_st, 2), "MT": round(r.giga_mt, 2), "pinned_workers": r.pinned,
+            "sample": f"float4 read-reduce over a 256 MiB (2^26 float) seeded buffer, 2^20 partial sums, C oracle "
+                      f"(no fast-math): {r.iters_st} passes on 1 thread, {r.iters_mt} passes on {r.threads_mt} threads "
+                      f"(each thread a contiguous share of the partial sums); whole CPU leg {dt:.1f} s",
+            "others": others}
 
 
 def main():

@@ -199,6 +199,31 @@ void orc_global_bandwidth(int width, const float *in, uint64_t n_floats, uint64_
     free(acc);
 }
 
+/* The partial sums of threads [t0,t1) only, out[t0..t1) written: sweeps the 1/T-strided
+ * segments one after the other, so each thread still adds its vectors in ascending order and the
+ * result is the same as above bit for bit.  Disjoint ranges may run on different host threads. */
+void orc_global_bandwidth_range(int width, const float *in, uint64_t n_floats, uint64_t T, uint64_t t0, uint64_t t1,
+                                float *out)
+{
+    const uint64_t nvec = n_floats / (uint64_t)width, span = t1 - t0;
+    float *acc = (float *)calloc((size_t)span * (size_t)width, sizeof(float));
+    for (uint64_t base = 0; base < nvec; base += T) {
+        const uint64_t lo = base + t0, hi = base + t1 < nvec ? base + t1 : nvec;
+        for (uint64_t i = lo; i < hi; i++) {
+            float *a = acc + (i - lo) * (uint64_t)width;
+            const float *v = in + i * (uint64_t)width;
+            for (int c = 0; c < width; c++) a[c] = a[c] + v[c];
+        }
+    }
+    for (uint64_t t = 0; t < span; t++) {
+        const float *a = acc + t * (uint64_t)width;
+        float s = a[0];
+        for (int c = 1; c < width; c++) s = s + a[c];
+        out[t0 + t] = s;
+    }
+    free(acc);
+}
+
 /* Same partial for one thread, with the buffer regenerated from the seed (uniform
  * [0,1), stream `stream`): lets a test check sampled threads of a buffer too large
  * to hold on the host. */

@@ -181,3 +181,87 @@ def fill_e4m3(n, seed, stream, dist, scale, first=0):
     out = np.empty(n, dtype=np.uint8)
     _bind_builders().orc_fill_e4m3(out.ctypes.data, n, seed, stream, dist, scale, first)
     return out
+
+
+def global_bandwidth_range(width, data, T, t0, t1, out=None):
+    data = np.ascontiguousarray(data, dtype=np.float32)
+    if out is None:
+        out = np.zeros(T, dtype=np.float32)
+    L = lib()
+    L.orc_global_bandwidth_range.argtypes = [C.c_int, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_void_p]
+    L.orc_global_bandwidth_range.restype = None
+    L.orc_global_bandwidth_range(width, data.ctypes.data, data.size, T, t0, t1, out.ctypes.data)
+    return out
+
+
+# --- CPU baseline harness (cpu_harness.c) -----------------------------------------------------------
+CPUH_READ_FLOAT4, CPUH_MAD_F32, CPUH_MFMA_BF16, CPUH_MFMA_I8, CPUH_GEMM_BF16 = range(5)
+
+
+class CpuhResult(C.Structure):
+    _fields_ = [("us_st", C.c_double), ("us_mt", C.c_double), ("iters_st", C.c_uint), ("iters_mt", C.c_uint),
+                ("threads_mt", C.c_int), ("pinned", C.c_int), ("units_per_iter_st", C.c_double),
+                ("units_per_iter_mt", C.c_double), ("giga_st", C.c_double), ("giga_mt", C.c_double)]
+
+
+def _bind_harness():
+    L = lib()
+    if getattr(L, "_harness_bound", False):
+        return L
+    vp, u64, u32, i32, dbl = C.c_void_p, C.c_uint64, C.c_uint, C.c_int, C.c_double
+    L.cpuh_pool_create.argtypes = [i32]; L.cpuh_pool_create.restype = vp
+    L.cpuh_pool_destroy.argtypes = [vp]; L.cpuh_pool_destroy.restype = None
+    L.cpuh_pool_max_threads.argtypes = [vp]; L.cpuh_pool_max_threads.restype = i32
+    L.cpuh_pool_pinned_cpu.argtypes = [vp, i32]; L.cpuh_pool_pinned_cpu.restype = i32
+    L.cpuh_pool_count.argtypes = [vp, i32, u64, vp]; L.cpuh_pool_count.restype = None
+    L.cpuh_pick_iters.argtypes = [dbl, u32, u32, u32]; L.cpuh_pick_iters.restype = u32
+    L.cpuh_time_sleep_body.argtypes = [vp, i32, u32, u32, C.POINTER(u32)]; L.cpuh_time_sleep_body.restype = dbl
+    L.cpuh_measure.argtypes = [vp, i32, u64, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure.restype = i32
+    L._harness_bound = True
+    return L
+
+
+class CpuPool:
+    """Persistent pinned worker pool of the CPU baseline harness."""
+
+    def __init__(self, max_threads=None):
+        self.L = _bind_harness()
+        self.max_threads = max_threads or len(os.sched_getaffinity(0))
+        self.h = self.L.cpuh_pool_create(self.max_threads)
+        if not self.h:
+            raise MemoryError("cpuh_pool_create failed")
+
+    def close(self):
+        if self.h:
+            self.L.cpuh_pool_destroy(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def pinned_cpu(self, tid):
+        return self.L.cpuh_pool_pinned_cpu(self.h, tid)
+
+    def count(self, n, iters):
+        counts = np.zeros(self.max_threads, dtype=np.uint64)
+        self.L.cpuh_pool_count(self.h, n, iters, counts.ctypes.data)
+        return counts
+
+    def time_sleep_body(self, n_threads, sleep_us, target_us):
+        iters = C.c_uint(0)
+        us = self.L.cpuh_time_sleep_body(self.h, n_threads, sleep_us, target_us, C.byref(iters))
+        return us, iters.value
+
+    def measure(self, kind, seed, warmup=2, target_us=2_000_000):
+        r = CpuhResult()
+        rc = self.L.cpuh_measure(self.h, kind, seed, warmup, target_us, C.byref(r))
+        if rc != 0:
+            raise RuntimeError(f"cpuh_measure({kind}) failed: {rc}")
+        return r
+
+
+def pick_iters(per_iter_us, target_us, forced, max_iters):
+    return _bind_harness().cpuh_pick_iters(per_iter_us, target_us, forced, max_iters)

@@ -1,0 +1,96 @@
+"""CPU baseline harness: pool, timing discipline, ST/MT accounting.
+
+The harness restates src/cpu/thread_pool.cpp:23-102 (pool), src/cpu/cpu_peak.cpp:46-128
+(run_workload), src/common/common.cpp:35-45 (pick_iters) and src/cpu/compute_common.h:21-60 (ST/MT
+values) of the reference.  These tests pin it against what those sources fix: the clamp rules of
+pick_iters at their documented corners, a body of known duration, the dispatch contract of the pool
+(exactly workers 0..n-1 run, each once), and the giga-unit formula.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+from oracle import workloads as wl
+
+
+@pytest.fixture(scope="module")
+def pool():
+    p = orc.CpuPool(min(4, len(os.sched_getaffinity(0))))
+    yield p
+    p.close()
+
+
+@pytest.mark.parametrize("per_iter, target, forced, cap, want", [
+    (10.0, 1000, 0, 10000, 100),          # target / per-iteration time
+    (0.01, 1000, 0, 10000, 1000),         # per-iteration time floors at 1 us
+    (1.0, 0, 0, 100000000, 5000000),      # target 0 means the 5 s legacy default
+    (1.0, 10**9, 0, 10000, 10000),        # clamp to the cap
+    (5000.0, 1000, 0, 10000, 1),          # never below one iteration
+    (123.0, 1000, 77, 10000, 77),         # forced wins over everything
+    (3.0, 1000, 0, 10000, 333),           # truncation, not rounding
+])
+def test_pick_iters_corners(per_iter, target, forced, cap, want):
+    assert orc.pick_iters(per_iter, target, forced, cap) == want
+
+
+def test_pool_runs_exactly_the_first_n_workers(pool):
+    for n in range(1, pool.max_threads + 1):
+        counts = pool.count(n, 7)
+        want = np.array([(t + 1) * 7 if t < n else 0 for t in range(pool.max_threads)], dtype=np.uint64)
+        assert (counts == want).all(), (n, counts)
+    # n outside [1, max] is clamped, as the reference's run() does
+    assert pool.count(0, 1)[0] == 1
+    assert (pool.count(pool.max_threads + 5, 1) > 0).all()
+
+
+def test_workers_are_pinned_to_their_own_cpu(pool):
+    pool.count(pool.max_threads, 1)  # every worker has started once this returns
+    allowed = os.sched_getaffinity(0)
+    for t in range(pool.max_threads):
+        got = pool.pinned_cpu(t)
+        if t in allowed:
+            assert got == t
+        else:
+            assert got in (t, -1)   # pinning outside the allowed set may be refused: best effort
+
+
+def test_run_workload_recovers_a_known_iteration_time(pool):
+    # a body that sleeps 500 us per iteration: the probe must grow past one iteration (2 ms rule), the
+    # batch must be sized for the 100 ms budget, and the mean must come back near 500 us (sleep overshoots)
+    for n in (1, pool.max_threads):
+        us, iters = pool.time_sleep_body(n, 500, 100_000)
+        assert 500.0 <= us < 900.0, us
+        assert 100_000 / 900.0 <= iters <= 100_000 / 500.0 + 1, iters
+
+
+def test_ranged_read_reduce_is_the_same_sum():
+    n, T = 1 << 18, 1 << 10
+    data = orc.fill_f32(n, wl.DEFAULT_SEED, wl.STREAM_BW, 0)
+    for width in (1, 2, 4):
+        whole = orc.global_bandwidth(width, data, T)
+        parts = np.zeros(T, dtype=np.float32)
+        for t0, t1 in ((0, 100), (100, 101), (101, 777), (777, T)):
+            orc.global_bandwidth_range(width, data, T, t0, t1, parts)
+        assert (parts.view(np.uint32) == whole.view(np.uint32)).all()
+    # ragged tail: the last stride is only partly filled
+    data = data[: n - 4 * 300]
+    whole = orc.global_bandwidth(4, data, T)
+    parts = np.zeros(T, dtype=np.float32)
+    orc.global_bandwidth_range(4, data, T, 0, 512, parts)
+    orc.global_bandwidth_range(4, data, T, 512, T, parts)
+    assert (parts.view(np.uint32) == whole.view(np.uint32)).all()
+
+
+def test_measure_reports_st_and_mt_in_giga_units(pool):
+    r = pool.measure(orc.CPUH_MAD_F32, wl.DEFAULT_SEED, warmup=1, target_us=50_000)
+    assert r.threads_mt == pool.max_threads
+    assert r.iters_st >= 1 and r.iters_mt >= 1
+    # one iteration = 8 items x 16 accumulators x 4096 fma x 2 flops
+    assert r.units_per_iter_st == 8 * 16 * 4096 * 2
+    assert r.giga_st == pytest.approx(r.units_per_iter_st / (r.us_st * 1e3))
+    assert r.giga_mt == pytest.approx(r.units_per_iter_mt * r.threads_mt / (r.us_mt * 1e3))
+    assert 0.05 < r.giga_st < 1000.0          # a scalar fma chain on any x86 core of this decade
+    with pytest.raises(RuntimeError):
+        pool.measure(99, 1)
