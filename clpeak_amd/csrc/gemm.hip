@@ -267,83 +267,171 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, u
     }
 }
 
-// fp8 e4m3 variant: one K=128 MFMA step per slab, compiler-scheduled.
-__device__ inline uint32_t swizzled(uint32_t row, uint32_t chunk) {
-  return row * kRowBytes + ((chunk ^ (row & 7u)) << 4);
+// ---- fp8 e4m3 ------------------------------------------------------------------------------------
+// Same tiling, LDS layout, loads and barrier discipline as above; a slab of 128 bytes per row is
+// exactly one K=128 matrix instruction per 16x16 tile, 32 instructions of 32 cycles per wave and step.
+// A lane's 32-byte operand is the two 16-byte chunks g and g+4 of its row (g = lane/16), which in
+// the swizzled layout are the addresses x and x^64: two ds_read_b128 fill the low and the high half
+// of the 8-register operand.
+//
+// There are no spare registers for a second set of fragments (128 accumulators + 96 fragment
+// registers), so fragments are reloaded in place as soon as their last use has issued.  The 32
+// instructions run as two sweeps over the 8 A fragments, first against B fragments 0,1 and then
+// against 2,3:
+//     MFMA  0..9    (i,0),(i,1): this step's A fragment 7 and B fragments 2,3 are read in gaps 0..2;
+//                   counted waits let row i start as soon as its own fragment has arrived
+//     wait all reads; wait own global loads; barrier    <- slab s+1 complete, slab s free
+//     MFMA 10..15   six of the wave's 8 global->LDS loads of slab s+2 (the other two in gaps 18, 20)
+//     MFMA 16..31   (i,2),(i,3): next step's B fragments 0,1 in gaps 16,17, next step's A fragment
+//                   i-1 after row i (a fragment is overwritten no sooner than one instruction after
+//                   its last use)
+#define MI355_MFMA_FP8(acc, blo, bhi, alo, ahi)                                                    \
+  do {                                                                                             \
+    const i32x8v b8_ = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7);                  \
+    const i32x8v a8_ = __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);                  \
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(acc) : "v"(b8_), "v"(a8_));   \
+  } while (0)
+
+// At most `n` LDS reads still outstanding (they return in order).
+#define MI355_WAIT_LGKM(n) asm volatile("s_waitcnt lgkmcnt(" #n ")" ::: "memory")
+
+struct Fp8Frags {
+  i32x4v a_lo[8], a_hi[8], b_lo[4], b_hi[4];
+};
+
+template <bool MAIN>
+__device__ __forceinline__ void gemm_fp8_step(f32x4v (&acc)[8][4], Fp8Frags &f, const GemmWalk &w, bool reads,
+                                              bool loads) {
+  const bool READS = MAIN || reads, LOADS = MAIN || loads;
+  const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u, an_hi = w.a_nxt ^ 64u, bn_hi = w.b_nxt ^ 64u;
+#define MM(i, j) MI355_MFMA_FP8(acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i])
+#define LDA(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst + (q) * 1024u)
+#define LDB(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst + kSlabBytes + (q) * 1024u)
+#define RD_A_NEXT(i, off)                                                                          \
+  if (READS) { MI355_DS_READ(f.a_lo[i], w.a_nxt, off); MI355_DS_READ(f.a_hi[i], an_hi, off); }
+#define RD_B_NEXT(j, off)                                                                          \
+  if (READS) { MI355_DS_READ(f.b_lo[j], w.b_nxt, off); MI355_DS_READ(f.b_hi[j], bn_hi, off); }
+  // On entry the reads of B fragments 0,1 and A fragments 0..6 of this step are in flight, in that order.
+  MI355_WAIT_LGKM(12);                                   // B0, B1, A0 have arrived
+  MM(0, 0); MI355_DS_READ(f.a_lo[7], w.a_cur, 14336); MI355_DS_READ(f.a_hi[7], a_hi, 14336);
+  MM(0, 1); MI355_DS_READ(f.b_lo[2], w.b_cur, 4096); MI355_DS_READ(f.b_hi[2], b_hi, 4096);
+  MI355_WAIT_LGKM(14);                                   // A1
+  MM(1, 0); MI355_DS_READ(f.b_lo[3], w.b_cur, 6144); MI355_DS_READ(f.b_hi[3], b_hi, 6144);
+  MM(1, 1);
+  MI355_WAIT_LGKM(14);                                   // A2
+  MM(2, 0); MM(2, 1);
+  MI355_WAIT_LGKM(12);                                   // A3
+  MM(3, 0); MM(3, 1);
+  MI355_WAIT_LGKM(10);                                   // A4
+  MM(4, 0); MM(4, 1);
+  // every read of this step's slab has returned (its buffer is free) and this wave's share of the
+  // next slab has landed
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier" ::: "memory");
+  MM(5, 0); LDA(0);
+  MM(5, 1); LDB(0);
+  MM(6, 0); LDA(1);
+  MM(6, 1); LDB(1);
+  MM(7, 0); LDA(2);
+  MM(7, 1); LDB(2);
+  MM(0, 2); RD_B_NEXT(0, 0);
+  MM(0, 3); RD_B_NEXT(1, 2048);
+  MM(1, 2); LDA(3);
+  MM(1, 3); RD_A_NEXT(0, 0);
+  MM(2, 2); LDB(3);
+  MM(2, 3); RD_A_NEXT(1, 2048);
+  MM(3, 2);
+  MM(3, 3); RD_A_NEXT(2, 4096);
+  MM(4, 2);
+  MM(4, 3); RD_A_NEXT(3, 6144);
+  MM(5, 2);
+  MM(5, 3); RD_A_NEXT(4, 8192);
+  MM(6, 2);
+  MM(6, 3); RD_A_NEXT(5, 10240);
+  MM(7, 2);
+  MM(7, 3); RD_A_NEXT(6, 12288);
+#undef RD_A_NEXT
+#undef RD_B_NEXT
+#undef LDA
+#undef LDB
+#undef MM
 }
 
 __global__ void __launch_bounds__(kThreads)
 gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, uint16_t *__restrict__ C,
                 uint32_t N, uint32_t k_bytes, float scale, uint32_t tiles_m, uint32_t tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-  const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const uint32_t tid = threadIdx.x, lane = tid % 64;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const uint32_t wm = wave / 4, wn = wave % 4;
   uint32_t tm, tn;
   tile_of_block(tiles_m, tiles_n, tm, tn);
-  const uint8_t *a_tile = A + (size_t)tm * kTile * k_bytes;
-  const uint8_t *b_tile = B + (size_t)tn * kTile * k_bytes;
+
+  // global -> LDS, exactly as in the bf16 kernel (rows are 128 bytes in both)
+  const uint32_t lrow = wave * 32u + lane / 8u, lchunk = (lane % 8u) ^ (lane / 8u);
+  const uint8_t *ga = A + ((size_t)tm * kTile + lrow) * k_bytes + lchunk * 16u;
+  const uint8_t *gb = B + ((size_t)tn * kTile + lrow) * k_bytes + lchunk * 16u;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+  const uint32_t dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 4096u);
+  auto fetch_slab = [&](uint32_t step, uint32_t buf) {
+    const size_t kb = (size_t)step * kRowBytes;
+    const uint32_t dst = dst_wave + buf * kBufBytes;
+#pragma unroll
+    for (uint32_t q = 0; q < 4; q++) {
+      load_to_lds(ga + kb + (size_t)q * 8u * k_bytes, dst + q * 1024u);
+      load_to_lds(gb + kb + (size_t)q * 8u * k_bytes, dst + kSlabBytes + q * 1024u);
+    }
+  };
+
+  // LDS -> fragments: chunk lane/16 of row lane%16 (low half of the operand); the high half is
+  // chunk lane/16 + 4, i.e. the address with bit 6 flipped.
+  const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
+  GemmWalk w;
+  w.a_cur = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
+  w.b_cur = lds_base + kSlabBytes + (wn * 64u + lane % 16u) * kRowBytes + swz0;
+  w.a_nxt = w.a_cur + kBufBytes;
+  w.b_nxt = w.b_cur + kBufBytes;
 
   f32x4v acc[8][4];
 #pragma unroll
   for (int i = 0; i < 8; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
-
-  constexpr int kChunksPerThread = kSlabBytes / 16 / kThreads;  // 4
-  i32x4v stage_a[kChunksPerThread], stage_b[kChunksPerThread];
-  auto global_fetch = [&](uint32_t kb) {
-#pragma unroll
-    for (int i = 0; i < kChunksPerThread; i++) {
-      const uint32_t q = tid + kThreads * i, row = q / 8u, c = q % 8u;
-      stage_a[i] = *reinterpret_cast<const i32x4v *>(a_tile + (size_t)row * k_bytes + kb + c * 16u);
-      stage_b[i] = *reinterpret_cast<const i32x4v *>(b_tile + (size_t)row * k_bytes + kb + c * 16u);
-    }
-  };
-  auto lds_commit = [&](uint32_t buf) {
-    uint8_t *sa = lds + (size_t)buf * kBufBytes, *sb = sa + kSlabBytes;
-#pragma unroll
-    for (int i = 0; i < kChunksPerThread; i++) {
-      const uint32_t q = tid + kThreads * i, row = q / 8u, c = q % 8u;
-      *reinterpret_cast<i32x4v *>(sa + swizzled(row, c)) = stage_a[i];
-      *reinterpret_cast<i32x4v *>(sb + swizzled(row, c)) = stage_b[i];
-    }
-  };
+  Fp8Frags f;
 
   const uint32_t steps = k_bytes / kRowBytes;
-  global_fetch(0);
-  lds_commit(0);
-  __syncthreads();
-
-  for (uint32_t s = 0; s < steps; s++) {
-    const uint32_t buf = s & 1u;
-    if (s + 1 < steps) global_fetch((s + 1) * kRowBytes);
-    const uint8_t *sa = lds + (size_t)buf * kBufBytes + (size_t)wm * 128 * kRowBytes;
-    const uint8_t *sb = lds + (size_t)buf * kBufBytes + kSlabBytes + (size_t)wn * 64 * kRowBytes;
-    // a lane's 32 codes are logical chunks 2*(lane/16) and 2*(lane/16)+1 (the same choice for
-    // A and B, which is all a dot product needs)
-    i32x8v bf[4];
-    const uint32_t c0 = 2u * (lane / 16u);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const uint32_t row = j * 16u + lane % 16u;
-      const i32x4v lo = *reinterpret_cast<const i32x4v *>(sb + swizzled(row, c0));
-      const i32x4v hi = *reinterpret_cast<const i32x4v *>(sb + swizzled(row, c0 + 1u));
-      bf[j] = (i32x8v){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    }
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const uint32_t row = i * 16u + lane % 16u;
-      const i32x4v lo = *reinterpret_cast<const i32x4v *>(sa + swizzled(row, c0));
-      const i32x4v hi = *reinterpret_cast<const i32x4v *>(sa + swizzled(row, c0 + 1u));
-      const i32x8v af = (i32x8v){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af, acc[i][j], MI355_F8F6F4_E4M3,
-                                                                       MI355_F8F6F4_E4M3, 0, 0x7f, 0, 0x7f);
-    }
-    if (s + 1 < steps) lds_commit(buf ^ 1u);
-    __syncthreads();
+  fetch_slab(0, 0);
+  if (steps > 1) fetch_slab(1, 1);
+  asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+  // what a step expects in flight on entry: B fragments 0,1 then A fragments 0..6
+  {
+    const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u;
+    MI355_DS_READ(f.b_lo[0], w.b_cur, 0); MI355_DS_READ(f.b_hi[0], b_hi, 0);
+    MI355_DS_READ(f.b_lo[1], w.b_cur, 2048); MI355_DS_READ(f.b_hi[1], b_hi, 2048);
+    MI355_DS_READ(f.a_lo[0], w.a_cur, 0); MI355_DS_READ(f.a_hi[0], a_hi, 0);
+    MI355_DS_READ(f.a_lo[1], w.a_cur, 2048); MI355_DS_READ(f.a_hi[1], a_hi, 2048);
+    MI355_DS_READ(f.a_lo[2], w.a_cur, 4096); MI355_DS_READ(f.a_hi[2], a_hi, 4096);
+    MI355_DS_READ(f.a_lo[3], w.a_cur, 6144); MI355_DS_READ(f.a_hi[3], a_hi, 6144);
+    MI355_DS_READ(f.a_lo[4], w.a_cur, 8192); MI355_DS_READ(f.a_hi[4], a_hi, 8192);
+    MI355_DS_READ(f.a_lo[5], w.a_cur, 10240); MI355_DS_READ(f.a_hi[5], a_hi, 10240);
+    MI355_DS_READ(f.a_lo[6], w.a_cur, 12288); MI355_DS_READ(f.a_hi[6], a_hi, 12288);
   }
+
+  w.voff = (lane / 8u) * k_bytes + lchunk * 16u;
+  w.row8 = 8u * k_bytes;
+  w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
+  w.gb = (uint64_t)(uintptr_t)(B + ((size_t)tn * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
+  w.dst = dst_wave;
+  auto advance = [&](uint32_t s) {
+    w.dst = dst_wave + ((s + 1) & 1u) * kBufBytes;
+    w.ga += kRowBytes;
+    w.gb += kRowBytes;
+    uint32_t t = w.a_cur; w.a_cur = w.a_nxt; w.a_nxt = t;
+    t = w.b_cur; w.b_cur = w.b_nxt; w.b_nxt = t;
+  };
+  uint32_t s = 0;
+  for (; s + 2 < steps; s++) { gemm_fp8_step<true>(acc, f, w, true, true); advance(s); }
+  for (; s < steps; s++) { gemm_fp8_step<false>(acc, f, w, s + 1 < steps, false); advance(s); }
+  asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
   const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 64u + 4u * (lane / 16u);
 #pragma unroll
