@@ -21,7 +21,8 @@
 //
 // Schedule of one step: 64 MFMAs per wave, 32 on fragment set F0 (first K half of the slab) then
 // 32 on F1 (second half); never more than one memory instruction between two MFMAs:
-//     MFMA  0..12   one LDS read of F1 in each of the first 12 gaps
+//     MFMA  0..12   the 12 LDS reads of F1, two in each of the first 6 gaps (a 128-bit read takes
+//                   about 8 cycles to issue, two fit in the 16-cycle shadow of an MFMA)
 //     wait F1; wait own global loads; barrier      <- slab s+1 complete, slab s free
 //     MFMA 13..39   the wave's 8 global->LDS loads of slab s+2, one every third MFMA
 //     MFMA 40..63   one LDS read of the next step's F0 in each of the first 12 gaps
@@ -113,19 +114,15 @@ __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8]
 #define LDA(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst + (q) * 1024u)
 #define LDB(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst + kSlabBytes + (q) * 1024u)
   bf16x8v(&x0a_)[8] = fa0; bf16x8v(&x0b_)[4] = fb0; bf16x8v(&x1a_)[8] = fa1; bf16x8v(&x1b_)[4] = fb1;
-  // ---- MFMAs 0..12 (on F0); the 12 reads of F1 in the first 12 gaps -----------------------------
-  MM(x0, 0, 0); MI355_DS_READ(fb1[0], b1, 0);
-  MM(x0, 0, 1); MI355_DS_READ(fb1[1], b1, 2048);
-  MM(x0, 0, 2); MI355_DS_READ(fb1[2], b1, 4096);
-  MM(x0, 0, 3); MI355_DS_READ(fb1[3], b1, 6144);
-  MM(x0, 1, 0); MI355_DS_READ(fa1[0], a1, 0);
-  MM(x0, 1, 1); MI355_DS_READ(fa1[1], a1, 2048);
-  MM(x0, 1, 2); MI355_DS_READ(fa1[2], a1, 4096);
-  MM(x0, 1, 3); MI355_DS_READ(fa1[3], a1, 6144);
-  MM(x0, 2, 0); MI355_DS_READ(fa1[4], a1, 8192);
-  MM(x0, 2, 1); MI355_DS_READ(fa1[5], a1, 10240);
-  MM(x0, 2, 2); MI355_DS_READ(fa1[6], a1, 12288);
-  MM(x0, 2, 3); MI355_DS_READ(fa1[7], a1, 14336);
+  // ---- MFMAs 0..12 (on F0); the 12 reads of F1 in the first 6 gaps ------------------------------
+  MM(x0, 0, 0); MI355_DS_READ(fb1[0], b1, 0); MI355_DS_READ(fb1[1], b1, 2048);
+  MM(x0, 0, 1); MI355_DS_READ(fb1[2], b1, 4096); MI355_DS_READ(fb1[3], b1, 6144);
+  MM(x0, 0, 2); MI355_DS_READ(fa1[0], a1, 0); MI355_DS_READ(fa1[1], a1, 2048);
+  MM(x0, 0, 3); MI355_DS_READ(fa1[2], a1, 4096); MI355_DS_READ(fa1[3], a1, 6144);
+  MM(x0, 1, 0); MI355_DS_READ(fa1[4], a1, 8192); MI355_DS_READ(fa1[5], a1, 10240);
+  MM(x0, 1, 1); MI355_DS_READ(fa1[6], a1, 12288); MI355_DS_READ(fa1[7], a1, 14336);
+  MM(x0, 1, 2); MM(x0, 1, 3);
+  MM(x0, 2, 0); MM(x0, 2, 1); MM(x0, 2, 2); MM(x0, 2, 3);
   MM(x0, 3, 0);
   MI355_WAIT_FRAGS(fa1, fb1);
   // every wave holds all fragments of this step's slab (its buffer is free) and every wave's
