@@ -20,10 +20,12 @@ SYMBOLS = [
     "mi355_global_bandwidth", "mi355_compute_mad", "mi355_launch_roundtrip",
     "mi355_mfma_dense", "mi355_smfmac", "mi355_mfma_raw",
     "mi355_gemm_bf16", "mi355_gemm_fp8_e4m3",
+    "mi355_local_bandwidth", "mi355_host_alloc", "mi355_host_free", "mi355_copy_async",
 ]
 
 OK, ERR_ARG, ERR_HIP, ERR_NODEV, ERR_ARCH, ERR_OOM = 0, -1, -2, -3, -4, -5
 DIST_U01, DIST_UPM1 = 0, 1
+H2D, D2H = 0, 1
 MAD_F32, MAD_F16, MAD_F64, MAD_MP, MAD_BF16, MAD_I32, MAD_I8DP = range(7)
 (MFMA_F16_16x16x32, MFMA_BF16_16x16x32, MFMA_F16_32x32x16, MFMA_BF16_32x32x16, MFMA_I8_16x16x64,
  MFMA_FP8_16x16x128, MFMA_BF8_16x16x128, MFMA_MXFP6_E2M3, MFMA_MXFP6_E3M2, MFMA_MXFP4_E2M1) = range(10)
@@ -80,6 +82,10 @@ def load_library(path=LIB_PATH):
     lib.mi355_mfma_raw.argtypes = [vp, i32, i32, vp, vp, vp, vp, vp, i32, i32, vp]
     lib.mi355_gemm_bf16.argtypes = [vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_gemm_fp8_e4m3.argtypes = [vp, vp, vp, vp, u32, u32, u32, C.c_float, C.c_float]
+    lib.mi355_local_bandwidth.argtypes = [vp, i32, vp, u32, u32, u32]
+    lib.mi355_host_alloc.argtypes = [vp, C.c_size_t, C.POINTER(vp)]
+    lib.mi355_host_free.argtypes = [vp, vp]
+    lib.mi355_copy_async.argtypes = [vp, vp, vp, C.c_size_t, i32]
     for name in SYMBOLS:
         if name != "mi355_last_error":
             getattr(lib, name).restype = C.c_int
@@ -185,6 +191,23 @@ class Device:
 
     def compute_mad(self, kind, width, seed, n_items, steps, outbuf, block_size=256):
         self._check(self.lib.mi355_compute_mad(self.h, kind, width, seed, n_items, steps, outbuf.ptr, block_size))
+
+    def local_bandwidth(self, width, outbuf, blocks, block_size=256, reps=64):
+        self._check(self.lib.mi355_local_bandwidth(self.h, width, outbuf.ptr, blocks, block_size, reps))
+
+    def host_alloc(self, nbytes):
+        """Pinned host buffer as a numpy uint8 array (free it with host_free)."""
+        import numpy as np
+        p = C.c_void_p()
+        self._check(self.lib.mi355_host_alloc(self.h, nbytes, C.byref(p)))
+        arr = np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), shape=(nbytes,))
+        return arr, p
+
+    def host_free(self, handle):
+        self._check(self.lib.mi355_host_free(self.h, handle))
+
+    def copy_async(self, dst_ptr, src_ptr, nbytes, direction):
+        self._check(self.lib.mi355_copy_async(self.h, dst_ptr, src_ptr, nbytes, direction))
 
     def launch_roundtrip(self, warmup, launches):
         us = C.c_double()

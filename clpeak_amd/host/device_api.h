@@ -28,6 +28,10 @@ struct Mi355Api {
   decltype(&mi355_smfmac) smfmac;
   decltype(&mi355_gemm_bf16) gemm_bf16;
   decltype(&mi355_gemm_fp8_e4m3) gemm_fp8_e4m3;
+  decltype(&mi355_local_bandwidth) local_bandwidth;
+  decltype(&mi355_host_alloc) host_alloc;
+  decltype(&mi355_host_free) host_free;
+  decltype(&mi355_copy_async) copy_async;
 };
 
 const Mi355Api &mi355_real_api();   // the entry points of libclpeak_mi355.so

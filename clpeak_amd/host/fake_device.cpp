@@ -70,12 +70,21 @@ int f_mfma_dense(mi355_dev *d, int, const void *, const void *, const uint8_t *,
 int f_smfmac(mi355_dev *d, int, const void *, const uint8_t *, const void *, void *, uint32_t, uint32_t, uint64_t *) { FAKE_ENTRY(d, "smfmac"); return MI355_OK; }
 int f_gemm_bf16(mi355_dev *d, const uint16_t *, const uint16_t *, uint16_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_bf16"); return MI355_OK; }
 int f_gemm_fp8(mi355_dev *d, const uint8_t *, const uint8_t *, uint16_t *, uint32_t, uint32_t, uint32_t, float, float) { FAKE_ENTRY(d, "gemm_fp8_e4m3"); return MI355_OK; }
+int f_local_bandwidth(mi355_dev *d, int, float *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "local_bandwidth"); return MI355_OK; }
+int f_host_alloc(mi355_dev *d, size_t bytes, void **p) {
+  FAKE_ENTRY(d, "host_alloc");
+  *p = malloc(bytes);
+  return *p ? MI355_OK : MI355_ERR_OOM;
+}
+int f_host_free(mi355_dev *, void *p) { free(p); return MI355_OK; }
+int f_copy_async(mi355_dev *d, void *, const void *, size_t, int) { FAKE_ENTRY(d, "copy_async"); return MI355_OK; }
 }  // namespace
 
 const Mi355Api &mi355_fake_api() {
   static const Mi355Api api = {
       f_device_count, f_open, f_close, f_get_props, f_last_error, f_alloc, f_free, f_upload, f_download, f_sync,
       f_timer_start, f_timer_stop, f_fill_f32, f_fill_bf16, f_fill_fp8, f_global_bandwidth, f_compute_mad,
-      f_launch_roundtrip, f_mfma_dense, f_smfmac, f_gemm_bf16, f_gemm_fp8};
+      f_launch_roundtrip, f_mfma_dense, f_smfmac, f_gemm_bf16, f_gemm_fp8,
+      f_local_bandwidth, f_host_alloc, f_host_free, f_copy_async};
   return api;
 }

@@ -88,6 +88,7 @@ int main(int argc, char **argv) {
     else if (a == "--small-shapes") {
       shape.madItems = 1 << 12; shape.madSteps = 64; shape.bwFloats = 1 << 22; shape.mfmaWavesPerCU = 1;
       shape.mfmaIters = 32; shape.gemmDim = 512; shape.latencyLaunches = 50;
+      shape.ldsThreads = 1 << 16; shape.transferBytes = 1 << 22;
     } else if (a.compare(0, 2, "--") == 0) {
       const bool neg = a.compare(0, 5, "--no-") == 0;
       const std::string name = a.substr(neg ? 5 : 2);

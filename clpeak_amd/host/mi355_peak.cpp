@@ -195,15 +195,11 @@ void Mi355Peak::runDevice(int ordinal, logger::BackendScope &backend) {
   if (isAllowedAs(Benchmark::Rocblas, Category::IntCompute)) runGemmInt();
   // bandwidth and latency
   if (isAllowed(Benchmark::GlobalBW)) runGlobalBandwidth();
-  if (isAllowed(Benchmark::LocalBW))
-    runNotBuilt("local_memory_bandwidth", "Local memory bandwidth", {"float", "float2", "float4"},
-                "Not built in the MI355X backend yet", ResultStatus::Skipped);
+  if (isAllowed(Benchmark::LocalBW)) runLocalBandwidth();
   if (isAllowed(Benchmark::ImageBW))
     runNotBuilt("image_memory_bandwidth", "Image memory bandwidth", {"float4"},
                 "Device has no image/texture support", ResultStatus::Unsupported);
-  if (isAllowed(Benchmark::TransferBW))
-    runNotBuilt("transfer_bandwidth", "Transfer bandwidth", {"h2d_pinned", "d2h_pinned"},
-                "Not built in the MI355X backend yet", ResultStatus::Skipped);
+  if (isAllowed(Benchmark::TransferBW)) runTransferBandwidth();
   if (isAllowed(Benchmark::KernelLatency)) runKernelLatency(cfg);
 
   device_ = nullptr;
@@ -459,6 +455,65 @@ void Mi355Peak::runGlobalBandwidth() {
     if (us <= 0.0f) test.skip(v.metric, ResultStatus::Error, "kernel launch failed", widthNote(v.width));
     else test.emit(v.metric, (float)((double)n * sizeof(float) / us / 1e3), widthNote(v.width));
   }
+}
+
+// LDS ping-pong, the reference's shape: 256 threads per workgroup, 64 repetitions, grid sized by
+// targetGlobalThreads (include/common/common.h:142-147); bytes = reps * 2 * width * 4 * threads
+// (src/rocm/local_bandwidth.cpp:63-65).
+void Mi355Peak::runLocalBandwidth() {
+  auto test = device_->beginTest({"local_memory_bandwidth", "Local memory bandwidth", "gbps", Category::Unknown,
+                                  "How many bytes per second the GPU moves through shared local memory (LDS), the "
+                                  "on-chip scratchpad a workgroup passes data through."});
+  static const struct { const char *metric; int width; } variants[] = {{"float", 1}, {"float2", 2}, {"float4", 4}};
+  const uint32_t bs = 256, reps = 64;
+  uint64_t threads = workload.ldsThreads;
+  if (threads == 0) threads = std::max<uint64_t>(32ull << 20, (uint64_t)props_.num_cus * 2048ull * 256ull);
+  const uint32_t blocks = (uint32_t)(threads / bs);
+  threads = (uint64_t)blocks * bs;
+  Buffer out(api_, dev_, threads * sizeof(float));
+  for (const auto &v : variants) {
+    if (!out) {
+      test.skip(v.metric, ResultStatus::Error, "Buffer alloc failed", widthNote(v.width));
+      continue;
+    }
+    const float us = runKernel([&] { return api_.local_bandwidth(dev_, v.width, (float *)out.ptr, blocks, bs, reps); },
+                               targetTimeUs, forceIters ? specifiedIters : 0);
+    if (us <= 0.0f) test.skip(v.metric, ResultStatus::Error, "kernel launch failed", widthNote(v.width));
+    else test.emit(v.metric, (float)((double)reps * 2.0 * v.width * sizeof(float) * (double)threads / us / 1e3), widthNote(v.width));
+  }
+}
+
+// Pinned host buffer <-> device buffer over PCIe, both directions, each timed like a kernel: warm-up
+// copies, a one-copy probe, a batch sized to the time budget between two events
+// (src/rocm/transfer_bandwidth.cpp:42-103).
+void Mi355Peak::runTransferBandwidth() {
+  auto test = device_->beginTest({"transfer_bandwidth", "Transfer bandwidth", "gbps", Category::Unknown,
+                                  "How fast data crosses between host memory and the card over the PCIe link; both "
+                                  "readings use pinned host memory."});
+  const char *h2dNote = "Host to device: sending data up to the card.";
+  const char *d2hNote = "Device to host: reading results back down.";
+  const size_t bytes = (size_t)workload.transferBytes;
+  Buffer dbuf(api_, dev_, bytes);
+  void *pinned = nullptr;
+  if (!dbuf) {
+    test.skip("h2d_pinned", ResultStatus::Error, "Failed to allocate device buffer", h2dNote);
+    test.skip("d2h_pinned", ResultStatus::Error, "Failed to allocate device buffer", d2hNote);
+    return;
+  }
+  if (api_.host_alloc(dev_, bytes, &pinned) != MI355_OK) {
+    test.skip("h2d_pinned", ResultStatus::Error, "Failed to allocate pinned host buffer", h2dNote);
+    test.skip("d2h_pinned", ResultStatus::Error, "Failed to allocate pinned host buffer", d2hNote);
+    return;
+  }
+  seeded_uniform_f32((float *)pinned, bytes / sizeof(float), workload.seed, MI355_STREAM_BW);
+  const unsigned forced = forceIters ? specifiedIters : 0;
+  const float usH2D = runKernel([&] { return api_.copy_async(dev_, dbuf.ptr, pinned, bytes, MI355_H2D); }, targetTimeUs, forced);
+  if (usH2D > 0.0f) test.emit("h2d_pinned", (float)((double)bytes / usH2D / 1e3), h2dNote);
+  else test.skip("h2d_pinned", ResultStatus::Error, "transfer failed", h2dNote);
+  const float usD2H = runKernel([&] { return api_.copy_async(dev_, pinned, dbuf.ptr, bytes, MI355_D2H); }, targetTimeUs, forced);
+  if (usD2H > 0.0f) test.emit("d2h_pinned", (float)((double)bytes / usD2H / 1e3), d2hNote);
+  else test.skip("d2h_pinned", ResultStatus::Error, "transfer failed", d2hNote);
+  api_.host_free(dev_, pinned);
 }
 
 void Mi355Peak::runNotBuilt(const char *tag, const char *display, std::initializer_list<std::string> metrics, const char *why,

@@ -36,6 +36,8 @@ class Mi355Peak : public Peak {
     uint32_t mfmaIters = 4096;
     uint32_t gemmDim = 8192;
     uint32_t latencyLaunches = 10000;
+    uint64_t ldsThreads = 0;              // 0: the reference's rule, max(32M, CUs * 2048 * 256)
+    uint64_t transferBytes = 1ull << 29;  // pinned staging buffer of the transfer test
   } workload;
 
  private:
@@ -58,6 +60,8 @@ class Mi355Peak : public Peak {
   void runGemmFp8();
   void runGemmInt();
   void runGlobalBandwidth();
+  void runLocalBandwidth();
+  void runTransferBandwidth();
   void runNotBuilt(const char *tag, const char *display, std::initializer_list<std::string> metrics, const char *why,
                    ResultStatus status);
   void runKernelLatency(const benchmark_config_t &cfg);

@@ -62,6 +62,10 @@ double seeded_normal(uint64_t seed, uint32_t stream, uint64_t i) {
   return std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586476925286766559 * u2);
 }
 
+void seeded_uniform_f32(float *dst, uint64_t n, uint64_t seed, uint32_t stream) {
+  for (uint64_t i = 0; i < n; i++) dst[i] = mi355_rng_u01(mi355_rng_word(seed, stream, i));
+}
+
 std::vector<uint8_t> seeded_operand(OperandFormat f, double sigma, uint64_t seed, uint32_t stream, uint64_t n) {
   const int bits = operand_bits(f);
   std::vector<uint8_t> out((n * bits + 7) / 8, 0);

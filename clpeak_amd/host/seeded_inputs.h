@@ -19,6 +19,9 @@ std::vector<uint8_t> seeded_e8m0(uint64_t seed, uint32_t stream, uint64_t n);
 // 2:4 keep patterns: one byte per group of four, first kept position | second << 2, first < second.
 std::vector<uint8_t> seeded_sparse_meta(uint64_t seed, uint32_t stream, uint64_t n);
 
+// dst[i] = uniform [0,1) element i of `stream` (the values the device fill of the bandwidth buffer writes).
+void seeded_uniform_f32(float *dst, uint64_t n, uint64_t seed, uint32_t stream);
+
 // Round a double once to the narrow format; exported for tests.
 uint32_t encode_operand(OperandFormat f, double x);
 double seeded_normal(uint64_t seed, uint32_t stream, uint64_t i);

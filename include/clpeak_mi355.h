@@ -112,6 +112,29 @@ int mi355_copy(mi355_dev *dev, void *dst, const void *src, size_t bytes);
 int mi355_global_bandwidth(mi355_dev *dev, int width, const float *in, uint64_t n_floats,
                            float *out, uint32_t blocks, uint32_t block_size);
 
+/* ---- local (LDS) memory bandwidth --------------------------------------------- */
+/* Takes over local_bandwidth_v1/v2/v4 (src/rocm/rocm_kernels/local_bandwidth.hip:3-66)
+ * and their launch in runLocalBandwidth (src/rocm/local_bandwidth.cpp:6-75).  width in
+ * {1,2,4} floats per LDS access.  Thread gid starts from (float)gid [, gid+1 [, gid+2,
+ * gid+3]]; per repetition it stores its vector to slot lid of the workgroup's LDS array,
+ * barrier, loads slot (lid+1) % block_size, barrier.  out[gid] = x [+ y [+ z + w]] of
+ * what it holds after `reps` repetitions (the reference runs LMEM_REPS = 64,
+ * include/common/common.h:58, and 256 threads per block).  out holds
+ * blocks*block_size floats; block_size a multiple of 64 in [64,1024]. */
+int mi355_local_bandwidth(mi355_dev *dev, int width, float *out, uint32_t blocks,
+                          uint32_t block_size, uint32_t reps);
+
+/* ---- host <-> device transfer bandwidth --------------------------------------- */
+/* The pieces of runTransferBandwidth (src/rocm/transfer_bandwidth.cpp:6-122):
+ * hipHostMalloc / hipHostFree of the pinned staging buffer (:32-40, :118) and the
+ * hipMemcpyAsync on the device stream that its runBatch repeats between two events
+ * (:52-60).  copy_async only enqueues; time a batch with mi355_timer_start/stop. */
+#define MI355_H2D 0
+#define MI355_D2H 1
+int mi355_host_alloc(mi355_dev *dev, size_t bytes, void **hptr);
+int mi355_host_free(mi355_dev *dev, void *hptr);
+int mi355_copy_async(mi355_dev *dev, void *dst, const void *src, size_t bytes, int direction);
+
 /* ---- vector MAD compute ------------------------------------------------------- */
 /* Takes over the compute_* kernels (src/rocm/rocm_kernels/compute_sp.hip:18-70,
  * compute_hp.hip, compute_dp.hip, compute_mp.hip, compute_bf16.hip,

@@ -240,6 +240,33 @@ float orc_global_bandwidth_thread(int width, uint64_t seed, uint32_t stream, uin
 }
 
 /* ------------------------------------------------------------------------- */
+/* LDS ping-pong (src/rocm/rocm_kernels/local_bandwidth.hip:3-66 of the reference): per
+ * workgroup an array of block_size vectors; each repetition every thread stores its vector
+ * to its slot and then takes over the slot of its right-hand neighbour (cyclically).  The
+ * array is simulated literally, one workgroup at a time. */
+void orc_local_bandwidth(int width, uint32_t blocks, uint32_t block_size, uint32_t reps, float *out)
+{
+    float *slots = (float *)malloc((size_t)block_size * 4 * sizeof(float));
+    float *regs = (float *)malloc((size_t)block_size * 4 * sizeof(float));
+    for (uint32_t b = 0; b < blocks; b++) {
+        for (uint32_t l = 0; l < block_size; l++)
+            for (int c = 0; c < width; c++) regs[l * 4 + c] = (float)(b * block_size + l + (uint32_t)c);
+        for (uint32_t r = 0; r < reps; r++) {
+            memcpy(slots, regs, (size_t)block_size * 4 * sizeof(float));           /* store, barrier */
+            for (uint32_t l = 0; l < block_size; l++)                              /* load neighbour, barrier */
+                memcpy(regs + l * 4, slots + ((l + 1) % block_size) * 4, 4 * sizeof(float));
+        }
+        for (uint32_t l = 0; l < block_size; l++) {
+            float s = regs[l * 4];
+            for (int c = 1; c < width; c++) s = s + regs[l * 4 + c];
+            out[b * block_size + l] = s;
+        }
+    }
+    free(slots);
+    free(regs);
+}
+
+/* ------------------------------------------------------------------------- */
 /* Vector MAD chains                                                           */
 /* ------------------------------------------------------------------------- */
 enum { MAD_F32 = 0, MAD_F16 = 1, MAD_F64 = 2, MAD_MP = 3, MAD_BF16 = 4, MAD_I32 = 5, MAD_I8DP = 6 };

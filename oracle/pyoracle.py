@@ -194,6 +194,15 @@ def global_bandwidth_range(width, data, T, t0, t1, out=None):
     return out
 
 
+def local_bandwidth(width, blocks, block_size, reps):
+    out = np.empty(blocks * block_size, dtype=np.float32)
+    L = lib()
+    L.orc_local_bandwidth.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p]
+    L.orc_local_bandwidth.restype = None
+    L.orc_local_bandwidth(width, blocks, block_size, reps, out.ctypes.data)
+    return out
+
+
 # --- CPU baseline harness (cpu_harness.c) -----------------------------------------------------------
 CPUH_READ_FLOAT4, CPUH_MAD_F32, CPUH_MFMA_BF16, CPUH_MFMA_I8, CPUH_GEMM_BF16 = range(5)
 

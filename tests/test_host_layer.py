@@ -84,7 +84,7 @@ def test_full_run_row_contract_and_xml(tmp_path):
         assert cat == CATEGORY_OF_UNIT[unit]
     # measured values carry exactly 4 decimals
     vals = [m[2] for _, _, _, ms in rows for m in ms if m[1] is None]
-    assert len(vals) == 38 and all(re.fullmatch(r"-?\d+\.\d{4}", v) for v in vals)
+    assert len(vals) == 43 and all(re.fullmatch(r"-?\d+\.\d{4}", v) for v in vals)
     # rows that are deliberate skips keep the reference's status
     status = {(t, m[0]): m[1] for _, t, _, ms in rows for m in ms}
     assert status[("kernel_launch_latency", "dispatch")] == "unsupported"
@@ -171,7 +171,7 @@ def test_dump_formats_round_trip(tmp_path):
     ok = [e for e in doc["entries"] if "value" in e]
     bad = [e for e in doc["entries"] if "status" in e]
     assert len(ok) + len(bad) == n_metrics and all("reason" in e for e in bad) and all("status" not in e for e in ok)
-    assert {e["status"] for e in bad} == {"unsupported", "skipped", "error"}
+    assert {e["status"] for e in bad} == {"unsupported", "error"}
     assert set(ok[0]) >= {"backend", "platform", "device", "driver", "category", "test", "metric", "unit", "display", "value"}
     # CSV: header + one row per metric, format_version first, 15 columns
     lines = c.read_text().strip().split("\n")

@@ -292,3 +292,27 @@ def test_gemm_tile_against_numpy_and_special_cases(fmt):
     I = np.zeros((M, K), dtype=A.dtype); I[np.arange(M), np.arange(M)] = one
     got = orc.gemm_tile(fmt, I, B, K, K, K, 0, 0, M, N)
     assert np.array_equal(got, b[:, :M].T)
+
+
+# --- LDS ping-pong ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("width", [1, 2, 4])
+@pytest.mark.parametrize("block_size, reps", [(64, 1), (256, 64), (128, 300), (64, 64)])
+def test_local_bandwidth_is_a_rotation(width, block_size, reps):
+    """After `reps` hand-overs a thread holds the start vector of the thread `reps` places to its
+    right, cyclically within its workgroup: out[b*bs + l] is a closed form of the indices.  A wrong
+    direction, an off-by-one in the repetition count or a rotation across workgroups all fail this."""
+    blocks = 5
+    got = orc.local_bandwidth(width, blocks, block_size, reps)
+    b, l = np.divmod(np.arange(blocks * block_size, dtype=np.uint32), block_size)
+    src = (b * block_size + (l + reps) % block_size).astype(np.uint32)
+    comps = [(src + c).astype(np.float32) for c in range(width)]
+    want = comps[0]
+    for c in comps[1:]:
+        want = (want + c).astype(np.float32)
+    assert (got.view(np.uint32) == want.view(np.uint32)).all()
+
+
+def test_local_bandwidth_large_indices_round_like_a_float_conversion():
+    # thread ids above 2^24 are not exact in fp32: the start value is the rounded conversion
+    got = orc.local_bandwidth(1, (1 << 24) // 256 + 2, 256, 0)
+    assert got[-1] == np.float32((1 << 24) + 511) and got[(1 << 24) + 1] == np.float32(1 << 24)
