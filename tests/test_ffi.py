@@ -1,0 +1,175 @@
+"""The embedding C ABI (include/clpeak_ffi.h) through ctypes, against the stand-in device.
+
+These restate the reference's own bridge tests (app/test/ffi_integration_test.dart:28-104: version
+and catalog, a quick run that streams events and saves XML, bad arguments, cancellation) and add the
+parts of the protocol that file leaves to the header (src/ffi/clpeak_ffi.h:40-82): string ownership,
+the busy code, numbers in the classic locale with four decimals.
+"""
+import ctypes as C
+import json
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOSTLIB = os.path.join(ROOT, "clpeak_amd", "libclpeak_host.so")
+HEADER = os.path.join(ROOT, "include", "clpeak_ffi.h")
+
+CALLBACK = C.CFUNCTYPE(None, C.c_void_p, C.c_void_p)
+RUN_OK, RUN_BAD_ARGS, RUN_CANCELLED, RUN_BUSY = 0, -1, -2, -3
+
+
+@pytest.fixture(scope="module")
+def ffi():
+    lib = C.CDLL(HOSTLIB)
+    lib.clpeak_version.restype = C.c_char_p
+    lib.clpeak_copy_backend_catalog_json.restype = C.c_void_p
+    lib.clpeak_free_string.argtypes = [C.c_void_p]
+    lib.clpeak_free_string.restype = None
+    lib.clpeak_launch.argtypes = [C.c_int, C.POINTER(C.c_char_p), CALLBACK, C.c_void_p]
+    lib.clpeak_launch.restype = C.c_int
+    lib.clpeak_request_cancel.restype = None
+    lib.clpeak_load_result_file_json.argtypes = [C.c_char_p]
+    lib.clpeak_load_result_file_json.restype = C.c_void_p
+    return lib
+
+
+def take_string(lib, p):
+    """Decode a malloc'd string and give it back to the library, as the contract demands."""
+    s = C.string_at(p).decode("utf-8")
+    lib.clpeak_free_string(p)
+    return s
+
+
+def launch(lib, args, on_event=None):
+    """Run with argv = ["clpeak", *args]; returns (rc, raw event strings)."""
+    raw = []
+
+    def cb(_user, p):
+        raw.append(take_string(lib, p))
+        if on_event:
+            on_event(json.loads(raw[-1]))
+
+    argv = [b"clpeak"] + [a.encode() for a in args]
+    arr = (C.c_char_p * len(argv))(*argv)
+    keep = CALLBACK(cb)
+    rc = lib.clpeak_launch(len(argv), arr, keep, None)
+    return rc, raw
+
+
+def test_header_symbols_are_exported(ffi):
+    declared = re.findall(r"CLPEAK_FFI_EXPORT[^;]*?\b(clpeak_\w+)\s*\(", open(HEADER).read())
+    assert sorted(declared) == sorted(["clpeak_version", "clpeak_copy_backend_catalog_json", "clpeak_free_string",
+                                       "clpeak_launch", "clpeak_request_cancel", "clpeak_load_result_file_json"])
+    for name in declared:
+        getattr(ffi, name)
+
+
+def test_version_and_catalog(ffi, monkeypatch):
+    assert ffi.clpeak_version()
+    monkeypatch.setenv("CLPEAK_FAKE_DEVICES", "2")
+    doc = json.loads(take_string(ffi, ffi.clpeak_copy_backend_catalog_json()))
+    (be,) = doc["backends"]
+    assert be["name"] == "ROCm" and be["available"] is True
+    devs = be["platforms"][0]["devices"]
+    assert [d["index"] for d in devs] == [0, 1]
+    assert devs[0] == {"index": 0, "name": "Fake MI355X", "type": "GPU", "driver": "7.2.0", "computeUnits": 256,
+                       "clockMHz": 2400, "globalMemBytes": 288 << 30, "fp16": True, "fp64": True}
+    monkeypatch.setenv("CLPEAK_FAKE_DEVICES", "0")
+    doc = json.loads(take_string(ffi, ffi.clpeak_copy_backend_catalog_json()))
+    assert doc == {"backends": [{"name": "ROCm", "available": False, "platforms": []}]}
+
+
+def test_quick_run_streams_events_and_saves_xml(ffi, tmp_path):
+    xml = tmp_path / "run.xml"
+    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "-i", "1", "--xml-file", str(xml)])
+    events = [json.loads(r) for r in raw]
+    assert rc == RUN_OK
+    assert events[-1] == {"t": "done", "status": 0, "cancelled": False}
+    kinds = [e["t"] for e in events]
+    assert kinds[0] == "backend_begin" and kinds[1] == "device" and kinds[-2] == "backend_end" and kinds[-3] == "device_end"
+    assert kinds.count("test_begin") == kinds.count("test_end")
+    dev = events[1]
+    assert dev["backend"] == "ROCm" and dev["device"] == "Fake MI355X" and dev["device_index"] == 0
+    assert [p["k"] for p in dev["props"]] == ["Arch", "HIP", "CUs", "Wave", "VRAM"]
+    metrics = [e for e in events if e["t"] == "metric"]
+    assert metrics and metrics[0]["backend"] == "ROCm"
+    assert any(m["status"] == "ok" and m["value"] > 0 for m in metrics)
+    assert {"category", "test", "display", "metric", "unit", "value", "status", "reason", "sub", "desc", "minfo"} <= set(metrics[0])
+    # what a test measures arrives on test_begin, a reading's own note rides the row
+    begin = next(e for e in events if e["t"] == "test_begin" and e["test"] == "global_memory_bandwidth")
+    assert begin["desc"] and begin["unit"] == "gbps" and begin["category"] == "bandwidth"
+    assert all(m["minfo"] for m in metrics if m["test"] == "global_memory_bandwidth")
+    # numbers: classic locale, four decimals, in the raw text
+    for r in raw:
+        if '"t":"metric"' in r:
+            assert re.search(r'"value":-?\d+\.\d{4}[,}]', r), r
+    # the saved file round-trips through the native loader
+    assert xml.exists()
+    doc = json.loads(take_string(ffi, ffi.clpeak_load_result_file_json(str(xml).encode())))
+    skipped_all = sum(len(e["metrics"]) for e in events if e["t"] == "test_skipped")
+    assert len(doc["entries"]) == len(metrics) + skipped_all
+    assert doc["format_version"] == 2 and doc["devices"][0]["device"] == "Fake MI355X"
+    row = next(e for e in doc["entries"] if e["test"] == "global_memory_bandwidth" and e["metric"] == "float4")
+    assert row["description"] == begin["desc"] and row["metric_description"]
+
+
+def test_bad_args_are_rejected_without_side_effects(ffi, tmp_path):
+    xml = tmp_path / "never.xml"
+    for args in (["--bogus-flag"], ["--help"], ["--version"], ["--list-devices"], ["--iters"], ["--xml-file", str(xml), "--iters", "x"]):
+        rc, raw = launch(ffi, args)
+        events = [json.loads(r) for r in raw]
+        assert rc == RUN_BAD_ARGS, args
+        assert [e["t"] for e in events] == ["note", "done"], args
+        assert events[0]["message"].startswith("clpeak:")
+        assert events[1] == {"t": "done", "status": RUN_BAD_ARGS, "cancelled": False}
+    assert not xml.exists()
+
+
+def test_cancel_stops_the_run_and_still_saves(ffi, tmp_path):
+    xml = tmp_path / "partial.xml"
+    seen = {"metrics": 0}
+
+    def on_event(e):
+        if e["t"] == "metric":
+            seen["metrics"] += 1
+            if seen["metrics"] == 3:
+                ffi.clpeak_request_cancel()     # any thread may call this; here: the run's own
+
+    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "--xml-file", str(xml)], on_event)
+    events = [json.loads(r) for r in raw]
+    assert rc == RUN_CANCELLED
+    assert events[-1] == {"t": "done", "status": RUN_CANCELLED, "cancelled": True}
+    # the running test finishes, the remaining ones are skipped silently
+    assert [e["test"] for e in events if e["t"] == "test_begin"] == ["single_precision_compute"]
+    doc = json.loads(take_string(ffi, ffi.clpeak_load_result_file_json(str(xml).encode())))
+    assert [e["test"] for e in doc["entries"]] == ["single_precision_compute"] * 3
+    # the flag resets at the start of the next launch
+    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "--kernel-launch-latency"])
+    assert rc == RUN_OK and json.loads(raw[-1])["cancelled"] is False
+
+
+def test_second_launch_while_running_is_busy_and_silent(ffi):
+    inner = {}
+
+    def on_event(e):
+        if e["t"] == "device" and "rc" not in inner:
+            inner["rc"], inner["raw"] = launch(ffi, ["--fake-device", "--small-shapes"])
+
+    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "--kernel-launch-latency"], on_event)
+    assert inner["rc"] == RUN_BUSY and inner["raw"] == []
+    assert rc == RUN_OK and json.loads(raw[-1])["t"] == "done"
+
+
+def test_skipped_backend_runs_nothing(ffi):
+    rc, raw = launch(ffi, ["--fake-device", "--no-rocm"])
+    assert rc == RUN_OK and [json.loads(r)["t"] for r in raw] == ["done"]
+
+
+def test_load_result_file_rejects_garbage(ffi, tmp_path):
+    assert ffi.clpeak_load_result_file_json(None) is None
+    assert ffi.clpeak_load_result_file_json(str(tmp_path / "missing.xml").encode()) is None
+    bad = tmp_path / "bad.json"
+    bad.write_text("{not json")
+    assert ffi.clpeak_load_result_file_json(str(bad).encode()) is None
