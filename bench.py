@@ -11,7 +11,7 @@ of the workload list).  `value` is its throughput in GB/s.  The same line carrie
                 the stream the kernel runs on;
   cpu_baseline  the CPU oracle's float4 read-reduce timed on this host (bounded sample);
   rows          every other kernel of the backend (float/float2 reads, MAD chains, launch
-                latency, dense MFMA, 2:4 SMFMAC, GEMM) with its absolute figure, the
+                latency, dense MFMA, 2:4 SMFMAC, GEMM, LDS, PCIe transfers) with its absolute figure, the
                 MI355X datasheet peak it is compared with and the fraction reached.
 
 One GPU only: the path has no exchange step, every unit of work is independent, so more
@@ -68,7 +68,37 @@ def bench_rows(dev, quick, only):
         _matrix_rows(dev, wl, add, budget, only)
     if "gemm" in only:
         _gemm_rows(dev, capi, wl, add, budget)
+    if "lds" in only:
+        _lds_rows(dev, add, budget)
+    if "transfer" in only:
+        _transfer_rows(dev, capi, add, budget)
     return rows
+
+
+def _lds_rows(dev, add, budget):
+    # --- LDS ping-pong: the reference's grid (max(32 Mi, CUs x 2048 x 256) threads), 64 repetitions -----
+    bs, reps = 256, 64
+    threads = max(32 << 20, dev.props.num_cus * 2048 * 256)
+    blocks = threads // bs
+    out = dev.alloc(blocks * bs * 4)
+    # 128 bytes per clock and CU at the 2.4 GHz boost clock
+    peak = 128 * dev.props.num_cus * 2.4
+    for width, metric in ((1, "float"), (2, "float2"), (4, "float4")):
+        us, _ = timed(dev, lambda: dev.local_bandwidth(width, out, blocks, bs, reps), **budget)
+        add("local_memory_bandwidth", metric, reps * 2 * width * 4 * blocks * bs / us / 1e3, "gbps", us, peak)
+    out.free()
+
+
+def _transfer_rows(dev, capi, add, budget):
+    # --- pinned host <-> device copies of 512 MiB ----------------------------------------------------
+    nbytes = 1 << 29
+    _, hp = dev.host_alloc(nbytes)
+    dbuf = dev.alloc(nbytes)
+    for metric, direction, d, s in (("h2d_pinned", capi.H2D, dbuf.ptr, hp), ("d2h_pinned", capi.D2H, hp, dbuf.ptr)):
+        us, _ = timed(dev, lambda: dev.copy_async(d, s, nbytes, direction), **budget)
+        add("transfer_bandwidth", metric, nbytes / us / 1e3, "gbps", us)
+    dbuf.free()
+    dev.host_free(hp)
 
 
 def _mad_rows(dev, capi, add, budget):
@@ -188,8 +218,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel over 1 GiB (20 launches): under rocprofv3 --pmc this "
                          "gives what FETCH_SIZE / WRITE_SIZE read for a transfer of known size")
-    ap.add_argument("--only", default="mad,latency,mfma,smfmac,gemm",
-                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,gemm")
+    ap.add_argument("--only", default="mad,latency,mfma,smfmac,gemm,lds,transfer",
+                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,gemm,lds,transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; the hot path has no multi-GPU step "
