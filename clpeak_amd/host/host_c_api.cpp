@@ -28,6 +28,14 @@ size_t clpeak_host_seeded_bytes(int what, unsigned long long seed, unsigned stre
   return v.size();
 }
 
+// fields of benchmark_config_t::forDevice(type): type 1 = CPU, 2 = GPU
+void clpeak_host_config_for_device(unsigned type, unsigned long long out[6]) {
+  const benchmark_config_t c = benchmark_config_t::forDevice((DeviceType)type);
+  out[0] = c.globalBWMaxSize; out[1] = c.computeWgsPerCU; out[2] = c.computeDPWgsPerCU;
+  out[3] = c.transferBWMaxSize; out[4] = c.targetTimeUs; out[5] = c.kernelLatencyIters;
+}
+
+int clpeak_host_cancel_requested(void) { return clpeak::cancelRequested() ? 1 : 0; }
 void clpeak_host_request_cancel(void) { clpeak::requestCancel(); }
 void clpeak_host_reset_cancel(void) { clpeak::resetCancel(); }
 }
