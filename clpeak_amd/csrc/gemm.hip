@@ -93,6 +93,7 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
 struct GemmWalk {
   uint32_t a_cur, b_cur, a_nxt, b_nxt;   // LDS byte addresses of this lane's first A / B fragment, both buffers
   uint32_t dst;                          // LDS destination of the wave's 32 A rows in the buffer to refill
+  uint32_t dst_a, dst_b;                 // ring variant: destinations of the wave's A rows / B rows
   uint64_t ga, gb;                       // uniform global addresses of those A / B rows in the next slab to fetch
   uint32_t voff;                         // this lane's byte offset from ga / gb within a group of 8 rows
   uint32_t row8;                         // bytes between rows r and r+8 (load q reads from base + q*row8)
@@ -107,12 +108,12 @@ struct GemmWalk {
 template <bool MAIN>
 __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8], bf16x8v (&fb0)[4],
                                           bf16x8v (&fa1)[8], bf16x8v (&fb1)[4], const GemmWalk &w,
-                                          bool reads, bool loads) {
-  const bool READS = MAIN || reads, LOADS = MAIN || loads;
+                                          bool reads, bool loads_a, bool loads_b) {
+  const bool READS = MAIN || reads, LOADS_A = MAIN || loads_a, LOADS_B = MAIN || loads_b;
   const uint32_t a1 = w.a_cur ^ 64u, b1 = w.b_cur ^ 64u;   // second K half of this step
 #define MM(F, i, j) MI355_MFMA_BF16(acc[i][j], F##b##_[j], F##a##_[i])
-#define LDA(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst + (q) * 1024u)
-#define LDB(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst + kSlabBytes + (q) * 1024u)
+#define LDA(q) if (LOADS_A) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
+#define LDB(q) if (LOADS_B) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
   bf16x8v(&x0a_)[8] = fa0; bf16x8v(&x0b_)[4] = fb0; bf16x8v(&x1a_)[8] = fa1; bf16x8v(&x1b_)[4] = fb1;
   // ---- MFMAs 0..12 (on F0); the 12 reads of F1 in the first 6 gaps ------------------------------
   MM(x0, 0, 0); MI355_DS_READ(fb1[0], b1, 0); MI355_DS_READ(fb1[1], b1, 2048);
@@ -125,25 +126,29 @@ __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8]
   MM(x0, 2, 0); MM(x0, 2, 1); MM(x0, 2, 2); MM(x0, 2, 3);
   MM(x0, 3, 0);
   MI355_WAIT_FRAGS(fa1, fb1);
-  // every wave holds all fragments of this step's slab (its buffer is free) and every wave's
-  // share of the next slab has landed
-  asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-  // ---- MFMAs 13..39: fetch the slab two steps ahead, one load every third MFMA -------------------
-  MM(x0, 3, 1); LDA(0);
+  // Every wave holds all fragments of this step's slab: its two slots are free.  Loads return in
+  // order, so with the 4 A loads of the last step (for the slab three steps ahead) still allowed in
+  // flight, this wave's B rows of the next slab and its A rows of the next slab (older still) have
+  // landed.
+  if (MAIN) asm volatile("s_waitcnt vmcnt(4)\n s_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+  // ---- MFMAs 13..39: B rows of the slab two steps ahead into the freed A slot, then A rows of the
+  //      slab three steps ahead into the freed B slot, one load every third MFMA --------------------
+  MM(x0, 3, 1); LDB(0);
   MM(x0, 3, 2); MM(x0, 3, 3);
-  MM(x0, 4, 0); LDB(0);
+  MM(x0, 4, 0); LDB(1);
   MM(x0, 4, 1); MM(x0, 4, 2);
-  MM(x0, 4, 3); LDA(1);
+  MM(x0, 4, 3); LDB(2);
   MM(x0, 5, 0); MM(x0, 5, 1);
-  MM(x0, 5, 2); LDB(1);
+  MM(x0, 5, 2); LDB(3);
   MM(x0, 5, 3); MM(x0, 6, 0);
-  MM(x0, 6, 1); LDA(2);
+  MM(x0, 6, 1); LDA(0);
   MM(x0, 6, 2); MM(x0, 6, 3);
-  MM(x0, 7, 0); LDB(2);
+  MM(x0, 7, 0); LDA(1);
   MM(x0, 7, 1); MM(x0, 7, 2);
-  MM(x0, 7, 3); LDA(3);
+  MM(x0, 7, 3); LDA(2);
   MM(x1, 0, 0); MM(x1, 0, 1);
-  MM(x1, 0, 2); LDB(3);
+  MM(x1, 0, 2); LDA(3);
   MM(x1, 0, 3); MM(x1, 1, 0);
   MM(x1, 1, 1); MM(x1, 1, 2); MM(x1, 1, 3);
   // ---- MFMAs 40..63 (on F1); F0 is dead since MFMA 31: the next step's F0 reads, one per gap -----
@@ -197,23 +202,21 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, u
   const uint8_t *gb = B + ((size_t)tn * kTile + lrow) * k_bytes + lchunk * 16u;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const uint32_t dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 4096u);
-  auto fetch_slab = [&](uint32_t step, uint32_t buf) {
+  // LDS is a ring of five 32 KiB slots; the A rows of slab t live in slot 2t mod 5, its B rows in slot
+  // (2t+1) mod 5.  Two and a half slabs are resident or in flight at any time.
+  auto slot_off = [](uint32_t k) { return (k >= 5u ? k - 5u : k) * (uint32_t)kSlabBytes; };
+  auto fetch_rows = [&](const uint8_t *g, uint32_t step, uint32_t slot) {
     const size_t kb = (size_t)step * kRowBytes;
-    const uint32_t dst = dst_wave + buf * kBufBytes;
 #pragma unroll
-    for (uint32_t q = 0; q < 4; q++) {
-      load_to_lds(ga + kb + (size_t)q * 8u * k_bytes, dst + q * 1024u);
-      load_to_lds(gb + kb + (size_t)q * 8u * k_bytes, dst + kSlabBytes + q * 1024u);
-    }
+    for (uint32_t q = 0; q < 4; q++) load_to_lds(g + kb + (size_t)q * 8u * k_bytes, dst_wave + slot * kSlabBytes + q * 1024u);
   };
 
-  // --- LDS -> fragments: byte addresses of this lane's first A / B fragment -------------------
+  // --- LDS -> fragments: byte addresses of this lane's first A / B fragment within a slot ----------
   // row (lane%16) of the wave's sub-tile, logical chunk ks*4 + lane/16, swizzled with row&7 = lane&7;
   // the second K half differs by bit 2 of the chunk index, i.e. by 64 bytes.
   const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
-  uint32_t a_cur = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
-  uint32_t b_cur = lds_base + kSlabBytes + (wn * 64u + lane % 16u) * kRowBytes + swz0;
-  uint32_t a_nxt = a_cur + kBufBytes, b_nxt = b_cur + kBufBytes;
+  const uint32_t lane_a = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
+  const uint32_t lane_b = lds_base + (wn * 64u + lane % 16u) * kRowBytes + swz0;
 
   f32x4v acc[8][4];
 #pragma unroll
@@ -223,31 +226,38 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, u
   bf16x8v fa0[8], fb0[4], fa1[8], fb1[4];
 
   const uint32_t steps = k_bytes / kRowBytes;
-  fetch_slab(0, 0);
-  if (steps > 1) fetch_slab(1, 1);
+  fetch_rows(ga, 0, 0);
+  fetch_rows(gb, 0, 1);
+  if (steps > 1) { fetch_rows(ga, 1, 2); fetch_rows(gb, 1, 3); }
+  if (steps > 2) fetch_rows(ga, 2, 4);
   asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-  MI355_READ_FRAGS(fa0, fb0, a_cur, b_cur);
-  MI355_WAIT_FRAGS(fa0, fb0);
 
   // The loads inside the loop take the scalar-base form (uniform 64-bit base + this lane's 32-bit
   // offset), which costs no vector ALU work: load q of the wave covers rows 8q..8q+7 of its 32.
   GemmWalk w;
-  w.a_cur = a_cur; w.b_cur = b_cur; w.a_nxt = a_nxt; w.b_nxt = b_nxt;
+  uint32_t k0 = 0;   // slot of the current slab's A rows
+  auto place = [&]() {
+    w.a_cur = lane_a + slot_off(k0);     w.b_cur = lane_b + slot_off(k0 + 1u);
+    w.a_nxt = lane_a + slot_off(k0 + 2u); w.b_nxt = lane_b + slot_off(k0 + 3u);
+    w.dst_b = dst_wave + slot_off(k0);   // B rows two slabs ahead take over the current A slot
+    w.dst_a = dst_wave + slot_off(k0 + 1u);   // A rows three slabs ahead take over the current B slot
+  };
+  place();
+  MI355_READ_FRAGS(fa0, fb0, w.a_cur, w.b_cur);
+  MI355_WAIT_FRAGS(fa0, fb0);
   w.voff = (lane / 8u) * k_bytes + lchunk * 16u;
   w.row8 = 8u * k_bytes;
-  w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
+  w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kTile + wave * 32u) * k_bytes + 3 * (size_t)kRowBytes);
   w.gb = (uint64_t)(uintptr_t)(B + ((size_t)tn * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
-  w.dst = dst_wave;
-  auto advance = [&](uint32_t s) {
-    w.dst = dst_wave + ((s + 1) & 1u) * kBufBytes;
+  auto advance = [&]() {
+    k0 = k0 + 2u >= 5u ? k0 + 2u - 5u : k0 + 2u;
+    place();
     w.ga += kRowBytes;
     w.gb += kRowBytes;
-    uint32_t t = w.a_cur; w.a_cur = w.a_nxt; w.a_nxt = t;
-    t = w.b_cur; w.b_cur = w.b_nxt; w.b_nxt = t;
   };
   uint32_t s = 0;
-  for (; s + 2 < steps; s++) { gemm_step<true>(acc, fa0, fb0, fa1, fb1, w, true, true); advance(s); }
-  for (; s < steps; s++) { gemm_step<false>(acc, fa0, fb0, fa1, fb1, w, s + 1 < steps, false); advance(s); }
+  for (; s + 3 < steps; s++) { gemm_step<true>(acc, fa0, fb0, fa1, fb1, w, true, true, true); advance(); }
+  for (; s < steps; s++) { gemm_step<false>(acc, fa0, fb0, fa1, fb1, w, s + 1 < steps, false, s + 2 < steps); advance(); }
   // wait states the compiler cannot know about, before the accumulators are read
   asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
@@ -453,6 +463,7 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
 }
 
 constexpr size_t kLdsBytes = 2 * (size_t)kBufBytes;  // two 64 KiB buffers
+constexpr size_t kRingBytes = 5 * (size_t)kSlabBytes;   // five 32 KiB slots: all 160 KiB of a CU
 
 }  // namespace
 
@@ -463,11 +474,11 @@ extern "C" int mi355_gemm_bf16(mi355_dev *dev, const uint16_t *A, const uint16_t
   static bool attr_set = false;
   if (!attr_set) {
     MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_bf16_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes));
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
     attr_set = true;
   }
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_bf16_kernel<<<tiles_m * tiles_n, kThreads, kLdsBytes, dev->stream>>>(
+  gemm_bf16_kernel<<<tiles_m * tiles_n, kThreads, kRingBytes, dev->stream>>>(
       (const uint8_t *)A, (const uint8_t *)B, C, N, K * 2u, tiles_m, tiles_n);
   MI355_LAUNCH_CHECK(dev, "gemm_bf16");
   return MI355_OK;
