@@ -132,41 +132,60 @@ __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8]
   // landed.
   if (MAIN) asm volatile("s_waitcnt vmcnt(4)\n s_barrier" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-  // ---- MFMAs 13..39: B rows of the slab two steps ahead into the freed A slot, then A rows of the
-  //      slab three steps ahead into the freed B slot, one load every third MFMA --------------------
-  MM(x0, 3, 1); LDB(0);
-  MM(x0, 3, 2); MM(x0, 3, 3);
-  MM(x0, 4, 0); LDB(1);
-  MM(x0, 4, 1); MM(x0, 4, 2);
-  MM(x0, 4, 3); LDB(2);
-  MM(x0, 5, 0); MM(x0, 5, 1);
-  MM(x0, 5, 2); LDB(3);
-  MM(x0, 5, 3); MM(x0, 6, 0);
-  MM(x0, 6, 1); LDA(0);
-  MM(x0, 6, 2); MM(x0, 6, 3);
-  MM(x0, 7, 0); LDA(1);
-  MM(x0, 7, 1); MM(x0, 7, 2);
-  MM(x0, 7, 3); LDA(2);
-  MM(x1, 0, 0); MM(x1, 0, 1);
-  MM(x1, 0, 2); LDA(3);
-  MM(x1, 0, 3); MM(x1, 1, 0);
-  MM(x1, 1, 1); MM(x1, 1, 2); MM(x1, 1, 3);
-  // ---- MFMAs 40..63 (on F1); F0 is dead since MFMA 31: the next step's F0 reads, one per gap -----
+  // ---- MFMAs 13..63: B rows of the slab two steps ahead into the freed A slot, then A rows of the slab
+  //      three steps ahead into the freed B slot, one load every sixth MFMA so that the fill path sees a
+  //      steady stream; from MFMA 40 on (F0 is dead since MFMA 31) the next step's F0 reads ------------
+  MM(x0, 3, 1);
+  MM(x0, 3, 2); LDB(0);
+  MM(x0, 3, 3);
+  MM(x0, 4, 0);
+  MM(x0, 4, 1);
+  MM(x0, 4, 2);
+  MM(x0, 4, 3);
+  MM(x0, 5, 0); LDB(1);
+  MM(x0, 5, 1);
+  MM(x0, 5, 2);
+  MM(x0, 5, 3);
+  MM(x0, 6, 0);
+  MM(x0, 6, 1);
+  MM(x0, 6, 2); LDB(2);
+  MM(x0, 6, 3);
+  MM(x0, 7, 0);
+  MM(x0, 7, 1);
+  MM(x0, 7, 2);
+  MM(x0, 7, 3);
+  MM(x1, 0, 0); LDB(3);
+  MM(x1, 0, 1);
+  MM(x1, 0, 2);
+  MM(x1, 0, 3);
+  MM(x1, 1, 0);
+  MM(x1, 1, 1);
+  MM(x1, 1, 2); LDA(0);
+  MM(x1, 1, 3);
   MM(x1, 2, 0); if (READS) MI355_DS_READ(fb0[0], w.b_nxt, 0);
   MM(x1, 2, 1); if (READS) MI355_DS_READ(fb0[1], w.b_nxt, 2048);
   MM(x1, 2, 2); if (READS) MI355_DS_READ(fb0[2], w.b_nxt, 4096);
   MM(x1, 2, 3); if (READS) MI355_DS_READ(fb0[3], w.b_nxt, 6144);
-  MM(x1, 3, 0); if (READS) MI355_DS_READ(fa0[0], w.a_nxt, 0);
-  MM(x1, 3, 1); if (READS) MI355_DS_READ(fa0[1], w.a_nxt, 2048);
-  MM(x1, 3, 2); if (READS) MI355_DS_READ(fa0[2], w.a_nxt, 4096);
-  MM(x1, 3, 3); if (READS) MI355_DS_READ(fa0[3], w.a_nxt, 6144);
-  MM(x1, 4, 0); if (READS) MI355_DS_READ(fa0[4], w.a_nxt, 8192);
-  MM(x1, 4, 1); if (READS) MI355_DS_READ(fa0[5], w.a_nxt, 10240);
-  MM(x1, 4, 2); if (READS) MI355_DS_READ(fa0[6], w.a_nxt, 12288);
-  MM(x1, 4, 3); if (READS) MI355_DS_READ(fa0[7], w.a_nxt, 14336);
-  MM(x1, 5, 0); MM(x1, 5, 1); MM(x1, 5, 2); MM(x1, 5, 3);
-  MM(x1, 6, 0); MM(x1, 6, 1); MM(x1, 6, 2); MM(x1, 6, 3);
-  MM(x1, 7, 0); MM(x1, 7, 1); MM(x1, 7, 2); MM(x1, 7, 3);
+  MM(x1, 3, 0); LDA(1);
+  MM(x1, 3, 1); if (READS) MI355_DS_READ(fa0[0], w.a_nxt, 0);
+  MM(x1, 3, 2); if (READS) MI355_DS_READ(fa0[1], w.a_nxt, 2048);
+  MM(x1, 3, 3); if (READS) MI355_DS_READ(fa0[2], w.a_nxt, 4096);
+  MM(x1, 4, 0); if (READS) MI355_DS_READ(fa0[3], w.a_nxt, 6144);
+  MM(x1, 4, 1); if (READS) MI355_DS_READ(fa0[4], w.a_nxt, 8192);
+  MM(x1, 4, 2); LDA(2);
+  MM(x1, 4, 3); if (READS) MI355_DS_READ(fa0[5], w.a_nxt, 10240);
+  MM(x1, 5, 0); if (READS) MI355_DS_READ(fa0[6], w.a_nxt, 12288);
+  MM(x1, 5, 1); if (READS) MI355_DS_READ(fa0[7], w.a_nxt, 14336);
+  MM(x1, 5, 2);
+  MM(x1, 5, 3);
+  MM(x1, 6, 0); LDA(3);
+  MM(x1, 6, 1);
+  MM(x1, 6, 2);
+  MM(x1, 6, 3);
+  MM(x1, 7, 0);
+  MM(x1, 7, 1);
+  MM(x1, 7, 2);
+  MM(x1, 7, 3);
   MI355_WAIT_FRAGS(fa0, fb0);
 #undef LDA
 #undef LDB
