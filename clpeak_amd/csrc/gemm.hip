@@ -3,15 +3,22 @@
 //
 // Tiling.  One workgroup of 512 threads (8 waves, 2 per SIMD) owns a 256x256 tile
 // of C and walks K in steps of one 128-byte row segment (64 bf16 or 128 fp8
-// elements).  The A and B slabs of a step (256 rows x 128 B each) live in LDS,
-// double buffered: 2 x 64 KiB of the CU's 160 KiB.  Waves form a 2 (M) x 4 (N) grid;
-// each wave owns 128x64 of C = 8x4 MFMA tiles of 16x16, 128 fp32 accumulators per
-// lane.
+// elements): per step an A slab and a B slab of 256 rows x 128 B = 32 KiB each.  Waves
+// form a 2 (M) x 4 (N) grid; each wave owns 128x64 of C = 8x4 MFMA tiles of 16x16,
+// 128 fp32 accumulators per lane.
+//
+// LDS ring.  All 160 KiB of the CU's LDS are five 32 KiB slots; the A slab of step t
+// lives in slot 2t mod 5, its B slab in slot (2t+1) mod 5.  When the barrier of step s
+// frees the two slots of slab s, the B slab of step s+2 is fetched into the old A slot
+// and the A slab of step s+3 into the old B slot: two and a half slabs are resident or
+// in flight at any time, half of the fetches have two steps to land, and the fill path
+// always has work queued.  Loads return in order, so the wait before a barrier lets the
+// wave's 4 youngest loads (the A rows three steps ahead) stay in flight.
 //
 // Data movement.  Global memory goes straight into LDS (global_load_lds_dwordx4, 16
 // bytes per lane, no staging registers, no ds_write): one such instruction moves 8
-// rows x 128 B.  The loads of slab s+2 are issued during step s, right after the barrier
-// that frees their buffer, so they have most of a step to land.
+// rows x 128 B; a wave issues 4 for its B rows and 4 for its A rows per step, spread
+// over the whole step.
 //
 // LDS layout.  A row's 128 bytes are eight 16-byte chunks; chunk c of row r is stored
 // at chunk position c ^ (r & 7).  A fragment read (16 lanes = 16 consecutive rows,
@@ -19,15 +26,14 @@
 // one bank group 16 times.  The direct-to-LDS load writes lane i at position i of its
 // 1 KiB destination, so lane i fetches the global chunk that belongs there.
 //
-// Schedule of one step: 64 MFMAs per wave, 32 on fragment set F0 (first K half of the slab) then
-// 32 on F1 (second half); never more than one memory instruction between two MFMAs:
+// Schedule of one bf16 step: 64 MFMAs per wave, 32 on fragment set F0 (first K half of the
+// slab) then 32 on F1 (second half):
 //     MFMA  0..12   the 12 LDS reads of F1, two in each of the first 6 gaps (a 128-bit read takes
 //                   about 8 cycles to issue, two fit in the 16-cycle shadow of an MFMA)
-//     wait F1; wait own global loads; barrier      <- slab s+1 complete, slab s free
-//     MFMA 13..39   the wave's 8 global->LDS loads of slab s+2, one every third MFMA
-//     MFMA 40..63   one LDS read of the next step's F0 in each of the first 12 gaps
-// One barrier per step, placed as early as the F1 reads allow so that the loads of slab s+2 have
-// the rest of this step and the start of the next to land.
+//     wait F1; wait own loads but the 4 youngest; barrier   <- slab s+1 complete, slab s free
+//     MFMA 13..63   the wave's 8 global->LDS loads, one every sixth MFMA; from MFMA 40 on the
+//                   12 LDS reads of the next step's F0, one per gap
+// One barrier per step, placed as early as the F1 reads allow.
 // The loop body is inline assembly so that this order is the order issued;
 // the compiler knows neither the LDS reads nor the MFMAs and therefore inserts no wait
 // states of its own: every s_waitcnt below is part of the schedule.
@@ -50,7 +56,6 @@ constexpr int kTile = 256;        // C tile edge
 constexpr int kRowBytes = 128;    // bytes of K per step, per row
 constexpr int kThreads = 512;
 constexpr int kSlabBytes = kTile * kRowBytes;   // 32 KiB per operand per step
-constexpr int kBufBytes = 2 * kSlabBytes;       // A slab then B slab
 
 typedef __attribute__((address_space(3))) void *lds_void_ptr;
 typedef const __attribute__((address_space(1))) void *global_void_ptr;
@@ -92,8 +97,7 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
 // State of one wave's walk along K that the step function advances.
 struct GemmWalk {
   uint32_t a_cur, b_cur, a_nxt, b_nxt;   // LDS byte addresses of this lane's first A / B fragment, both buffers
-  uint32_t dst;                          // LDS destination of the wave's 32 A rows in the buffer to refill
-  uint32_t dst_a, dst_b;                 // ring variant: destinations of the wave's A rows / B rows
+  uint32_t dst_a, dst_b;                 // LDS destinations of the wave's 32 A rows / 32 B rows to fetch
   uint64_t ga, gb;                       // uniform global addresses of those A / B rows in the next slab to fetch
   uint32_t voff;                         // this lane's byte offset from ga / gb within a group of 8 rows
   uint32_t row8;                         // bytes between rows r and r+8 (load q reads from base + q*row8)
@@ -327,12 +331,12 @@ struct Fp8Frags {
 
 template <bool MAIN>
 __device__ __forceinline__ void gemm_fp8_step(f32x4v (&acc)[8][4], Fp8Frags &f, const GemmWalk &w, bool reads,
-                                              bool loads) {
-  const bool READS = MAIN || reads, LOADS = MAIN || loads;
+                                              bool loads_a, bool loads_b) {
+  const bool READS = MAIN || reads, LOADS_A = MAIN || loads_a, LOADS_B = MAIN || loads_b;
   const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u, an_hi = w.a_nxt ^ 64u, bn_hi = w.b_nxt ^ 64u;
 #define MM(i, j) MI355_MFMA_FP8(acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i])
-#define LDA(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst + (q) * 1024u)
-#define LDB(q) if (LOADS) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst + kSlabBytes + (q) * 1024u)
+#define LDA(q) if (LOADS_A) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
+#define LDB(q) if (LOADS_B) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
 #define RD_A_NEXT(i, off)                                                                          \
   if (READS) { MI355_DS_READ(f.a_lo[i], w.a_nxt, off); MI355_DS_READ(f.a_hi[i], an_hi, off); }
 #define RD_B_NEXT(j, off)                                                                          \
@@ -350,24 +354,25 @@ __device__ __forceinline__ void gemm_fp8_step(f32x4v (&acc)[8][4], Fp8Frags &f, 
   MM(3, 0); MM(3, 1);
   MI355_WAIT_LGKM(10);                                   // A4
   MM(4, 0); MM(4, 1);
-  // every read of this step's slab has returned (its buffer is free) and this wave's share of the
-  // next slab has landed
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier" ::: "memory");
-  MM(5, 0); LDA(0);
-  MM(5, 1); LDB(0);
-  MM(6, 0); LDA(1);
-  MM(6, 1); LDB(1);
-  MM(7, 0); LDA(2);
-  MM(7, 1); LDB(2);
+  // every read of this step's slab has returned (its two slots are free); with the 4 A loads of the
+  // last step still allowed in flight, this wave's share of the next slab has landed
+  if (MAIN) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n s_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier" ::: "memory");
+  MM(5, 0); LDB(0);
+  MM(5, 1);
+  MM(6, 0); LDB(1);
+  MM(6, 1);
+  MM(7, 0); LDB(2);
+  MM(7, 1); LDB(3);
   MM(0, 2); RD_B_NEXT(0, 0);
   MM(0, 3); RD_B_NEXT(1, 2048);
-  MM(1, 2); LDA(3);
+  MM(1, 2); LDA(0);
   MM(1, 3); RD_A_NEXT(0, 0);
-  MM(2, 2); LDB(3);
+  MM(2, 2); LDA(1);
   MM(2, 3); RD_A_NEXT(1, 2048);
-  MM(3, 2);
+  MM(3, 2); LDA(2);
   MM(3, 3); RD_A_NEXT(2, 4096);
-  MM(4, 2);
+  MM(4, 2); LDA(3);
   MM(4, 3); RD_A_NEXT(3, 6144);
   MM(5, 2);
   MM(5, 3); RD_A_NEXT(4, 8192);
@@ -398,24 +403,18 @@ gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, ui
   const uint8_t *gb = B + ((size_t)tn * kTile + lrow) * k_bytes + lchunk * 16u;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const uint32_t dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 4096u);
-  auto fetch_slab = [&](uint32_t step, uint32_t buf) {
+  auto slot_off = [](uint32_t k) { return (k >= 5u ? k - 5u : k) * (uint32_t)kSlabBytes; };
+  auto fetch_rows = [&](const uint8_t *g, uint32_t step, uint32_t slot) {
     const size_t kb = (size_t)step * kRowBytes;
-    const uint32_t dst = dst_wave + buf * kBufBytes;
 #pragma unroll
-    for (uint32_t q = 0; q < 4; q++) {
-      load_to_lds(ga + kb + (size_t)q * 8u * k_bytes, dst + q * 1024u);
-      load_to_lds(gb + kb + (size_t)q * 8u * k_bytes, dst + kSlabBytes + q * 1024u);
-    }
+    for (uint32_t q = 0; q < 4; q++) load_to_lds(g + kb + (size_t)q * 8u * k_bytes, dst_wave + slot * kSlabBytes + q * 1024u);
   };
 
   // LDS -> fragments: chunk lane/16 of row lane%16 (low half of the operand); the high half is
   // chunk lane/16 + 4, i.e. the address with bit 6 flipped.
   const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
-  GemmWalk w;
-  w.a_cur = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
-  w.b_cur = lds_base + kSlabBytes + (wn * 64u + lane % 16u) * kRowBytes + swz0;
-  w.a_nxt = w.a_cur + kBufBytes;
-  w.b_nxt = w.b_cur + kBufBytes;
+  const uint32_t lane_a = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
+  const uint32_t lane_b = lds_base + (wn * 64u + lane % 16u) * kRowBytes + swz0;
 
   f32x4v acc[8][4];
 #pragma unroll
@@ -425,9 +424,21 @@ gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, ui
   Fp8Frags f;
 
   const uint32_t steps = k_bytes / kRowBytes;
-  fetch_slab(0, 0);
-  if (steps > 1) fetch_slab(1, 1);
+  fetch_rows(ga, 0, 0);
+  fetch_rows(gb, 0, 1);
+  if (steps > 1) { fetch_rows(ga, 1, 2); fetch_rows(gb, 1, 3); }
+  if (steps > 2) fetch_rows(ga, 2, 4);
   asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+
+  GemmWalk w;
+  uint32_t k0 = 0;   // slot of the current slab's A rows (the ring of the bf16 kernel)
+  auto place = [&]() {
+    w.a_cur = lane_a + slot_off(k0);      w.b_cur = lane_b + slot_off(k0 + 1u);
+    w.a_nxt = lane_a + slot_off(k0 + 2u); w.b_nxt = lane_b + slot_off(k0 + 3u);
+    w.dst_b = dst_wave + slot_off(k0);
+    w.dst_a = dst_wave + slot_off(k0 + 1u);
+  };
+  place();
   // what a step expects in flight on entry: B fragments 0,1 then A fragments 0..6
   {
     const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u;
@@ -444,19 +455,17 @@ gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, ui
 
   w.voff = (lane / 8u) * k_bytes + lchunk * 16u;
   w.row8 = 8u * k_bytes;
-  w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
+  w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kTile + wave * 32u) * k_bytes + 3 * (size_t)kRowBytes);
   w.gb = (uint64_t)(uintptr_t)(B + ((size_t)tn * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
-  w.dst = dst_wave;
-  auto advance = [&](uint32_t s) {
-    w.dst = dst_wave + ((s + 1) & 1u) * kBufBytes;
+  auto advance = [&]() {
+    k0 = k0 + 2u >= 5u ? k0 + 2u - 5u : k0 + 2u;
+    place();
     w.ga += kRowBytes;
     w.gb += kRowBytes;
-    uint32_t t = w.a_cur; w.a_cur = w.a_nxt; w.a_nxt = t;
-    t = w.b_cur; w.b_cur = w.b_nxt; w.b_nxt = t;
   };
   uint32_t s = 0;
-  for (; s + 2 < steps; s++) { gemm_fp8_step<true>(acc, f, w, true, true); advance(s); }
-  for (; s < steps; s++) { gemm_fp8_step<false>(acc, f, w, s + 1 < steps, false); advance(s); }
+  for (; s + 3 < steps; s++) { gemm_fp8_step<true>(acc, f, w, true, true, true); advance(); }
+  for (; s < steps; s++) { gemm_fp8_step<false>(acc, f, w, s + 1 < steps, false, s + 2 < steps); advance(); }
   asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
   const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 64u + 4u * (lane / 16u);
@@ -481,7 +490,6 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
   return MI355_OK;
 }
 
-constexpr size_t kLdsBytes = 2 * (size_t)kBufBytes;  // two 64 KiB buffers
 constexpr size_t kRingBytes = 5 * (size_t)kSlabBytes;   // five 32 KiB slots: all 160 KiB of a CU
 
 }  // namespace
@@ -510,11 +518,11 @@ extern "C" int mi355_gemm_fp8_e4m3(mi355_dev *dev, const uint8_t *A, const uint8
   static bool attr_set = false;
   if (!attr_set) {
     MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_fp8_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes));
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
     attr_set = true;
   }
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_fp8_kernel<<<tiles_m * tiles_n, kThreads, kLdsBytes, dev->stream>>>(
+  gemm_fp8_kernel<<<tiles_m * tiles_n, kThreads, kRingBytes, dev->stream>>>(
       A, B, C, N, K, scale_a * scale_b, tiles_m, tiles_n);
   MI355_LAUNCH_CHECK(dev, "gemm_fp8_e4m3");
   return MI355_OK;
