@@ -310,11 +310,11 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, u
 // against 2,3:
 //     MFMA  0..9    (i,0),(i,1): this step's A fragment 7 and B fragments 2,3 are read in gaps 0..2;
 //                   counted waits let row i start as soon as its own fragment has arrived
-//     wait all reads; wait own global loads; barrier    <- slab s+1 complete, slab s free
-//     MFMA 10..15   six of the wave's 8 global->LDS loads of slab s+2 (the other two in gaps 18, 20)
+//     wait all reads; wait own loads but the 4 youngest; barrier   <- slab s+1 complete, slab s free
+//     MFMA 10..15   the wave's 4 loads of B rows (slab s+2)
 //     MFMA 16..31   (i,2),(i,3): next step's B fragments 0,1 in gaps 16,17, next step's A fragment
 //                   i-1 after row i (a fragment is overwritten no sooner than one instruction after
-//                   its last use)
+//                   its last use); the wave's 4 loads of A rows (slab s+3) in the even gaps 18..24
 #define MI355_MFMA_FP8(acc, blo, bhi, alo, ahi)                                                    \
   do {                                                                                             \
     const i32x8v b8_ = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7);                  \
