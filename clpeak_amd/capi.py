@@ -155,6 +155,9 @@ class Device:
         a = np.ascontiguousarray(array)
         return DeviceBuffer(self, max(a.nbytes, 1)).upload(a)
 
+    def memset(self, buf, byte, nbytes=None):
+        self._check(self.lib.mi355_memset(self.h, buf.ptr, byte, buf.nbytes if nbytes is None else nbytes))
+
     def sync(self):
         self._check(self.lib.mi355_sync(self.h))
 
