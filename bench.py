@@ -9,7 +9,8 @@ of the workload list).  `value` is its throughput in GB/s.  The same line carrie
 
   roofline      the headline kernel against the 8 TB/s HBM3E peak, from HIP events on
                 the stream the kernel runs on;
-  cpu_baseline  the CPU oracle's float4 read-reduce timed on this host (bounded sample);
+  cpu_baseline  the reference's own DRAM read kernel (where its build exists) and the CPU oracle's kernels,
+                timed on this host with the reference's CPU discipline (bounded samples);
   rows          every other kernel of the backend (float/float2 reads, MAD chains, launch
                 latency, dense MFMA, 2:4 SMFMAC, GEMM, LDS, PCIe transfers) with its absolute figure, the
                 MI355X datasheet peak it is compared with and the fraction reached.
@@ -184,17 +185,24 @@ def _gemm_rows(dev, capi, wl, add, budget):
 
 
 def cpu_baseline(target_us=2_000_000, extra_target_us=1_000_000):
-    """The oracle's kernels on this host's cores, timed with the reference's CPU discipline (pinned
-    persistent pool, warm-ups, settle phase before the all-core run, adaptive probe, one timed batch
-    sized to the budget): one thread (ST) and every logical core (MT).  The headline figure is the
-    float4 read-reduce in its CPU-sized form (2^26 floats, 2^20 partial sums); the other workloads are
-    listed under "others" on bounded samples."""
+    """CPU figures beside the GPU ones, all timed with the reference's CPU discipline (pinned persistent
+    pool, warm-ups, settle phase before the all-core run, adaptive probe, one timed batch sized to the
+    budget), at one thread (ST) and at every logical core (MT).
+
+    Where the build of the reference's own CPU kernels exists (oracle/_ref, made from the reference's
+    sources on the machine that has them) the headline value is the reference's DRAM read kernel and its
+    fp32 chain is listed too (kind "reference"); the oracle's kernels on the seeded workloads (kind
+    "port") are always listed under "port"."""
     from oracle import pyoracle as orc
     cores = len(os.sched_getaffinity(0))
     t0 = time.perf_counter()
+    ref = orc.reference_kernels()
     with orc.CpuPool(cores) as pool:
         r = pool.measure(orc.CPUH_READ_FLOAT4, SEED, 2, target_us)
-        others = {}
+        port = {"global_memory_bandwidth float4": {
+            "ST": round(r.giga_st, 2), "MT": round(r.giga_mt, 2), "unit": "GB/s", "threads": r.threads_mt,
+            "iters_ST": r.iters_st, "iters_MT": r.iters_mt,
+            "sample": "float4 read-reduce over a 256 MiB (2^26 float) seeded buffer, 2^20 partial sums, one pass per iteration"}}
         for name, kind, unit, what in (
                 ("single_precision_compute float", orc.CPUH_MAD_F32, "gflops",
                  "8 work-items x 16 accumulators x 4096 fma per iteration"),
@@ -202,15 +210,29 @@ def cpu_baseline(target_us=2_000_000, extra_target_us=1_000_000):
                 ("mfma_int8", orc.CPUH_MFMA_I8, "gops", "4 emulated 16x16x64 int8 products per iteration"),
                 ("rocblas-fp bf16", orc.CPUH_GEMM_BF16, "gflops", "one 64x64 tile of the K=8192 bf16 GEMM per iteration")):
             q = pool.measure(kind, SEED, 2, extra_target_us)
-            others[name] = {"ST": round(q.giga_st, 3), "MT": round(q.giga_mt, 3), "unit": unit, "threads": q.threads_mt,
-                            "iters_ST": q.iters_st, "iters_MT": q.iters_mt, "sample": what}
+            port[name] = {"ST": round(q.giga_st, 3), "MT": round(q.giga_mt, 3), "unit": unit, "threads": q.threads_mt,
+                          "iters_ST": q.iters_st, "iters_MT": q.iters_mt, "sample": what}
+        reference = None
+        if ref is not None:
+            rd = pool.measure_read_fn(ref["read_fn"], ref["populate_fn"], 1 << 26, 2, target_us)
+            ch = pool.measure_chain_fn(ref["fp32_fn"], ref["fp32_ops"], 2, extra_target_us)
+            reference = {"isa": ref["isa"],
+                         "global_memory_bandwidth read": {"ST": round(rd.giga_st, 2), "MT": round(rd.giga_mt, 2), "unit": "GB/s",
+                                                          "iters_ST": rd.iters_st, "iters_MT": rd.iters_mt},
+                         "single_precision_compute float": {"ST": round(ch.giga_st, 2), "MT": round(ch.giga_mt, 2),
+                                                            "unit": "gflops", "iters_ST": ch.iters_st, "iters_MT": ch.iters_mt}}
     dt = time.perf_counter() - t0
-    return {"value": round(r.giga_mt, 2), "unit": "GB/s", "cores": r.threads_mt, "kind": "port",
-            "ST": round(r.giga_st, 2), "MT": round(r.giga_mt, 2), "pinned_workers": r.pinned,
-            "sample": f"float4 read-reduce over a 256 MiB (2^26 float) seeded buffer, 2^20 partial sums, C oracle "
-                      f"(no fast-math): {r.iters_st} passes on 1 thread, {r.iters_mt} passes on {r.threads_mt} threads "
-                      f"(each thread a contiguous share of the partial sums); whole CPU leg {dt:.1f} s",
-            "others": others}
+    if reference is not None:
+        value, kind = reference["global_memory_bandwidth read"]["MT"], "reference"
+        sample = (f"the reference's DRAM read kernel (readBufferChecksum, {ref['isa']} build of its own source) over a 256 MiB "
+                  f"array filled by its populate(), per-thread contiguous chunks: {rd.iters_st} passes on 1 thread, "
+                  f"{rd.iters_mt} passes on {rd.threads_mt} threads; whole CPU leg {dt:.1f} s")
+    else:
+        value, kind = port["global_memory_bandwidth float4"]["MT"], "port"
+        sample = (f"float4 read-reduce over a 256 MiB (2^26 float) seeded buffer, 2^20 partial sums, C oracle (no fast-math): "
+                  f"{r.iters_st} passes on 1 thread, {r.iters_mt} passes on {r.threads_mt} threads; whole CPU leg {dt:.1f} s")
+    return {"value": value, "unit": "GB/s", "cores": r.threads_mt, "kind": kind, "pinned_workers": r.pinned,
+            "sample": sample, "reference": reference, "port": port}
 
 
 def main():

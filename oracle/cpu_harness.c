@@ -15,8 +15,10 @@
  *     units_per_iter * threads / (us * 1e3) in giga-units (reference:
  *     src/cpu/compute_common.h:21-60).
  *
- * Only tests and the cpu_baseline leg of the benchmark driver load this.  The bodies call the
- * oracle's own functions (no fast-math, no contraction), so what is timed is the checker.
+ * Only tests and the cpu_baseline leg of the benchmark driver load this.  The built-in bodies call
+ * the oracle's own functions (no fast-math, no contraction), so what is timed is the checker; the
+ * *_fn entry points time kernels handed in as function pointers instead, which is how the
+ * reference's own CPU kernels are timed where a build of them exists.
  */
 #define _GNU_SOURCE
 #include <math.h>
@@ -386,6 +388,117 @@ int cpuh_measure(cpuh_pool *p, int kind, uint64_t seed, unsigned warmup, unsigne
     free(w->buf); free(w->partials); free(w->mad_out); free(w->A); free(w->B); free(w->tiles);
     free(w->ga); free(w->gb); free(w->gc); free(w);
     return rc;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Kernels handed in as function pointers (the reference's own CPU kernels, where a build of them
+ * exists): the chain signature and the streaming-read signature of src/cpu/cpu_kernels.h:62-66.   */
+typedef double (*cpuh_chain_fn)(uint64_t outer);
+typedef uint64_t (*cpuh_read_fn)(const float *p, size_t m, uint64_t iters);
+typedef void (*cpuh_populate_fn)(float *p, unsigned long long n);
+
+typedef struct {
+    cpuh_chain_fn chain;
+    cpuh_read_fn read;
+    cpuh_populate_fn populate;
+    float *buf;
+    uint64_t n_floats;
+    int n_threads;        /* threads of the dispatch being timed: the buffer is split among them */
+    double sink[MAX_T];
+    uint64_t xsink[MAX_T];
+} fn_workload;
+
+static void body_chain_fn(void *c, int tid, uint64_t iters)
+{
+    fn_workload *w = (fn_workload *)c;
+    w->sink[tid] += w->chain(iters);
+}
+
+/* per-thread contiguous chunk, the last thread takes the remainder (src/cpu/bandwidth.cpp:283-288) */
+static void chunk_of(const fn_workload *w, int tid, int n, uint64_t *lo, uint64_t *hi)
+{
+    const uint64_t per = w->n_floats / (uint64_t)n;
+    *lo = (uint64_t)tid * per;
+    *hi = tid == n - 1 ? w->n_floats : *lo + per;
+}
+
+static void body_read_fn(void *c, int tid, uint64_t iters)
+{
+    fn_workload *w = (fn_workload *)c;
+    uint64_t lo, hi;
+    chunk_of(w, tid, w->n_threads, &lo, &hi);
+    w->xsink[tid] ^= w->read(w->buf + lo, (size_t)(hi - lo), iters);
+}
+
+static void body_first_touch(void *c, int tid, uint64_t iters)
+{
+    fn_workload *w = (fn_workload *)c;
+    (void)iters;
+    uint64_t lo, hi;
+    chunk_of(w, tid, w->n_threads, &lo, &hi);
+    w->populate(w->buf + lo, hi - lo);
+}
+
+static void finish(cpuh_pool *p, cpuh_result *r, int n, double units_st, double units_mt)
+{
+    r->threads_mt = n;
+    r->pinned = 0;
+    for (int t = 0; t < n; t++) r->pinned += p->pinned_cpu[t] == t;
+    r->units_per_iter_st = units_st;
+    r->units_per_iter_mt = units_mt;
+    r->giga_st = r->us_st > 0.0 ? units_st / (r->us_st * 1e3) : -1.0;
+    r->giga_mt = r->us_mt > 0.0 ? units_mt * (double)n / (r->us_mt * 1e3) : -1.0;
+}
+
+/* A compute chain at 1 thread and at every worker: value = ops_per_iter * threads / (us * 1e3). */
+int cpuh_measure_chain_fn(cpuh_pool *p, cpuh_chain_fn fn, double ops_per_iter, unsigned warmup, unsigned target_us,
+                          cpuh_result *r)
+{
+    if (!fn || !r) return -1;
+    const int n = p->n_max > MAX_T ? MAX_T : p->n_max;
+    fn_workload *w = (fn_workload *)calloc(1, sizeof(*w));
+    if (!w) return -3;
+    w->chain = fn;
+    memset(r, 0, sizeof(*r));
+    r->us_st = cpuh_run_workload(p, 1, body_chain_fn, w, warmup, target_us, 0, &r->iters_st);
+    r->us_mt = cpuh_run_workload(p, n, body_chain_fn, w, warmup, target_us, 0, &r->iters_mt);
+    finish(p, r, n, ops_per_iter, ops_per_iter);
+    volatile double keep = 0.0;
+    for (int t = 0; t < n; t++) keep += w->sink[t];
+    (void)keep;
+    free(w);
+    return 0;
+}
+
+/* A streaming read over one shared array of n_floats, first-touched in parallel by the threads that
+ * will read it and split into per-thread contiguous chunks; one iteration = one pass over the whole
+ * array, value = n_floats * 4 / (us * 1e3) GB/s (src/cpu/bandwidth.cpp:274-321). */
+int cpuh_measure_read_fn(cpuh_pool *p, cpuh_read_fn fn, cpuh_populate_fn populate, uint64_t n_floats, unsigned warmup,
+                         unsigned target_us, cpuh_result *r)
+{
+    if (!fn || !populate || !r || n_floats == 0) return -1;
+    const int n = p->n_max > MAX_T ? MAX_T : p->n_max;
+    fn_workload *w = (fn_workload *)calloc(1, sizeof(*w));
+    if (!w) return -3;
+    w->read = fn;
+    w->populate = populate;
+    w->n_floats = n_floats / (uint64_t)n * (uint64_t)n;
+    w->buf = (float *)aligned_alloc(64, w->n_floats * sizeof(float));
+    if (!w->buf) { free(w); return -3; }
+    w->n_threads = n;
+    cpuh_pool_run(p, n, body_first_touch, w, 1);
+    memset(r, 0, sizeof(*r));
+    w->n_threads = 1;
+    r->us_st = cpuh_run_workload(p, 1, body_read_fn, w, warmup, target_us, 0, &r->iters_st);
+    w->n_threads = n;
+    r->us_mt = cpuh_run_workload(p, n, body_read_fn, w, warmup, target_us, 0, &r->iters_mt);
+    finish(p, r, n, (double)w->n_floats * 4.0, (double)w->n_floats * 4.0 / (double)n);
+    volatile uint64_t keep = 0;
+    for (int t = 0; t < n; t++) keep ^= w->xsink[t];
+    (void)keep;
+    free(w->buf);
+    free(w);
+    return 0;
 }
 
 /* Test hook: a body that sleeps `ctx` microseconds per iteration, so the discipline can be checked

@@ -226,6 +226,8 @@ def _bind_harness():
     L.cpuh_pick_iters.argtypes = [dbl, u32, u32, u32]; L.cpuh_pick_iters.restype = u32
     L.cpuh_time_sleep_body.argtypes = [vp, i32, u32, u32, C.POINTER(u32)]; L.cpuh_time_sleep_body.restype = dbl
     L.cpuh_measure.argtypes = [vp, i32, u64, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure.restype = i32
+    L.cpuh_measure_chain_fn.argtypes = [vp, vp, dbl, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure_chain_fn.restype = i32
+    L.cpuh_measure_read_fn.argtypes = [vp, vp, vp, u64, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure_read_fn.restype = i32
     L._harness_bound = True
     return L
 
@@ -270,6 +272,55 @@ class CpuPool:
         if rc != 0:
             raise RuntimeError(f"cpuh_measure({kind}) failed: {rc}")
         return r
+
+
+    def measure_chain_fn(self, fn_ptr, ops_per_iter, warmup=2, target_us=2_000_000):
+        """Times a `double fn(uint64_t outer)` chain given as a raw function pointer."""
+        r = CpuhResult()
+        rc = self.L.cpuh_measure_chain_fn(self.h, fn_ptr, ops_per_iter, warmup, target_us, C.byref(r))
+        if rc != 0:
+            raise RuntimeError(f"cpuh_measure_chain_fn failed: {rc}")
+        return r
+
+    def measure_read_fn(self, read_ptr, populate_ptr, n_floats, warmup=2, target_us=2_000_000):
+        """Times a `uint64_t fn(const float*, size_t, uint64_t iters)` streaming read over a shared array."""
+        r = CpuhResult()
+        rc = self.L.cpuh_measure_read_fn(self.h, read_ptr, populate_ptr, n_floats, warmup, target_us, C.byref(r))
+        if rc != 0:
+            raise RuntimeError(f"cpuh_measure_read_fn failed: {rc}")
+        return r
+
+
+REF_LIB_PATH = os.path.join(_HERE, "_ref", "libclpeak_ref.so")
+
+
+def reference_kernels():
+    """The reference's own CPU kernels (built by ref.mk where its checkout is present), for the widest ISA
+    this host runs: dict(isa, fp32_fn, fp32_ops, read_fn, populate_fn), or None when the build is absent."""
+    if not os.path.exists(REF_LIB_PATH):
+        return None
+    flags = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("flags"):
+                    flags = line
+                    break
+    except OSError:
+        return None
+    have = set(flags.split())
+    if {"avx512f", "avx512bw", "avx512vl", "avx512dq"} <= have:
+        isa, name = 1, "AVX-512"
+    elif {"avx2", "fma", "f16c"} <= have:
+        isa, name = 0, "AVX2+FMA"
+    else:
+        return None
+    R = C.CDLL(REF_LIB_PATH)
+    R.ref_fp32_chain_fn.argtypes = [C.c_int]; R.ref_fp32_chain_fn.restype = C.c_void_p
+    R.ref_fp32_chain_ops.argtypes = [C.c_int]; R.ref_fp32_chain_ops.restype = C.c_double
+    R.ref_readsum_fn.argtypes = [C.c_int]; R.ref_readsum_fn.restype = C.c_void_p
+    return {"isa": name, "lib": R, "fp32_fn": R.ref_fp32_chain_fn(isa), "fp32_ops": R.ref_fp32_chain_ops(isa),
+            "read_fn": R.ref_readsum_fn(isa), "populate_fn": C.cast(R.ref_populate, C.c_void_p).value}
 
 
 def pick_iters(per_iter_us, target_us, forced, max_iters):

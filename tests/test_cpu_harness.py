@@ -94,3 +94,37 @@ def test_measure_reports_st_and_mt_in_giga_units(pool):
     assert 0.05 < r.giga_st < 1000.0          # a scalar fma chain on any x86 core of this decade
     with pytest.raises(RuntimeError):
         pool.measure(99, 1)
+
+
+def test_chain_given_as_function_pointer_is_priced_per_thread(pool):
+    import ctypes as C
+    import time
+    calls = []
+
+    @C.CFUNCTYPE(C.c_double, C.c_uint64)
+    def chain(outer):           # 200 us per outer iteration, whatever thread runs it
+        calls.append(outer)
+        time.sleep(200e-6 * outer)
+        return 1.0
+
+    r = pool.measure_chain_fn(C.cast(chain, C.c_void_p).value, 1000.0, warmup=1, target_us=40_000)
+    assert r.threads_mt == pool.max_threads and r.units_per_iter_st == 1000.0
+    assert 200.0 <= r.us_st < 450.0 and 200.0 <= r.us_mt < 450.0
+    # 1000 units per 200+ us on one thread: < 5 giga-units / 1000; MT counts every thread's units
+    assert r.giga_st == pytest.approx(1000.0 / (r.us_st * 1e3))
+    assert r.giga_mt == pytest.approx(1000.0 * r.threads_mt / (r.us_mt * 1e3))
+    # the timed batch is ONE dispatch whose body loops itself: the batch sizes were passed as `outer`
+    assert r.iters_st in calls and calls.count(r.iters_mt) >= pool.max_threads
+
+
+def test_reference_kernels_run_under_the_harness(pool):
+    ref = orc.reference_kernels()
+    if ref is None:
+        pytest.skip("reference build (oracle/_ref) not present")
+    # ops per outer iteration = INNER * NACC * LANES * 2 of the ISA's table entry (src/cpu/cpu_kernels_impl.h:54)
+    assert ref["fp32_ops"] in (4096 * 12 * 8 * 2.0, 4096 * 24 * 16 * 2.0)
+    ch = pool.measure_chain_fn(ref["fp32_fn"], ref["fp32_ops"], warmup=1, target_us=50_000)
+    assert 5.0 < ch.giga_st < 500.0 and ch.giga_mt > ch.giga_st        # a SIMD FMA chain, scaling with threads
+    rd = pool.measure_read_fn(ref["read_fn"], ref["populate_fn"], 1 << 24, warmup=1, target_us=50_000)
+    assert 1.0 < rd.giga_st < 200.0 and rd.giga_mt > 0.8 * rd.giga_st
+    assert rd.units_per_iter_st == (1 << 24) // pool.max_threads * pool.max_threads * 4.0
