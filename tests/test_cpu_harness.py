@@ -61,8 +61,8 @@ def test_run_workload_recovers_a_known_iteration_time(pool):
     # batch must be sized for the 100 ms budget, and the mean must come back near 500 us (sleep overshoots)
     for n in (1, pool.max_threads):
         us, iters = pool.time_sleep_body(n, 500, 100_000)
-        assert 500.0 <= us < 900.0, us
-        assert 100_000 / 900.0 <= iters <= 100_000 / 500.0 + 1, iters
+        assert 500.0 <= us < 1500.0, us          # sleep overshoots, more so on a busy machine
+        assert 100_000 / 1500.0 <= iters <= 100_000 / 500.0 + 1, iters
 
 
 def test_ranged_read_reduce_is_the_same_sum():
