@@ -68,7 +68,9 @@ def bench_rows(dev, quick, only):
     if "mfma" in only or "smfmac" in only:
         _matrix_rows(dev, wl, add, budget, only)
     if "gemm" in only:
-        _gemm_rows(dev, capi, wl, add, budget)
+        _gemm_rows(dev, capi, wl, add, budget, constant=False)
+    if "gemm_const" in only:
+        _gemm_rows(dev, capi, wl, add, budget, constant=True)
     if "lds" in only:
         _lds_rows(dev, add, budget)
     if "transfer" in only:
@@ -157,7 +159,7 @@ def _matrix_rows(dev, wl, add, budget, only):
     clk.free()
 
 
-def _gemm_rows(dev, capi, wl, add, budget):
+def _gemm_rows(dev, capi, wl, add, budget, constant):
     # --- GEMM 8192^3 ---------------------------------------------------------------------------
     M = N = K = 8192
     for fp8 in (False, True):
@@ -171,15 +173,15 @@ def _gemm_rows(dev, capi, wl, add, budget):
             dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1)
             dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
             fn = lambda: dev.gemm_bf16(dA, dB, dC, M, N, K)
+        metric = "fp8_e4m3" if fp8 else "bf16"
+        if constant:
+            # the same launch on the reference's buffers (every byte 0x38 / 0x3f, src/rocm/rocblas.cpp:211-212,
+            # src/rocm/hipblaslt_gemm.cpp:271-273): constant operands draw less power, the part holds a higher clock
+            dev.memset(dA, 0x38 if fp8 else 0x3f); dev.memset(dB, 0x38 if fp8 else 0x3f)
+            metric += " constant operands"
         us, _ = timed(dev, fn, **budget)
-        add("hipblaslt-fp8" if fp8 else "rocblas-fp", "fp8_e4m3" if fp8 else "bf16", 2.0 * M * N * K / us / 1e6, "tflops", us,
+        add("hipblaslt-fp8" if fp8 else "rocblas-fp", metric, 2.0 * M * N * K / us / 1e6, "tflops", us,
             PEAK["fp8" if fp8 else "bf16"], shape="8192x8192x8192")
-        # the same launch on the reference's buffers (every byte 0x38 / 0x3f, src/rocm/rocblas.cpp:211-212,
-        # src/rocm/hipblaslt_gemm.cpp:271-273): constant operands draw less power, the part holds a higher clock
-        dev.memset(dA, 0x38 if fp8 else 0x3f); dev.memset(dB, 0x38 if fp8 else 0x3f)
-        us, _ = timed(dev, fn, **budget)
-        add("hipblaslt-fp8" if fp8 else "rocblas-fp", ("fp8_e4m3" if fp8 else "bf16") + " constant operands",
-            2.0 * M * N * K / us / 1e6, "tflops", us, PEAK["fp8" if fp8 else "bf16"], shape="8192x8192x8192")
         for b in (dA, dB, dC):
             b.free()
 
@@ -246,8 +248,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel over 1 GiB (20 launches): under rocprofv3 --pmc this "
                          "gives what FETCH_SIZE / WRITE_SIZE read for a transfer of known size")
-    ap.add_argument("--only", default="mad,latency,mfma,smfmac,gemm,lds,transfer",
-                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,gemm,lds,transfer")
+    ap.add_argument("--only", default="mad,latency,mfma,smfmac,gemm,gemm_const,lds,transfer",
+                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,gemm,gemm_const,lds,transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; the hot path has no multi-GPU step "
@@ -322,7 +324,7 @@ HEADLINE_BLOCKS_PER_CU = 1
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in
 # KiB per dispatch), each scaled by what the counter reads for the plain copy kernel of known size
 # (FETCH_SIZE x 2.0000, WRITE_SIZE x 1.0000): profiles/hbm_float4_read_4GiB_traffic.md.
-TRAFFIC_BYTES_PER_LAUNCH = 4295155713
+TRAFFIC_BYTES_PER_LAUNCH = 4295163904
 
 if __name__ == "__main__":
     main()
