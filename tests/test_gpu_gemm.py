@@ -80,3 +80,23 @@ def test_gemm_8192_sampled_tiles(dev, fp8):
     rng = np.random.default_rng(2)
     tiles = [(int(m) * 128, int(n) * 128) for m, n in zip(rng.integers(0, 64, 64), rng.integers(0, 64, 64))]
     _check_tiles(dev, fp8, 8192, 8192, 8192, tiles)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("steps", [1, 2, 3, 4, 5, 6, 7, 11])
+def test_gemm_every_short_k_walk(dev, fp8, steps):
+    """K walks of 1..7 and 11 steps of 128 bytes: the prologue fills up to five ring slots, the
+    steady-state step needs four or more steps, and the last three steps each prefetch less; every
+    combination of those paths has its own K here.  One 256x256 tile, all four 128x128 quarters."""
+    K = steps * (128 if fp8 else 64)
+    _check_tiles(dev, fp8, 256, 256, K, [(0, 0), (0, 128), (128, 0), (128, 128)])
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_gemm_non_square_grid_visits_every_tile_once(dev, fp8):
+    """3 x 5 tiles (15 is not a multiple of the 8 XCDs: the plain tile order) and 8 x 2 tiles (the
+    XCD-banded order with fewer than 4 tile rows per band): every output tile is written, none twice
+    with different data (the output starts as a NaN pattern and every checked tile is finite and right)."""
+    for M, N in ((768, 1280), (2048, 512)):
+        tiles = [(m, n) for m in range(0, M, 256) for n in range(0, N, 256)]
+        _check_tiles(dev, fp8, M, N, 512, tiles)
