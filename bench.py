@@ -160,28 +160,41 @@ def _matrix_rows(dev, wl, add, budget, only):
 
 
 def _gemm_rows(dev, capi, wl, add, budget, constant):
-    # --- GEMM 8192^3 ---------------------------------------------------------------------------
+    # --- GEMM 8192^3: (test, metric, bytes per element, bytes per output, peak key, unit, constant fill byte) ----
     M = N = K = 8192
-    for fp8 in (False, True):
-        eb = 1 if fp8 else 2
-        dA, dB, dC = dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * 2)
-        if fp8:
-            dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, 448.0)
-            dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, 448.0)
-            fn = lambda: dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1 / 448.0, 1 / 448.0)
-        else:
-            dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1)
-            dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+    s43, s52 = 448.0, 57344.0
+    kinds = [("rocblas-fp", "fp16", 2, 2, "f16", "tflops", 0x3c),
+             ("rocblas-fp", "bf16", 2, 2, "bf16", "tflops", 0x3f),
+             ("hipblaslt-fp8", "fp8_e4m3", 1, 2, "fp8", "tflops", 0x38),
+             ("hipblaslt-fp8", "fp8_e5m2", 1, 2, "fp8", "tflops", 0x38),
+             ("rocblas-int", "int8", 1, 4, "int8", "tops", 0x01)]
+    for test, metric, eb, ob, peak, unit, const_byte in kinds:
+        dA, dB, dC = dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * ob)
+        if metric == "fp16":
+            dev.fill_f16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_f16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            fn = lambda: dev.gemm_f16(dA, dB, dC, M, N, K)
+        elif metric == "bf16":
+            dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
             fn = lambda: dev.gemm_bf16(dA, dB, dC, M, N, K)
-        metric = "fp8_e4m3" if fp8 else "bf16"
+        elif metric == "fp8_e4m3":
+            dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, s43)
+            dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, s43)
+            fn = lambda: dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1 / s43, 1 / s43)
+        elif metric == "fp8_e5m2":
+            dev.fill_fp8_e5m2(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, s52)
+            dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, s43)
+            fn = lambda: dev.gemm_fp8_e5m2(dA, dB, dC, M, N, K, 1 / s52, 1 / s43)
+        else:
+            dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
+            fn = lambda: dev.gemm_i8(dA, dB, dC, M, N, K)
         if constant:
-            # the same launch on the reference's buffers (every byte 0x38 / 0x3f, src/rocm/rocblas.cpp:211-212,
-            # src/rocm/hipblaslt_gemm.cpp:271-273): constant operands draw less power, the part holds a higher clock
-            dev.memset(dA, 0x38 if fp8 else 0x3f); dev.memset(dB, 0x38 if fp8 else 0x3f)
+            # the same launch on constant buffers, as the reference fills them (every byte 0x3f / 0x38,
+            # src/rocm/rocblas.cpp:211-212, src/rocm/hipblaslt_gemm.cpp:271-273): constant operands draw less
+            # power and the part holds a higher clock
+            dev.memset(dA, const_byte); dev.memset(dB, const_byte)
             metric += " constant operands"
         us, _ = timed(dev, fn, **budget)
-        add("hipblaslt-fp8" if fp8 else "rocblas-fp", metric, 2.0 * M * N * K / us / 1e6, "tflops", us,
-            PEAK["fp8" if fp8 else "bf16"], shape="8192x8192x8192")
+        add(test, metric, 2.0 * M * N * K / us / 1e6, unit, us, PEAK[peak], shape="8192x8192x8192")
         for b in (dA, dB, dC):
             b.free()
 

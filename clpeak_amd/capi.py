@@ -21,6 +21,7 @@ SYMBOLS = [
     "mi355_mfma_dense", "mi355_smfmac", "mi355_mfma_raw",
     "mi355_gemm_bf16", "mi355_gemm_fp8_e4m3",
     "mi355_local_bandwidth", "mi355_host_alloc", "mi355_host_free", "mi355_copy_async",
+    "mi355_fill_f16", "mi355_fill_fp8_e5m2", "mi355_fill_i8", "mi355_gemm_f16", "mi355_gemm_i8", "mi355_gemm_fp8_e5m2",
 ]
 
 OK, ERR_ARG, ERR_HIP, ERR_NODEV, ERR_ARCH, ERR_OOM = 0, -1, -2, -3, -4, -5
@@ -83,6 +84,12 @@ def load_library(path=LIB_PATH):
     lib.mi355_gemm_bf16.argtypes = [vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_gemm_fp8_e4m3.argtypes = [vp, vp, vp, vp, u32, u32, u32, C.c_float, C.c_float]
     lib.mi355_local_bandwidth.argtypes = [vp, i32, vp, u32, u32, u32]
+    lib.mi355_fill_f16.argtypes = [vp, vp, u64, u64, u32, i32]
+    lib.mi355_fill_fp8_e5m2.argtypes = [vp, vp, u64, u64, u32, i32, C.c_float]
+    lib.mi355_fill_i8.argtypes = [vp, vp, u64, u64, u32]
+    lib.mi355_gemm_f16.argtypes = [vp, vp, vp, vp, u32, u32, u32]
+    lib.mi355_gemm_i8.argtypes = [vp, vp, vp, vp, u32, u32, u32]
+    lib.mi355_gemm_fp8_e5m2.argtypes = [vp, vp, vp, vp, u32, u32, u32, C.c_float, C.c_float]
     lib.mi355_host_alloc.argtypes = [vp, C.c_size_t, C.POINTER(vp)]
     lib.mi355_host_free.argtypes = [vp, vp]
     lib.mi355_copy_async.argtypes = [vp, vp, vp, C.c_size_t, i32]
@@ -186,6 +193,15 @@ class Device:
     def fill_fp8_e4m3(self, buf, n, seed, stream, dist, scale):
         self._check(self.lib.mi355_fill_fp8_e4m3(self.h, buf.ptr, n, seed, stream, dist, scale))
 
+    def fill_f16(self, buf, n, seed, stream, dist):
+        self._check(self.lib.mi355_fill_f16(self.h, buf.ptr, n, seed, stream, dist))
+
+    def fill_fp8_e5m2(self, buf, n, seed, stream, dist, scale):
+        self._check(self.lib.mi355_fill_fp8_e5m2(self.h, buf.ptr, n, seed, stream, dist, scale))
+
+    def fill_i8(self, buf, n, seed, stream):
+        self._check(self.lib.mi355_fill_i8(self.h, buf.ptr, n, seed, stream))
+
     def copy(self, dst, src, nbytes):
         self._check(self.lib.mi355_copy(self.h, dst.ptr, src.ptr, nbytes))
 
@@ -232,6 +248,15 @@ class Device:
 
     def gemm_bf16(self, A, B, Cbuf, M, N, K):
         self._check(self.lib.mi355_gemm_bf16(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K))
+
+    def gemm_f16(self, A, B, Cbuf, M, N, K):
+        self._check(self.lib.mi355_gemm_f16(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K))
+
+    def gemm_i8(self, A, B, Cbuf, M, N, K):
+        self._check(self.lib.mi355_gemm_i8(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K))
+
+    def gemm_fp8_e5m2(self, A, B, Cbuf, M, N, K, scale_a, scale_b):
+        self._check(self.lib.mi355_gemm_fp8_e5m2(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K, scale_a, scale_b))
 
     def gemm_fp8_e4m3(self, A, B, Cbuf, M, N, K, scale_a, scale_b):
         self._check(self.lib.mi355_gemm_fp8_e4m3(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K, scale_a, scale_b))

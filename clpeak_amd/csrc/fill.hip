@@ -32,6 +32,25 @@ __global__ void fill_fp8_kernel(uint8_t *dst, uint64_t n, uint64_t seed, uint32_
     dst[i] = mi355_f32_to_e4m3(draw(seed, stream, i, dist) * scale);
 }
 
+__global__ void fill_f16_kernel(uint16_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    dst[i] = mi355_f32_to_f16(draw(seed, stream, i, dist));
+}
+
+__global__ void fill_e5m2_kernel(uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist,
+                                 float scale) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    dst[i] = mi355_f32_to_e5m2(draw(seed, stream, i, dist) * scale);
+}
+
+__global__ void fill_i8_kernel(int8_t *dst, uint64_t n, uint64_t seed, uint32_t stream) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    dst[i] = (int8_t)((int)(mi355_rng_word(seed, stream, i) >> 60) - 8);
+}
+
 typedef int copy_vec __attribute__((ext_vector_type(4)));
 __global__ void copy_kernel(copy_vec *__restrict__ dst, const copy_vec *__restrict__ src, uint64_t n) {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
@@ -77,6 +96,32 @@ extern "C" int mi355_fill_fp8_e4m3(mi355_dev *dev, uint8_t *dst, uint64_t n, uin
   if (int rc = check_fill(dev, dst, n, dist)) return rc;
   fill_fp8_kernel<<<fill_grid(n), kFillBlock, 0, dev->stream>>>(dst, n, seed, stream, dist, scale);
   MI355_LAUNCH_CHECK(dev, "fill_fp8_e4m3");
+  return MI355_OK;
+}
+
+extern "C" int mi355_fill_f16(mi355_dev *dev, uint16_t *dst, uint64_t n, uint64_t seed, uint32_t stream,
+                              int dist) {
+  MI355_ENTER(dev);
+  if (int rc = check_fill(dev, dst, n, dist)) return rc;
+  fill_f16_kernel<<<fill_grid(n), kFillBlock, 0, dev->stream>>>(dst, n, seed, stream, dist);
+  MI355_LAUNCH_CHECK(dev, "fill_f16");
+  return MI355_OK;
+}
+
+extern "C" int mi355_fill_fp8_e5m2(mi355_dev *dev, uint8_t *dst, uint64_t n, uint64_t seed,
+                                   uint32_t stream, int dist, float scale) {
+  MI355_ENTER(dev);
+  if (int rc = check_fill(dev, dst, n, dist)) return rc;
+  fill_e5m2_kernel<<<fill_grid(n), kFillBlock, 0, dev->stream>>>(dst, n, seed, stream, dist, scale);
+  MI355_LAUNCH_CHECK(dev, "fill_fp8_e5m2");
+  return MI355_OK;
+}
+
+extern "C" int mi355_fill_i8(mi355_dev *dev, int8_t *dst, uint64_t n, uint64_t seed, uint32_t stream) {
+  MI355_ENTER(dev);
+  if (int rc = check_fill(dev, dst, n, MI355_DIST_U01)) return rc;
+  fill_i8_kernel<<<fill_grid(n), kFillBlock, 0, dev->stream>>>(dst, n, seed, stream);
+  MI355_LAUNCH_CHECK(dev, "fill_i8");
   return MI355_OK;
 }
 

@@ -93,6 +93,15 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
 // acc(transposed tile) += B_frag . A_frag^T
 #define MI355_MFMA_BF16(acc, fb, fa) \
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(fb), "v"(fa))
+#define MI355_MFMA_F16(acc, fb, fa) \
+  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(fb), "v"(fa))
+// int8: 16 bytes per lane are K=16 of the 64, the accumulator registers hold int32
+#define MI355_MFMA_I8(acc, fb, fa) \
+  asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc) : "v"(fb), "v"(fa))
+
+// Operand types of the kernel that walks a slab as two K halves (16 bytes per lane and half):
+// bf16 and f16 (K=32 per instruction, fp32 accumulate) and int8 (K=64, int32 accumulate).
+enum { kBf16 = 0, kF16 = 1, kI8 = 2 };
 
 // State of one wave's walk along K that the step function advances.
 struct GemmWalk {
@@ -109,13 +118,18 @@ struct GemmWalk {
 // the MFMA before it, while two in a row would stall the matrix pipe.
 // MAIN: a step of the steady state; otherwise `reads` / `loads` are run-time (wave-uniform)
 // switches for the last steps, which have nothing left to prefetch.
-template <bool MAIN>
+template <bool MAIN, int KIND>
 __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8], bf16x8v (&fb0)[4],
                                           bf16x8v (&fa1)[8], bf16x8v (&fb1)[4], const GemmWalk &w,
                                           bool reads, bool loads_a, bool loads_b) {
   const bool READS = MAIN || reads, LOADS_A = MAIN || loads_a, LOADS_B = MAIN || loads_b;
   const uint32_t a1 = w.a_cur ^ 64u, b1 = w.b_cur ^ 64u;   // second K half of this step
-#define MM(F, i, j) MI355_MFMA_BF16(acc[i][j], F##b##_[j], F##a##_[i])
+#define MM(F, i, j)                                                                                \
+  do {                                                                                             \
+    if (KIND == kBf16) MI355_MFMA_BF16(acc[i][j], F##b##_[j], F##a##_[i]);                         \
+    else if (KIND == kF16) MI355_MFMA_F16(acc[i][j], F##b##_[j], F##a##_[i]);                      \
+    else MI355_MFMA_I8(acc[i][j], F##b##_[j], F##a##_[i]);                                         \
+  } while (0)
 #define LDA(q) if (LOADS_A) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
 #define LDB(q) if (LOADS_B) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
   bf16x8v(&x0a_)[8] = fa0; bf16x8v(&x0b_)[4] = fb0; bf16x8v(&x1a_)[8] = fa1; bf16x8v(&x1b_)[4] = fb1;
@@ -207,8 +221,9 @@ __device__ inline void tile_of_block(uint32_t tiles_m, uint32_t tiles_n, uint32_
   tn = in_group / rows_here;
 }
 
+template <int KIND>
 __global__ void __launch_bounds__(kThreads)
-gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, uint16_t *__restrict__ C,
+gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, void *__restrict__ Cout,
                  uint32_t N, uint32_t k_bytes, uint32_t tiles_m, uint32_t tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const uint32_t tid = threadIdx.x, lane = tid % 64;
@@ -279,21 +294,29 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, u
     w.gb += kRowBytes;
   };
   uint32_t s = 0;
-  for (; s + 3 < steps; s++) { gemm_step<true>(acc, fa0, fb0, fa1, fb1, w, true, true, true); advance(); }
-  for (; s < steps; s++) { gemm_step<false>(acc, fa0, fb0, fa1, fb1, w, s + 1 < steps, false, s + 2 < steps); advance(); }
+  for (; s + 3 < steps; s++) { gemm_step<true, KIND>(acc, fa0, fb0, fa1, fb1, w, true, true, true); advance(); }
+  for (; s < steps; s++) { gemm_step<false, KIND>(acc, fa0, fb0, fa1, fb1, w, s + 1 < steps, false, s + 2 < steps); advance(); }
   // wait states the compiler cannot know about, before the accumulators are read
   asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
-  // --- epilogue: round to bf16, 4 consecutive N elements per lane -----------------------------
+  // --- epilogue: 4 consecutive N elements per lane; bf16 / f16 rounded from fp32, int32 as it is ----
   const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 64u + 4u * (lane / 16u);
 #pragma unroll
   for (int i = 0; i < 8; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      const uint16_t h0 = mi355_f32_to_bf16(acc[i][j][0]), h1 = mi355_f32_to_bf16(acc[i][j][1]);
-      const uint16_t h2 = mi355_f32_to_bf16(acc[i][j][2]), h3 = mi355_f32_to_bf16(acc[i][j][3]);
-      const uint2 packed = make_uint2((uint32_t)h0 | ((uint32_t)h1 << 16), (uint32_t)h2 | ((uint32_t)h3 << 16));
-      *reinterpret_cast<uint2 *>(C + (size_t)(row0 + i * 16u) * N + col0 + j * 16u) = packed;
+      const size_t at = (size_t)(row0 + i * 16u) * N + col0 + j * 16u;
+      if (KIND == kI8) {
+        i32x4v bits;
+        __builtin_memcpy(&bits, &acc[i][j], sizeof(bits));
+        *reinterpret_cast<i32x4v *>(static_cast<int32_t *>(Cout) + at) = bits;
+      } else {
+        uint16_t h[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) h[r] = KIND == kBf16 ? mi355_f32_to_bf16(acc[i][j][r]) : mi355_f32_to_f16(acc[i][j][r]);
+        const uint2 packed = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+        *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(Cout) + at) = packed;
+      }
     }
 }
 
@@ -315,11 +338,16 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, u
 //     MFMA 16..31   (i,2),(i,3): next step's B fragments 0,1 in gaps 16,17, next step's A fragment
 //                   i-1 after row i (a fragment is overwritten no sooner than one instruction after
 //                   its last use); the wave's 4 loads of A rows (slab s+3) in the even gaps 18..24
-#define MI355_MFMA_FP8(acc, blo, bhi, alo, ahi)                                                    \
+// E5M2: the A matrix holds e5m2 codes, B stays e4m3.  A fragments are the second source operand
+// here (transposed product), whose format field is blgp.
+#define MI355_MFMA_FP8(E5M2, acc, blo, bhi, alo, ahi)                                              \
   do {                                                                                             \
     const i32x8v b8_ = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7);                  \
     const i32x8v a8_ = __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);                  \
-    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(acc) : "v"(b8_), "v"(a8_));   \
+    if (E5M2)                                                                                      \
+      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 blgp:1" : "+v"(acc) : "v"(b8_), "v"(a8_));         \
+    else                                                                                           \
+      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(acc) : "v"(b8_), "v"(a8_)); \
   } while (0)
 
 // At most `n` LDS reads still outstanding (they return in order).
@@ -329,12 +357,12 @@ struct Fp8Frags {
   i32x4v a_lo[8], a_hi[8], b_lo[4], b_hi[4];
 };
 
-template <bool MAIN>
+template <bool MAIN, bool E5M2>
 __device__ __forceinline__ void gemm_fp8_step(f32x4v (&acc)[8][4], Fp8Frags &f, const GemmWalk &w, bool reads,
                                               bool loads_a, bool loads_b) {
   const bool READS = MAIN || reads, LOADS_A = MAIN || loads_a, LOADS_B = MAIN || loads_b;
   const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u, an_hi = w.a_nxt ^ 64u, bn_hi = w.b_nxt ^ 64u;
-#define MM(i, j) MI355_MFMA_FP8(acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i])
+#define MM(i, j) MI355_MFMA_FP8(E5M2, acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i])
 #define LDA(q) if (LOADS_A) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
 #define LDB(q) if (LOADS_B) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
 #define RD_A_NEXT(i, off)                                                                          \
@@ -387,6 +415,7 @@ __device__ __forceinline__ void gemm_fp8_step(f32x4v (&acc)[8][4], Fp8Frags &f, 
 #undef MM
 }
 
+template <bool E5M2>
 __global__ void __launch_bounds__(kThreads)
 gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, uint16_t *__restrict__ C,
                 uint32_t N, uint32_t k_bytes, float scale, uint32_t tiles_m, uint32_t tiles_n) {
@@ -464,8 +493,8 @@ gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, ui
     w.gb += kRowBytes;
   };
   uint32_t s = 0;
-  for (; s + 3 < steps; s++) { gemm_fp8_step<true>(acc, f, w, true, true, true); advance(); }
-  for (; s < steps; s++) { gemm_fp8_step<false>(acc, f, w, s + 1 < steps, false, s + 2 < steps); advance(); }
+  for (; s + 3 < steps; s++) { gemm_fp8_step<true, E5M2>(acc, f, w, true, true, true); advance(); }
+  for (; s < steps; s++) { gemm_fp8_step<false, E5M2>(acc, f, w, s + 1 < steps, false, s + 2 < steps); advance(); }
   asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
   const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 64u + 4u * (lane / 16u);
@@ -492,38 +521,67 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
 
 constexpr size_t kRingBytes = 5 * (size_t)kSlabBytes;   // five 32 KiB slots: all 160 KiB of a CU
 
+template <int KIND>
+int launch_halves(mi355_dev *dev, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N,
+                  uint32_t K, uint32_t elem) {
+  if (int rc = check_shapes(dev, A, B, C, M, N, K, elem)) return rc;
+  static bool attr_set = false;
+  if (!attr_set) {
+    MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_bf16_kernel<KIND>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
+    attr_set = true;
+  }
+  const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
+  gemm_bf16_kernel<KIND><<<tiles_m * tiles_n, kThreads, kRingBytes, dev->stream>>>(
+      (const uint8_t *)A, (const uint8_t *)B, C, N, K * elem, tiles_m, tiles_n);
+  MI355_LAUNCH_CHECK(dev, what);
+  return MI355_OK;
+}
+
+template <bool E5M2>
+int launch_fp8(mi355_dev *dev, const char *what, const uint8_t *A, const uint8_t *B, uint16_t *C, uint32_t M,
+               uint32_t N, uint32_t K, float scale) {
+  if (int rc = check_shapes(dev, A, B, C, M, N, K, 1)) return rc;
+  static bool attr_set = false;
+  if (!attr_set) {
+    MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_fp8_kernel<E5M2>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
+    attr_set = true;
+  }
+  const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
+  gemm_fp8_kernel<E5M2><<<tiles_m * tiles_n, kThreads, kRingBytes, dev->stream>>>(A, B, C, N, K, scale, tiles_m, tiles_n);
+  MI355_LAUNCH_CHECK(dev, what);
+  return MI355_OK;
+}
+
 }  // namespace
 
 extern "C" int mi355_gemm_bf16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C, uint32_t M,
                                uint32_t N, uint32_t K) {
   MI355_ENTER(dev);
-  if (int rc = check_shapes(dev, A, B, C, M, N, K, 2)) return rc;
-  static bool attr_set = false;
-  if (!attr_set) {
-    MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_bf16_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
-    attr_set = true;
-  }
-  const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_bf16_kernel<<<tiles_m * tiles_n, kThreads, kRingBytes, dev->stream>>>(
-      (const uint8_t *)A, (const uint8_t *)B, C, N, K * 2u, tiles_m, tiles_n);
-  MI355_LAUNCH_CHECK(dev, "gemm_bf16");
-  return MI355_OK;
+  return launch_halves<kBf16>(dev, "gemm_bf16", A, B, C, M, N, K, 2);
+}
+
+extern "C" int mi355_gemm_f16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C, uint32_t M,
+                              uint32_t N, uint32_t K) {
+  MI355_ENTER(dev);
+  return launch_halves<kF16>(dev, "gemm_f16", A, B, C, M, N, K, 2);
+}
+
+extern "C" int mi355_gemm_i8(mi355_dev *dev, const int8_t *A, const int8_t *B, int32_t *C, uint32_t M, uint32_t N,
+                             uint32_t K) {
+  MI355_ENTER(dev);
+  return launch_halves<kI8>(dev, "gemm_i8", A, B, C, M, N, K, 1);
 }
 
 extern "C" int mi355_gemm_fp8_e4m3(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C, uint32_t M,
                                    uint32_t N, uint32_t K, float scale_a, float scale_b) {
   MI355_ENTER(dev);
-  if (int rc = check_shapes(dev, A, B, C, M, N, K, 1)) return rc;
-  static bool attr_set = false;
-  if (!attr_set) {
-    MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_fp8_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
-    attr_set = true;
-  }
-  const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_fp8_kernel<<<tiles_m * tiles_n, kThreads, kRingBytes, dev->stream>>>(
-      A, B, C, N, K, scale_a * scale_b, tiles_m, tiles_n);
-  MI355_LAUNCH_CHECK(dev, "gemm_fp8_e4m3");
-  return MI355_OK;
+  return launch_fp8<false>(dev, "gemm_fp8_e4m3", A, B, C, M, N, K, scale_a * scale_b);
+}
+
+extern "C" int mi355_gemm_fp8_e5m2(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C, uint32_t M,
+                                   uint32_t N, uint32_t K, float scale_a, float scale_b) {
+  MI355_ENTER(dev);
+  return launch_fp8<true>(dev, "gemm_fp8_e5m2", A, B, C, M, N, K, scale_a * scale_b);
 }

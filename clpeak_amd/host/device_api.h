@@ -32,6 +32,12 @@ struct Mi355Api {
   decltype(&mi355_host_alloc) host_alloc;
   decltype(&mi355_host_free) host_free;
   decltype(&mi355_copy_async) copy_async;
+  decltype(&mi355_fill_f16) fill_f16;
+  decltype(&mi355_fill_fp8_e5m2) fill_fp8_e5m2;
+  decltype(&mi355_fill_i8) fill_i8;
+  decltype(&mi355_gemm_f16) gemm_f16;
+  decltype(&mi355_gemm_i8) gemm_i8;
+  decltype(&mi355_gemm_fp8_e5m2) gemm_fp8_e5m2;
 };
 
 const Mi355Api &mi355_real_api();   // the entry points of libclpeak_mi355.so

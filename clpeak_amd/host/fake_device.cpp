@@ -78,6 +78,12 @@ int f_host_alloc(mi355_dev *d, size_t bytes, void **p) {
 }
 int f_host_free(mi355_dev *, void *p) { free(p); return MI355_OK; }
 int f_copy_async(mi355_dev *d, void *, const void *, size_t, int) { FAKE_ENTRY(d, "copy_async"); return MI355_OK; }
+int f_fill_f16(mi355_dev *d, uint16_t *, uint64_t, uint64_t, uint32_t, int) { FAKE_ENTRY(d, "fill_f16"); return MI355_OK; }
+int f_fill_e5m2(mi355_dev *d, uint8_t *, uint64_t, uint64_t, uint32_t, int, float) { FAKE_ENTRY(d, "fill_fp8_e5m2"); return MI355_OK; }
+int f_fill_i8(mi355_dev *d, int8_t *, uint64_t, uint64_t, uint32_t) { FAKE_ENTRY(d, "fill_i8"); return MI355_OK; }
+int f_gemm_f16(mi355_dev *d, const uint16_t *, const uint16_t *, uint16_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_f16"); return MI355_OK; }
+int f_gemm_i8(mi355_dev *d, const int8_t *, const int8_t *, int32_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_i8"); return MI355_OK; }
+int f_gemm_e5m2(mi355_dev *d, const uint8_t *, const uint8_t *, uint16_t *, uint32_t, uint32_t, uint32_t, float, float) { FAKE_ENTRY(d, "gemm_fp8_e5m2"); return MI355_OK; }
 }  // namespace
 
 const Mi355Api &mi355_fake_api() {
@@ -85,6 +91,7 @@ const Mi355Api &mi355_fake_api() {
       f_device_count, f_open, f_close, f_get_props, f_last_error, f_alloc, f_free, f_upload, f_download, f_sync,
       f_timer_start, f_timer_stop, f_fill_f32, f_fill_bf16, f_fill_fp8, f_global_bandwidth, f_compute_mad,
       f_launch_roundtrip, f_mfma_dense, f_smfmac, f_gemm_bf16, f_gemm_fp8,
-      f_local_bandwidth, f_host_alloc, f_host_free, f_copy_async};
+      f_local_bandwidth, f_host_alloc, f_host_free, f_copy_async,
+      f_fill_f16, f_fill_e5m2, f_fill_i8, f_gemm_f16, f_gemm_i8, f_gemm_e5m2};
   return api;
 }

@@ -381,56 +381,82 @@ void Mi355Peak::runSparseMfma(Category phase) {
 }
 
 // ---- GEMM (the slots of the vendor-library tests) ------------------------------------------------------------------
+// One GEMM row: fill the operands on the device, time the launch like any kernel, emit 2*D^3 / time.
+void Mi355Peak::runGemmRow(logger::TestScope &test, const char *metric, const char *note, size_t elemBytes, size_t outBytes,
+                           const std::function<int(void *, void *)> &fill, const std::function<int(void *, void *, void *)> &launch) {
+  const uint32_t D = workload.gemmDim;
+  Buffer A(api_, dev_, (size_t)D * D * elemBytes), B(api_, dev_, (size_t)D * D * elemBytes), C(api_, dev_, (size_t)D * D * outBytes);
+  if (!(A && B && C) || fill(A.ptr, B.ptr) != MI355_OK) {
+    test.skip(metric, ResultStatus::Error, "Failed to allocate or fill GEMM buffers", note);
+    return;
+  }
+  const float us = runKernel([&] { return launch(A.ptr, B.ptr, C.ptr); }, targetTimeUs, forceIters ? specifiedIters : 0);
+  if (us <= 0.0f) test.skip(metric, ResultStatus::Error, "kernel launch failed", note);
+  else test.emit(metric, (float)(2.0 * D * D * D * 1e6 / us / 1e12), {false, note});
+}
+
 void Mi355Peak::runGemmFp() {
   auto test = device_->beginTest({"rocblas-fp", "rocBLAS GEMM peak", "tflops", Category::Unknown,
-                                  "Square GEMM.  The bf16 row is this backend's hand-written MFMA kernel "
-                                  "(LDS double-buffered 256x256x64 tiles), not a vendor library."});
+                                  "Square GEMM.  The fp16 and bf16 rows are this backend's hand-written MFMA kernel "
+                                  "(256x256 tiles, LDS ring, K contiguous in both operands), not a vendor library."});
   const char *notBuilt = "No hand-written kernel for this type in the MI355X backend (no vendor BLAS is used)";
   test.skip("fp32", ResultStatus::Unsupported, notBuilt);
   test.skip("fp64", ResultStatus::Unsupported, notBuilt);
-  test.skip("fp16", ResultStatus::Unsupported, notBuilt);
   const uint32_t D = workload.gemmDim;
-  Buffer A(api_, dev_, (size_t)D * D * 2), B(api_, dev_, (size_t)D * D * 2), C(api_, dev_, (size_t)D * D * 2);
-  const bool ok = A && B && C &&
-                  api_.fill_bf16(dev_, (uint16_t *)A.ptr, (uint64_t)D * D, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1) == MI355_OK &&
-                  api_.fill_bf16(dev_, (uint16_t *)B.ptr, (uint64_t)D * D, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1) == MI355_OK;
-  if (!ok) {
-    test.skip("bf16", ResultStatus::Error, "Failed to allocate or fill GEMM buffers");
-    return;
-  }
-  const float us = runKernel([&] { return api_.gemm_bf16(dev_, (const uint16_t *)A.ptr, (const uint16_t *)B.ptr, (uint16_t *)C.ptr, D, D, D); },
-                             targetTimeUs, forceIters ? specifiedIters : 0);
-  if (us <= 0.0f) test.skip("bf16", ResultStatus::Error, "kernel launch failed");
-  else test.emit("bf16", (float)(2.0 * D * D * D * 1e6 / us / 1e12), "bf16 inputs, fp32 accumulation, bf16 output; A row-major, B column-major.");
+  const uint64_t n = (uint64_t)D * D;
+  runGemmRow(test, "fp16", "IEEE half inputs, fp32 accumulation, half output; A row-major, B column-major.", 2, 2,
+             [&](void *a, void *b) {
+               const int rc = api_.fill_f16(dev_, (uint16_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
+               return rc != MI355_OK ? rc : api_.fill_f16(dev_, (uint16_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
+             },
+             [&](void *a, void *b, void *c) { return api_.gemm_f16(dev_, (const uint16_t *)a, (const uint16_t *)b, (uint16_t *)c, D, D, D); });
+  runGemmRow(test, "bf16", "bf16 inputs, fp32 accumulation, bf16 output; A row-major, B column-major.", 2, 2,
+             [&](void *a, void *b) {
+               const int rc = api_.fill_bf16(dev_, (uint16_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
+               return rc != MI355_OK ? rc : api_.fill_bf16(dev_, (uint16_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
+             },
+             [&](void *a, void *b, void *c) { return api_.gemm_bf16(dev_, (const uint16_t *)a, (const uint16_t *)b, (uint16_t *)c, D, D, D); });
 }
 
 void Mi355Peak::runGemmFp8() {
   auto test = device_->beginTest({"hipblaslt-fp8", "hipBLASLt FP8 GEMM peak", "tflops", Category::Unknown,
-                                  "Square FP8 GEMM with per-tensor scales.  The e4m3 row is this backend's hand-written "
-                                  "MFMA kernel, not a vendor library."});
+                                  "Square FP8 GEMM with per-tensor scales.  The e4m3 and e5m2 rows are this backend's "
+                                  "hand-written MFMA kernel, not a vendor library."});
   const uint32_t D = workload.gemmDim;
-  const float scale = 448.0f;   // uniform [-1,1) stretched over the e4m3 range
-  {
-    Buffer A(api_, dev_, (size_t)D * D), B(api_, dev_, (size_t)D * D), C(api_, dev_, (size_t)D * D * 2);
-    const bool ok = A && B && C &&
-                    api_.fill_fp8_e4m3(dev_, (uint8_t *)A.ptr, (uint64_t)D * D, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1, scale) == MI355_OK &&
-                    api_.fill_fp8_e4m3(dev_, (uint8_t *)B.ptr, (uint64_t)D * D, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1, scale) == MI355_OK;
-    float us = -1.0f;
-    if (ok)
-      us = runKernel([&] { return api_.gemm_fp8_e4m3(dev_, (const uint8_t *)A.ptr, (const uint8_t *)B.ptr, (uint16_t *)C.ptr, D, D, D, 1.0f / scale, 1.0f / scale); },
-                     targetTimeUs, forceIters ? specifiedIters : 0);
-    if (!ok) test.skip("fp8_e4m3", ResultStatus::Error, "Failed to allocate or fill GEMM buffers");
-    else if (us <= 0.0f) test.skip("fp8_e4m3", ResultStatus::Error, "kernel launch failed");
-    else test.emit("fp8_e4m3", (float)(2.0 * D * D * D * 1e6 / us / 1e12), "OCP e4m3 inputs, per-tensor fp32 scales, fp32 accumulation, bf16 output.");
-  }
-  const char *notBuilt = "No hand-written kernel for this type in the MI355X backend (no vendor BLAS is used)";
-  test.skip("fp8_e5m2", ResultStatus::Unsupported, notBuilt);
-  test.skip("mxf4_e2m1", ResultStatus::Unsupported, notBuilt);
+  const uint64_t n = (uint64_t)D * D;
+  const float s43 = 448.0f, s52 = 57344.0f;   // uniform [-1,1) stretched over the range of the format
+  runGemmRow(test, "fp8_e4m3", "OCP e4m3 inputs, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2,
+             [&](void *a, void *b) {
+               const int rc = api_.fill_fp8_e4m3(dev_, (uint8_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1, s43);
+               return rc != MI355_OK ? rc : api_.fill_fp8_e4m3(dev_, (uint8_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1, s43);
+             },
+             [&](void *a, void *b, void *c) {
+               return api_.gemm_fp8_e4m3(dev_, (const uint8_t *)a, (const uint8_t *)b, (uint16_t *)c, D, D, D, 1.0f / s43, 1.0f / s43);
+             });
+  runGemmRow(test, "fp8_e5m2", "An OCP e5m2 A against an e4m3 B, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2,
+             [&](void *a, void *b) {
+               const int rc = api_.fill_fp8_e5m2(dev_, (uint8_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1, s52);
+               return rc != MI355_OK ? rc : api_.fill_fp8_e4m3(dev_, (uint8_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1, s43);
+             },
+             [&](void *a, void *b, void *c) {
+               return api_.gemm_fp8_e5m2(dev_, (const uint8_t *)a, (const uint8_t *)b, (uint16_t *)c, D, D, D, 1.0f / s52, 1.0f / s43);
+             });
+  test.skip("mxf4_e2m1", ResultStatus::Unsupported,
+            "No hand-written kernel for this type in the MI355X backend (no vendor BLAS is used)");
 }
 
 void Mi355Peak::runGemmInt() {
-  auto test = device_->beginTest({"rocblas-int", "rocBLAS GEMM peak", "tops", Category::Unknown, ""});
-  test.skip("int8", ResultStatus::Unsupported, "No hand-written kernel for this type in the MI355X backend (no vendor BLAS is used)");
+  auto test = device_->beginTest({"rocblas-int", "rocBLAS GEMM peak", "tops", Category::Unknown,
+                                  "Square int8 GEMM with int32 accumulation and output: this backend's hand-written MFMA "
+                                  "kernel, not a vendor library."});
+  const uint32_t D = workload.gemmDim;
+  const uint64_t n = (uint64_t)D * D;
+  runGemmRow(test, "int8", "8-bit integers in [-8, 7], 32-bit totals; A row-major, B column-major.", 1, 4,
+             [&](void *a, void *b) {
+               const int rc = api_.fill_i8(dev_, (int8_t *)a, n, workload.seed, MI355_STREAM_GEMM_A);
+               return rc != MI355_OK ? rc : api_.fill_i8(dev_, (int8_t *)b, n, workload.seed, MI355_STREAM_GEMM_B);
+             },
+             [&](void *a, void *b, void *c) { return api_.gemm_i8(dev_, (const int8_t *)a, (const int8_t *)b, (int32_t *)c, D, D, D); });
 }
 
 // ---- bandwidth, latency ---------------------------------------------------------------------------------------------

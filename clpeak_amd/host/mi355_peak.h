@@ -56,6 +56,8 @@ class Mi355Peak : public Peak {
   void runUnsupportedMatrixRows(Category phase, bool wmma);
   void runMfma(Category phase);
   void runSparseMfma(Category phase);
+  void runGemmRow(logger::TestScope &test, const char *metric, const char *note, size_t elemBytes, size_t outBytes,
+                  const std::function<int(void *, void *)> &fill, const std::function<int(void *, void *, void *)> &launch);
   void runGemmFp();
   void runGemmFp8();
   void runGemmInt();

@@ -94,6 +94,11 @@ int mi355_fill_bf16(mi355_dev *dev, uint16_t *dst, uint64_t n, uint64_t seed, ui
 /* Same values multiplied by `scale` (fp32) then rounded to nearest-even OCP
  * e4m3fn with saturation to +-448 (fp8 GEMM operands). */
 int mi355_fill_fp8_e4m3(mi355_dev *dev, uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist, float scale);
+/* The same for the other GEMM operand types: IEEE half (nearest even), OCP e5m2 with
+ * saturation to +-57344, and int8 = (z >> 60) - 8, uniform in [-8, 7]. */
+int mi355_fill_f16(mi355_dev *dev, uint16_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist);
+int mi355_fill_fp8_e5m2(mi355_dev *dev, uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist, float scale);
+int mi355_fill_i8(mi355_dev *dev, int8_t *dst, uint64_t n, uint64_t seed, uint32_t stream);
 
 /* Plain device-to-device copy kernel (16 bytes per lane, grid-stride).  No counterpart in
  * the reference; it exists so that the HBM byte counters (FETCH_SIZE / WRITE_SIZE) can be
@@ -234,6 +239,19 @@ int mi355_mfma_raw(mi355_dev *dev, int sparse, int kind,
 int mi355_gemm_bf16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C,
                     uint32_t M, uint32_t N, uint32_t K);
 int mi355_gemm_fp8_e4m3(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C,
+                        uint32_t M, uint32_t N, uint32_t K, float scale_a, float scale_b);
+/* The other rows of the same two tests, same layouts and shape rules:
+ *   "fp16" of runRocblas (src/rocm/rocblas.cpp:265-300: half operands, fp32 accumulate):
+ *          C is IEEE half;
+ *   "int8" of runRocblas (src/rocm/rocblas.cpp:309-333: i8 operands, i32 accumulate and output):
+ *          C is int32, K a multiple of 128;
+ *   "fp8_e5m2" of runHipblasLt (src/rocm/hipblaslt_gemm.cpp:393-396: an e5m2 A against an e4m3 B):
+ *          C is bf16 = scale_a*scale_b * (A.B). */
+int mi355_gemm_f16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C,
+                   uint32_t M, uint32_t N, uint32_t K);
+int mi355_gemm_i8(mi355_dev *dev, const int8_t *A, const int8_t *B, int32_t *C,
+                  uint32_t M, uint32_t N, uint32_t K);
+int mi355_gemm_fp8_e5m2(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C,
                         uint32_t M, uint32_t N, uint32_t K, float scale_a, float scale_b);
 
 #ifdef __cplusplus

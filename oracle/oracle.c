@@ -526,26 +526,31 @@ int orc_smfmac(int kind, const void *Ac, const uint8_t *meta, const void *B, voi
 /* GEMM tiles                                                                  */
 /* ------------------------------------------------------------------------- */
 /* C[m][n] = scale * sum_k A[m][k]*B[n][k] for m in [m0,m0+tm), n in [n0,n0+tn), summed
- * in double, returned as double (the test rounds / compares).  fmt: 1 bf16, 2 e4m3fn. */
-int orc_gemm_tile(int fmt, const void *A, const void *B, uint32_t K, uint32_t lda, uint32_t ldb,
-                  uint32_t m0, uint32_t n0, uint32_t tm, uint32_t tn, double scale, double *C)
+ * in double, returned as double (the test rounds / compares).  Operand formats: 0 f16, 1 bf16,
+ * 2 e4m3fn, 3 e5m2, 7 int8 (two's complement); A and B may differ. */
+static int gemm_elem_bytes(int fmt) { return fmt == 0 || fmt == 1 ? 2 : (fmt == 2 || fmt == 3 || fmt == 7 ? 1 : 0); }
+
+static double gemm_elem(int fmt, const uint8_t *p)
 {
-    if (fmt != 1 && fmt != 2) return -1;
-    const int eb = fmt == 1 ? 2 : 1;
+    if (fmt == 7) return (double)(int8_t)p[0];
+    return orc_decode(fmt, gemm_elem_bytes(fmt) == 2 ? (uint32_t)(p[0] | (p[1] << 8)) : p[0]);
+}
+
+int orc_gemm_tile2(int fmt_a, int fmt_b, const void *A, const void *B, uint32_t K, uint32_t lda, uint32_t ldb,
+                   uint32_t m0, uint32_t n0, uint32_t tm, uint32_t tn, double scale, double *C)
+{
+    const int ea = gemm_elem_bytes(fmt_a), eb = gemm_elem_bytes(fmt_b);
+    if (!ea || !eb) return -1;
     /* decode the rows once */
     double *a = (double *)malloc((size_t)tm * K * sizeof(double));
     double *b = (double *)malloc((size_t)tn * K * sizeof(double));
     if (!a || !b) { free(a); free(b); return -3; }
     for (uint32_t i = 0; i < tm; i++)
-        for (uint32_t k = 0; k < K; k++) {
-            const uint8_t *p = (const uint8_t *)A + ((size_t)(m0 + i) * lda + k) * eb;
-            a[(size_t)i * K + k] = orc_decode(fmt, eb == 2 ? (uint32_t)(p[0] | (p[1] << 8)) : p[0]);
-        }
+        for (uint32_t k = 0; k < K; k++)
+            a[(size_t)i * K + k] = gemm_elem(fmt_a, (const uint8_t *)A + ((size_t)(m0 + i) * lda + k) * (size_t)ea);
     for (uint32_t j = 0; j < tn; j++)
-        for (uint32_t k = 0; k < K; k++) {
-            const uint8_t *p = (const uint8_t *)B + ((size_t)(n0 + j) * ldb + k) * eb;
-            b[(size_t)j * K + k] = orc_decode(fmt, eb == 2 ? (uint32_t)(p[0] | (p[1] << 8)) : p[0]);
-        }
+        for (uint32_t k = 0; k < K; k++)
+            b[(size_t)j * K + k] = gemm_elem(fmt_b, (const uint8_t *)B + ((size_t)(n0 + j) * ldb + k) * (size_t)eb);
     #pragma omp parallel for schedule(static)
     for (uint32_t i = 0; i < tm; i++)
         for (uint32_t j = 0; j < tn; j++) {
@@ -557,6 +562,13 @@ int orc_gemm_tile(int fmt, const void *A, const void *B, uint32_t K, uint32_t ld
     free(a);
     free(b);
     return 0;
+}
+
+int orc_gemm_tile(int fmt, const void *A, const void *B, uint32_t K, uint32_t lda, uint32_t ldb,
+                  uint32_t m0, uint32_t n0, uint32_t tm, uint32_t tn, double scale, double *C)
+{
+    if (fmt != 1 && fmt != 2) return -1;
+    return orc_gemm_tile2(fmt, fmt, A, B, K, lda, ldb, m0, n0, tm, tn, scale, C);
 }
 
 /* ------------------------------------------------------------------------- */
@@ -623,6 +635,20 @@ void orc_fill_e4m3(uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int
         const uint64_t z = orc_rng_word(seed, stream, first + i);
         const float v = (dist == 0 ? u01_of(z) : upm1_of(z)) * scale; /* fp32 product, as on the device */
         dst[i] = (uint8_t)fmt_encode(&FMT_E4M3, (double)v);
+    }
+}
+
+/* Any of the formats 0 f16, 1 bf16, 2 e4m3fn, 3 e5m2: encode(fmt, fp32(u * scale)), as the device fills. */
+void orc_fill_fmt(int fmt, void *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist, float scale, uint64_t first)
+{
+    const orc_fmt *f = fmt_by_id(fmt);
+    #pragma omp parallel for schedule(static)
+    for (uint64_t i = 0; i < n; i++) {
+        const uint64_t z = orc_rng_word(seed, stream, first + i);
+        const float v = (dist == 0 ? u01_of(z) : upm1_of(z)) * scale;
+        const uint32_t code = fmt_encode(f, (double)v);
+        if (fmt <= 1) ((uint16_t *)dst)[i] = (uint16_t)code;
+        else ((uint8_t *)dst)[i] = (uint8_t)code;
     }
 }
 

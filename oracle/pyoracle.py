@@ -124,6 +124,29 @@ def gemm_tile(fmt, A, B, K, lda, ldb, m0, n0, tm, tn, scale=1.0):
     return out
 
 
+def gemm_tile2(fmt_a, fmt_b, A, B, K, lda, ldb, m0, n0, tm, tn, scale=1.0):
+    """fmt: FMT_F16 / FMT_BF16 / FMT_E4M3 / FMT_E5M2 or FMT_I8; A and B may differ."""
+    out = np.empty((tm, tn), dtype=np.float64)
+    L = lib()
+    L.orc_gemm_tile2.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p] + [C.c_uint32] * 7 + [C.c_double, C.c_void_p]
+    L.orc_gemm_tile2.restype = C.c_int
+    rc = L.orc_gemm_tile2(fmt_a, fmt_b, A.ctypes.data, B.ctypes.data, K, lda, ldb, m0, n0, tm, tn, scale, out.ctypes.data)
+    assert rc == 0, rc
+    return out
+
+
+FMT_I8 = 7
+
+
+def fill_fmt(fmt, n, seed, stream, dist, scale=1.0, first=0):
+    out = np.empty(n, dtype=np.uint16 if fmt <= FMT_BF16 else np.uint8)
+    L = lib()
+    L.orc_fill_fmt.argtypes = [C.c_int, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint32, C.c_int, C.c_float, C.c_uint64]
+    L.orc_fill_fmt.restype = None
+    L.orc_fill_fmt(fmt, out.ctypes.data, n, seed, stream, dist, scale, first)
+    return out
+
+
 def _bind_builders():
     L = lib()
     if getattr(L, "_builders_bound", False):

@@ -63,6 +63,23 @@ def test_fill_bf16_and_fp8_bit_exact(dev):
     b16.free(); b8.free()
 
 
+def test_fill_f16_e5m2_i8_bit_exact(dev):
+    n = (1 << 18) + 7
+    b16 = dev.alloc(n * 2)
+    for dist in (0, 1):
+        dev.fill_f16(b16, n, SEED, wl.STREAM_GEMM_A, dist)
+        assert np.array_equal(b16.download(np.uint16, n), orc.fill_fmt(orc.FMT_F16, n, SEED, wl.STREAM_GEMM_A, dist))
+    b8 = dev.alloc(n)
+    for scale in (1.0, 3.0, 57344.0, 1e6):   # the last one exercises saturation at 57344
+        dev.fill_fp8_e5m2(b8, n, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, scale)
+        want = orc.fill_fmt(orc.FMT_E5M2, n, SEED, wl.STREAM_GEMM_B, 1, scale)
+        assert np.array_equal(b8.download(np.uint8, n), want), scale
+    dev.fill_i8(b8, n, SEED, wl.STREAM_GEMM_A)
+    got = b8.download(np.int8, n)
+    assert np.array_equal(got, orc.fill_int8(SEED, wl.STREAM_GEMM_A, n)) and got.min() == -8 and got.max() == 7
+    b16.free(); b8.free()
+
+
 def test_copy_kernel(dev):
     n = (1 << 20) + 16
     src = dev.from_host(orc.fill_f32(n, SEED, 3, 0))

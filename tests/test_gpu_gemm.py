@@ -100,3 +100,67 @@ def test_gemm_non_square_grid_visits_every_tile_once(dev, fp8):
     for M, N in ((768, 1280), (2048, 512)):
         tiles = [(m, n) for m in range(0, M, 256) for n in range(0, N, 256)]
         _check_tiles(dev, fp8, M, N, 512, tiles)
+
+
+# --- the other operand types of the same two kernels -------------------------------------------------
+E5M2_SCALE = 57344.0
+
+
+def _check_kind(dev, kind, M, N, K, tiles, tile=128):
+    """kind in f16 / i8 / e5m2 (an e5m2 A against an e4m3 B).  int8 is compared bit for bit."""
+    eb = 2 if kind == "f16" else 1
+    dA, dB = dev.alloc(M * K * eb), dev.alloc(N * K * eb)
+    dC = dev.alloc(M * N * (4 if kind == "i8" else 2))
+    dev.memset(dC, 0xff)
+    if kind == "f16":
+        dev.fill_f16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1)
+        dev.fill_f16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+        dev.gemm_f16(dA, dB, dC, M, N, K)
+        fa = fb = orc.FMT_F16; scale = 1.0
+    elif kind == "i8":
+        dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A)
+        dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
+        dev.gemm_i8(dA, dB, dC, M, N, K)
+        fa = fb = orc.FMT_I8; scale = 1.0
+    else:
+        dev.fill_fp8_e5m2(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, E5M2_SCALE)
+        dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, FP8_SCALE)
+        dev.gemm_fp8_e5m2(dA, dB, dC, M, N, K, 1.0 / E5M2_SCALE, 1.0 / FP8_SCALE)
+        fa, fb = orc.FMT_E5M2, orc.FMT_E4M3; scale = 1.0 / (E5M2_SCALE * FP8_SCALE)
+    in_dt = np.uint16 if eb == 2 else np.uint8
+    for (m0, n0) in tiles:
+        a = dA.download(in_dt, tile * K, offset_bytes=m0 * K * eb)
+        b = dB.download(in_dt, tile * K, offset_bytes=n0 * K * eb)
+        ref = orc.gemm_tile2(fa, fb, a, b, K, K, K, 0, 0, tile, tile, scale)
+        got = np.empty((tile, tile), dtype=np.float64)
+        for i in range(tile):
+            if kind == "i8":
+                got[i] = dC.download(np.int32, tile, offset_bytes=((m0 + i) * N + n0) * 4)
+            elif kind == "f16":
+                got[i] = dC.download(np.float16, tile, offset_bytes=((m0 + i) * N + n0) * 2)
+            else:
+                row = dC.download(np.uint16, tile, offset_bytes=((m0 + i) * N + n0) * 2)
+                got[i] = (row.astype(np.uint32) << 16).view(np.float32)
+        assert np.all(np.isfinite(got)), (m0, n0)
+        if kind == "i8":
+            assert np.array_equal(got, ref), (m0, n0)      # integers: exact in double, exact on the GPU
+        else:
+            rms = float(np.sqrt((ref ** 2).mean()))
+            err = np.abs(got - ref)
+            assert np.all(err <= 1e-2 * np.abs(ref) + 1e-2 * rms), (m0, n0, float(err.max()), rms)
+    for b in (dA, dB, dC):
+        b.free()
+
+
+@pytest.mark.parametrize("kind", ["f16", "i8", "e5m2"])
+@pytest.mark.parametrize("steps", [1, 2, 3, 4, 5, 9])
+def test_gemm_other_types_short_walks(dev, kind, steps):
+    K = steps * (64 if kind == "f16" else 128)
+    _check_kind(dev, kind, 256, 256, K, [(0, 0), (0, 128), (128, 0), (128, 128)])
+
+
+@pytest.mark.parametrize("kind", ["f16", "i8", "e5m2"])
+def test_gemm_other_types_8192_sampled_tiles(dev, kind):
+    rng = np.random.default_rng(3)
+    tiles = [(int(m) * 128, int(n) * 128) for m, n in zip(rng.integers(0, 64, 12), rng.integers(0, 64, 12))]
+    _check_kind(dev, kind, 8192, 8192, 8192, tiles)

@@ -316,3 +316,42 @@ def test_local_bandwidth_large_indices_round_like_a_float_conversion():
     # thread ids above 2^24 are not exact in fp32: the start value is the rounded conversion
     got = orc.local_bandwidth(1, (1 << 24) // 256 + 2, 256, 0)
     assert got[-1] == np.float32((1 << 24) + 511) and got[(1 << 24) + 1] == np.float32(1 << 24)
+
+
+# --- GEMM tiles with mixed operand formats, generic fills -------------------------------------------
+def test_gemm_tile2_int8_and_mixed_formats_against_numpy():
+    rng = np.random.default_rng(0)
+    a = rng.integers(-8, 8, (4, 256), dtype=np.int8)
+    b = rng.integers(-8, 8, (5, 256), dtype=np.int8)
+    got = orc.gemm_tile2(orc.FMT_I8, orc.FMT_I8, a, b, 256, 256, 256, 0, 0, 4, 5)
+    assert np.array_equal(got, a.astype(np.int64) @ b.astype(np.int64).T)
+    # an e5m2 A against an e4m3 B (finite codes only), offsets and a scale: transposing the operands or
+    # swapping the two decoders changes the result
+    ca = rng.integers(0, 256, (6, 128), dtype=np.uint8)
+    cb = rng.integers(0, 256, (7, 128), dtype=np.uint8)
+    ca[(ca & 0x7f) > 0x7b] = 0x3c
+    cb[(cb & 0x7f) == 0x7f] = 0x38
+    got = orc.gemm_tile2(orc.FMT_E5M2, orc.FMT_E4M3, ca, cb, 128, 128, 128, 2, 3, 3, 2, 0.5)
+    want = 0.5 * (orc.decode(orc.FMT_E5M2, ca[2:5]) @ orc.decode(orc.FMT_E4M3, cb[3:5]).T)
+    assert np.allclose(got, want, rtol=1e-12, atol=0)
+    swapped = 0.5 * (orc.decode(orc.FMT_E4M3, ca[2:5]) @ orc.decode(orc.FMT_E5M2, cb[3:5]).T)
+    assert not np.allclose(got, swapped)
+    # f16 against numpy's own half decoding
+    ha = rng.standard_normal((3, 64)).astype(np.float16)
+    hb = rng.standard_normal((4, 64)).astype(np.float16)
+    got = orc.gemm_tile2(orc.FMT_F16, orc.FMT_F16, ha.view(np.uint16), hb.view(np.uint16), 64, 64, 64, 0, 0, 3, 4)
+    assert np.allclose(got, ha.astype(np.float64) @ hb.astype(np.float64).T, rtol=1e-12)
+
+
+def test_generic_fill_matches_library_roundings():
+    import torch
+    n = 20000
+    u = orc.fill_f32(n, wl.DEFAULT_SEED, wl.STREAM_GEMM_A, 1)
+    assert np.array_equal(orc.fill_fmt(orc.FMT_F16, n, wl.DEFAULT_SEED, wl.STREAM_GEMM_A, 1), u.astype(np.float16).view(np.uint16))
+    assert np.array_equal(orc.fill_fmt(orc.FMT_BF16, n, wl.DEFAULT_SEED, wl.STREAM_GEMM_A, 1), orc.fill_bf16(n, wl.DEFAULT_SEED, wl.STREAM_GEMM_A, 1))
+    for scale in (1.0, 3.0, 57344.0):
+        want = (torch.from_numpy(u) * scale).to(torch.float8_e5m2).view(torch.uint8).numpy()
+        assert np.array_equal(orc.fill_fmt(orc.FMT_E5M2, n, wl.DEFAULT_SEED, wl.STREAM_GEMM_A, 1, scale), want), scale
+    # beyond the largest finite value the fill saturates (torch would give inf there)
+    sat = orc.fill_fmt(orc.FMT_E5M2, n, wl.DEFAULT_SEED, wl.STREAM_GEMM_A, 1, 1e6)
+    assert set(np.unique(sat & 0x7f)) <= set(range(0x7c)) and (sat & 0x7f).max() == 0x7b
