@@ -46,22 +46,33 @@ def kernel_body(asm, name):
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
-def test_gemm_bf16_fits_the_register_file(tmp_path):
+def test_gemm_kernels_fit_the_register_file(tmp_path):
     asm = device_asm(tmp_path, "gemm.hip")
     meta = kernel_metadata(asm)
-    name = next(k for k in meta if "gemm_bf16_kernel" in k)
-    m = meta[name]
-    assert m["vgpr_spill_count"] == 0, m
-    assert m["private_segment_fixed_size"] == 0, m
-    # 8 waves per workgroup, 2 per SIMD: at most 256 registers each
-    assert m["vgpr_count"] <= 256, m
-    body = kernel_body(asm, name)
-    # two instances of the step (steady state and tail), 64 MFMAs each, and nothing else
-    assert body.count("v_mfma_f32_16x16x32_bf16") == 128
-    # the direct-to-LDS loads: 8 in the prologue halves (2 slabs) + 8 per steady-state step
-    assert body.count("global_load_lds_dwordx4") >= 8 + 8
-    # no LDS stores at all on this path
-    assert "ds_write" not in body
+    # (kernel template, instantiation tag in the mangled name) -> the matrix instruction of its loop and how
+    # many of them two instances of the step (steady state and tail) hold
+    expect = {("gemm_bf16_kernel", "ILi0E"): ("v_mfma_f32_16x16x32_bf16", 128),
+              ("gemm_bf16_kernel", "ILi1E"): ("v_mfma_f32_16x16x32_f16", 128),
+              ("gemm_bf16_kernel", "ILi2E"): ("v_mfma_i32_16x16x64_i8", 128),
+              ("gemm_fp8_kernel", "ILb0E"): ("v_mfma_f32_16x16x128_f8f6f4", 64),
+              ("gemm_fp8_kernel", "ILb1E"): ("v_mfma_f32_16x16x128_f8f6f4", 64)}
+    for (kernel, tag), (insn, count) in expect.items():
+        name = next(k for k in meta if kernel + tag in k)
+        m = meta[name]
+        assert m["vgpr_spill_count"] == 0, (name, m)
+        assert m["private_segment_fixed_size"] == 0, (name, m)
+        # 8 waves per workgroup, 2 per SIMD: at most 256 registers each
+        assert m["vgpr_count"] <= 256, (name, m)
+        # the whole LDS of a CU is requested at launch (dynamic), none statically
+        assert m.get("group_segment_fixed_size", 0) == 0, (name, m)
+        body = kernel_body(asm, name)
+        assert body.count(insn) == count, (name, body.count(insn))
+        if tag == "ILb1E":
+            assert body.count("blgp:1") == count      # the e5m2 operand is the second source
+        # the direct-to-LDS loads: 20 in the prologue (five ring slots) + 8 per steady-state step
+        assert body.count("global_load_lds_dwordx4") >= 20 + 8, name
+        # no LDS stores at all on this path
+        assert "ds_write" not in body, name
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
