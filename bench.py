@@ -199,6 +199,47 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
             b.free()
 
 
+def _llc_bytes():
+    """Total last-level cache of the machine: the sum of the distinct L3 caches sysfs lists."""
+    seen, total = set(), 0
+    base = "/sys/devices/system/cpu"
+    try:
+        cpus = [d for d in os.listdir(base) if d.startswith("cpu") and d[3:].isdigit()]
+    except OSError:
+        return 0
+    for c in cpus:
+        d = os.path.join(base, c, "cache", "index3")
+        try:
+            shared = open(os.path.join(d, "shared_cpu_list")).read().strip()
+            size = open(os.path.join(d, "size")).read().strip()
+        except OSError:
+            continue
+        if shared in seen:
+            continue
+        seen.add(shared)
+        mult = {"K": 1 << 10, "M": 1 << 20, "G": 1 << 30}.get(size[-1].upper(), 1)
+        total += int(size[:-1] if size[-1].isalpha() else size) * mult
+    return total
+
+
+def _stream_floats(threads):
+    """Array length of the DRAM test, the reference's rule (src/cpu/bandwidth.cpp:250-265): four times the
+    last-level cache, at least 64 MiB, at most 512 MiB unless that is less than twice the cache."""
+    llc = _llc_bytes()
+    array_bytes = max(4 * llc, 64 << 20)
+    try:
+        total_mem = os.sysconf("SC_PAGE_SIZE") * os.sysconf("SC_PHYS_PAGES")
+    except (ValueError, OSError):
+        total_mem = 0
+    cap = min(512 << 20, total_mem // 16) if total_mem else 512 << 20
+    if cap < 2 * llc:
+        cap = 2 * llc
+    # A virtual machine can under-report its caches (one 32 MiB L3 for 16 vCPUs that really sit on several
+    # chiplets), which would leave every thread's chunk cache-resident: never go below 2 GiB.
+    n = max(min(array_bytes, cap), 2 << 30) // 4
+    return max(n // threads * threads, threads), llc
+
+
 def cpu_baseline(target_us=2_000_000, extra_target_us=1_000_000):
     """CPU figures beside the GPU ones, all timed with the reference's CPU discipline (pinned persistent
     pool, warm-ups, settle phase before the all-core run, adaptive probe, one timed batch sized to the
@@ -229,7 +270,8 @@ def cpu_baseline(target_us=2_000_000, extra_target_us=1_000_000):
                           "iters_ST": q.iters_st, "iters_MT": q.iters_mt, "sample": what}
         reference = None
         if ref is not None:
-            rd = pool.measure_read_fn(ref["read_fn"], ref["populate_fn"], 1 << 26, 2, target_us)
+            n_stream, llc = _stream_floats(cores)
+            rd = pool.measure_read_fn(ref["read_fn"], ref["populate_fn"], n_stream, 2, target_us)
             ch = pool.measure_chain_fn(ref["fp32_fn"], ref["fp32_ops"], 2, extra_target_us)
             reference = {"isa": ref["isa"],
                          "global_memory_bandwidth read": {"ST": round(rd.giga_st, 2), "MT": round(rd.giga_mt, 2), "unit": "GB/s",
@@ -239,8 +281,9 @@ def cpu_baseline(target_us=2_000_000, extra_target_us=1_000_000):
     dt = time.perf_counter() - t0
     if reference is not None:
         value, kind = reference["global_memory_bandwidth read"]["MT"], "reference"
-        sample = (f"the reference's DRAM read kernel (readBufferChecksum, {ref['isa']} build of its own source) over a 256 MiB "
-                  f"array filled by its populate(), per-thread contiguous chunks: {rd.iters_st} passes on 1 thread, "
+        sample = (f"the reference's DRAM read kernel (readBufferChecksum, {ref['isa']} build of its own source) over a "
+                  f"{n_stream * 4 >> 20} MiB array (its sizing rule but at least 2 GiB; reported last-level cache {llc >> 20} MiB) filled by its populate(), "
+                  f"per-thread contiguous chunks: {rd.iters_st} passes on 1 thread, "
                   f"{rd.iters_mt} passes on {rd.threads_mt} threads; whole CPU leg {dt:.1f} s")
     else:
         value, kind = port["global_memory_bandwidth float4"]["MT"], "port"
