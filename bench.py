@@ -167,10 +167,20 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
              ("rocblas-fp", "bf16", 2, 2, "bf16", "tflops", 0x3f),
              ("hipblaslt-fp8", "fp8_e4m3", 1, 2, "fp8", "tflops", 0x38),
              ("hipblaslt-fp8", "fp8_e5m2", 1, 2, "fp8", "tflops", 0x38),
+             ("hipblaslt-fp8", "mxf4_e2m1", 0.5, 2, "fp4", "tflops", 0x22),
              ("rocblas-int", "int8", 1, 4, "int8", "tops", 0x01)]
     for test, metric, eb, ob, peak, unit, const_byte in kinds:
-        dA, dB, dC = dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * ob)
-        if metric == "fp16":
+        dA, dB, dC = dev.alloc(int(M * K * eb)), dev.alloc(int(N * K * eb)), dev.alloc(M * N * ob)
+        extra = []
+        if metric == "mxf4_e2m1":
+            dSA, dSB = dev.alloc(M * K // 32), dev.alloc(N * K // 32)
+            extra = [dSA, dSB]
+            dev.fill_bytes(dA, M * K // 2, SEED, wl.STREAM_GEMM_A, 0, 256); dev.fill_bytes(dB, N * K // 2, SEED, wl.STREAM_GEMM_B, 0, 256)
+            dev.fill_bytes(dSA, M * K // 32, SEED, wl.STREAM_SCALE_A, 123, 9); dev.fill_bytes(dSB, N * K // 32, SEED, wl.STREAM_SCALE_B, 123, 9)
+            if constant:
+                dev.memset(dSA, 0x7f); dev.memset(dSB, 0x7f)
+            fn = lambda: dev.gemm_mxfp4(dA, dB, dSA, dSB, dC, M, N, K)
+        elif metric == "fp16":
             dev.fill_f16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_f16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
             fn = lambda: dev.gemm_f16(dA, dB, dC, M, N, K)
         elif metric == "bf16":

@@ -22,6 +22,7 @@ SYMBOLS = [
     "mi355_gemm_bf16", "mi355_gemm_fp8_e4m3",
     "mi355_local_bandwidth", "mi355_host_alloc", "mi355_host_free", "mi355_copy_async",
     "mi355_fill_f16", "mi355_fill_fp8_e5m2", "mi355_fill_i8", "mi355_gemm_f16", "mi355_gemm_i8", "mi355_gemm_fp8_e5m2",
+    "mi355_gemm_mxfp4", "mi355_fill_bytes",
 ]
 
 OK, ERR_ARG, ERR_HIP, ERR_NODEV, ERR_ARCH, ERR_OOM = 0, -1, -2, -3, -4, -5
@@ -90,6 +91,8 @@ def load_library(path=LIB_PATH):
     lib.mi355_gemm_f16.argtypes = [vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_gemm_i8.argtypes = [vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_gemm_fp8_e5m2.argtypes = [vp, vp, vp, vp, u32, u32, u32, C.c_float, C.c_float]
+    lib.mi355_gemm_mxfp4.argtypes = [vp, vp, vp, vp, vp, vp, u32, u32, u32]
+    lib.mi355_fill_bytes.argtypes = [vp, vp, u64, u64, u32, u32, u32]
     lib.mi355_host_alloc.argtypes = [vp, C.c_size_t, C.POINTER(vp)]
     lib.mi355_host_free.argtypes = [vp, vp]
     lib.mi355_copy_async.argtypes = [vp, vp, vp, C.c_size_t, i32]
@@ -248,6 +251,12 @@ class Device:
 
     def gemm_bf16(self, A, B, Cbuf, M, N, K):
         self._check(self.lib.mi355_gemm_bf16(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K))
+
+    def gemm_mxfp4(self, A, B, SA, SB, Cbuf, M, N, K):
+        self._check(self.lib.mi355_gemm_mxfp4(self.h, A.ptr, B.ptr, SA.ptr, SB.ptr, Cbuf.ptr, M, N, K))
+
+    def fill_bytes(self, buf, n, seed, stream, lo, span):
+        self._check(self.lib.mi355_fill_bytes(self.h, buf.ptr, n, seed, stream, lo, span))
 
     def gemm_f16(self, A, B, Cbuf, M, N, K):
         self._check(self.lib.mi355_gemm_f16(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K))

@@ -88,6 +88,7 @@ extern "C" int mi355_close(mi355_dev *dev) {
   if (!dev) return MI355_OK;
   (void)hipSetDevice(dev->ordinal);
   if (dev->stream) (void)hipStreamSynchronize(dev->stream);
+  if (dev->mx_scratch) (void)hipFree(dev->mx_scratch);
   if (dev->ev_start) (void)hipEventDestroy(dev->ev_start);
   if (dev->ev_stop) (void)hipEventDestroy(dev->ev_stop);
   if (dev->stream) (void)hipStreamDestroy(dev->stream);

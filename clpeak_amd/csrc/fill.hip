@@ -51,6 +51,12 @@ __global__ void fill_i8_kernel(int8_t *dst, uint64_t n, uint64_t seed, uint32_t 
     dst[i] = (int8_t)((int)(mi355_rng_word(seed, stream, i) >> 60) - 8);
 }
 
+__global__ void fill_bytes_kernel(uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream, uint32_t lo, uint32_t span) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    dst[i] = (uint8_t)(lo + mi355_rng_below(mi355_rng_word(seed, stream, i), span));
+}
+
 typedef int copy_vec __attribute__((ext_vector_type(4)));
 __global__ void copy_kernel(copy_vec *__restrict__ dst, const copy_vec *__restrict__ src, uint64_t n) {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
@@ -122,6 +128,16 @@ extern "C" int mi355_fill_i8(mi355_dev *dev, int8_t *dst, uint64_t n, uint64_t s
   if (int rc = check_fill(dev, dst, n, MI355_DIST_U01)) return rc;
   fill_i8_kernel<<<fill_grid(n), kFillBlock, 0, dev->stream>>>(dst, n, seed, stream);
   MI355_LAUNCH_CHECK(dev, "fill_i8");
+  return MI355_OK;
+}
+
+extern "C" int mi355_fill_bytes(mi355_dev *dev, uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream,
+                                uint32_t lo, uint32_t span) {
+  MI355_ENTER(dev);
+  if (int rc = check_fill(dev, dst, n, MI355_DIST_U01)) return rc;
+  MI355_REQUIRE(dev, span >= 1 && lo + span <= 256, "fill_bytes: [lo, lo+span) must lie within a byte");
+  fill_bytes_kernel<<<fill_grid(n), kFillBlock, 0, dev->stream>>>(dst, n, seed, stream, lo, span);
+  MI355_LAUNCH_CHECK(dev, "fill_bytes");
   return MI355_OK;
 }
 

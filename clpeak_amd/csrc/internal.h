@@ -13,6 +13,9 @@ struct mi355_dev {
   hipEvent_t   ev_stop   = nullptr;
   mi355_props_t props{};
   std::string  last_error;
+  // scratch owned by the handle: scale bytes of the block-scaled GEMM laid out per lane (grown on demand)
+  void        *mx_scratch = nullptr;
+  size_t       mx_scratch_bytes = 0;
 };
 
 // Error text for failures that have no handle to hang on (open, device_count).

@@ -38,6 +38,8 @@ struct Mi355Api {
   decltype(&mi355_gemm_f16) gemm_f16;
   decltype(&mi355_gemm_i8) gemm_i8;
   decltype(&mi355_gemm_fp8_e5m2) gemm_fp8_e5m2;
+  decltype(&mi355_gemm_mxfp4) gemm_mxfp4;
+  decltype(&mi355_fill_bytes) fill_bytes;
 };
 
 const Mi355Api &mi355_real_api();   // the entry points of libclpeak_mi355.so

@@ -84,6 +84,8 @@ int f_fill_i8(mi355_dev *d, int8_t *, uint64_t, uint64_t, uint32_t) { FAKE_ENTRY
 int f_gemm_f16(mi355_dev *d, const uint16_t *, const uint16_t *, uint16_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_f16"); return MI355_OK; }
 int f_gemm_i8(mi355_dev *d, const int8_t *, const int8_t *, int32_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_i8"); return MI355_OK; }
 int f_gemm_e5m2(mi355_dev *d, const uint8_t *, const uint8_t *, uint16_t *, uint32_t, uint32_t, uint32_t, float, float) { FAKE_ENTRY(d, "gemm_fp8_e5m2"); return MI355_OK; }
+int f_gemm_mxfp4(mi355_dev *d, const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *, uint16_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_mxfp4"); return MI355_OK; }
+int f_fill_bytes(mi355_dev *d, uint8_t *, uint64_t, uint64_t, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "fill_bytes"); return MI355_OK; }
 }  // namespace
 
 const Mi355Api &mi355_fake_api() {
@@ -92,6 +94,7 @@ const Mi355Api &mi355_fake_api() {
       f_timer_start, f_timer_stop, f_fill_f32, f_fill_bf16, f_fill_fp8, f_global_bandwidth, f_compute_mad,
       f_launch_roundtrip, f_mfma_dense, f_smfmac, f_gemm_bf16, f_gemm_fp8,
       f_local_bandwidth, f_host_alloc, f_host_free, f_copy_async,
-      f_fill_f16, f_fill_e5m2, f_fill_i8, f_gemm_f16, f_gemm_i8, f_gemm_e5m2};
+      f_fill_f16, f_fill_e5m2, f_fill_i8, f_gemm_f16, f_gemm_i8, f_gemm_e5m2,
+      f_gemm_mxfp4, f_fill_bytes};
   return api;
 }

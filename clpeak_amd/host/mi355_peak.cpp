@@ -420,8 +420,8 @@ void Mi355Peak::runGemmFp() {
 
 void Mi355Peak::runGemmFp8() {
   auto test = device_->beginTest({"hipblaslt-fp8", "hipBLASLt FP8 GEMM peak", "tflops", Category::Unknown,
-                                  "Square FP8 GEMM with per-tensor scales.  The e4m3 and e5m2 rows are this backend's "
-                                  "hand-written MFMA kernel, not a vendor library."});
+                                  "Square FP8 / FP4 GEMM with per-tensor or per-block scales: this backend's hand-written MFMA kernels, "
+                                  "not a vendor library."});
   const uint32_t D = workload.gemmDim;
   const uint64_t n = (uint64_t)D * D;
   const float s43 = 448.0f, s52 = 57344.0f;   // uniform [-1,1) stretched over the range of the format
@@ -441,8 +441,25 @@ void Mi355Peak::runGemmFp8() {
              [&](void *a, void *b, void *c) {
                return api_.gemm_fp8_e5m2(dev_, (const uint8_t *)a, (const uint8_t *)b, (uint16_t *)c, D, D, D, 1.0f / s52, 1.0f / s43);
              });
-  test.skip("mxf4_e2m1", ResultStatus::Unsupported,
-            "No hand-written kernel for this type in the MI355X backend (no vendor BLAS is used)");
+  // block-scaled FP4: two e2m1 codes per byte, one E8M0 scale per 32 elements (2^-4 .. 2^4)
+  const char *mxNote = "OCP MXFP4: e2m1 inputs with one E8M0 scale per 32 elements along K, fp32 accumulation, bf16 output.";
+  {
+    Buffer A(api_, dev_, (size_t)n / 2), B(api_, dev_, (size_t)n / 2), SA(api_, dev_, (size_t)n / 32), SB(api_, dev_, (size_t)n / 32),
+        C(api_, dev_, (size_t)n * 2);
+    const bool ok = A && B && SA && SB && C && D % 256 == 0 &&
+                    api_.fill_bytes(dev_, (uint8_t *)A.ptr, n / 2, workload.seed, MI355_STREAM_GEMM_A, 0, 256) == MI355_OK &&
+                    api_.fill_bytes(dev_, (uint8_t *)B.ptr, n / 2, workload.seed, MI355_STREAM_GEMM_B, 0, 256) == MI355_OK &&
+                    api_.fill_bytes(dev_, (uint8_t *)SA.ptr, n / 32, workload.seed, MI355_STREAM_SCALE_A, 123, 9) == MI355_OK &&
+                    api_.fill_bytes(dev_, (uint8_t *)SB.ptr, n / 32, workload.seed, MI355_STREAM_SCALE_B, 123, 9) == MI355_OK;
+    float us = -1.0f;
+    if (ok)
+      us = runKernel([&] { return api_.gemm_mxfp4(dev_, (const uint8_t *)A.ptr, (const uint8_t *)B.ptr, (const uint8_t *)SA.ptr,
+                                                   (const uint8_t *)SB.ptr, (uint16_t *)C.ptr, D, D, D); },
+                     targetTimeUs, forceIters ? specifiedIters : 0);
+    if (!ok) test.skip("mxf4_e2m1", ResultStatus::Error, "Failed to allocate or fill GEMM buffers", mxNote);
+    else if (us <= 0.0f) test.skip("mxf4_e2m1", ResultStatus::Error, "kernel launch failed", mxNote);
+    else test.emit("mxf4_e2m1", (float)(2.0 * D * D * D * 1e6 / us / 1e12), {false, mxNote});
+  }
 }
 
 void Mi355Peak::runGemmInt() {

@@ -254,6 +254,21 @@ int mi355_gemm_i8(mi355_dev *dev, const int8_t *A, const int8_t *B, int32_t *C,
 int mi355_gemm_fp8_e5m2(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C,
                         uint32_t M, uint32_t N, uint32_t K, float scale_a, float scale_b);
 
+/*   "mxf4_e2m1" of runHipblasLt (src/rocm/hipblaslt_gemm.cpp:398-512: block-scaled FP4, one
+ *          UE8M0 scale per 32 elements along K, fp32 accumulate, bf16 output).  A[M][K/2] and
+ *          B[N][K/2] hold e2m1 codes two per byte (low nibble = even k), K contiguous;
+ *          scale_a[M][K/32], scale_b[N][K/32] hold E8M0 bytes (value 2^(byte-127)).
+ *          C[m][n] = sum_k A[m][k]*2^sa[m][k/32] * B[n][k]*2^sb[n][k/32].  K a multiple of 256.
+ *          Each call first rewrites the scales into the order the kernel loads them (two small
+ *          launches, part of the timed work); the copy lives in a scratch buffer of the same size
+ *          that the handle allocates on the first call and on growth, and frees in mi355_close. */
+int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
+                     const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K);
+/* Operands for it: dst[i] = lo + floor(span * (z >> 32) / 2^32), a uniform byte in [lo, lo+span)
+ * (span 256, lo 0: random code pairs; lo 123, span 9: scales 2^-4 .. 2^4). */
+int mi355_fill_bytes(mi355_dev *dev, uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream,
+                     uint32_t lo, uint32_t span);
+
 #ifdef __cplusplus
 }
 #endif

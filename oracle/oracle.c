@@ -571,6 +571,45 @@ int orc_gemm_tile(int fmt, const void *A, const void *B, uint32_t K, uint32_t ld
     return orc_gemm_tile2(fmt, fmt, A, B, K, lda, ldb, m0, n0, tm, tn, scale, C);
 }
 
+/* Block-scaled FP4 tile: A[M][K/2], B[N][K/2] hold e2m1 codes two per byte (low nibble = even k),
+ * SA[M][K/32], SB[N][K/32] E8M0 bytes; C[m][n] = sum_k a*2^(sa-127) * b*2^(sb-127), in double. */
+int orc_gemm_mx_tile(const uint8_t *A, const uint8_t *B, const uint8_t *SA, const uint8_t *SB, uint32_t K,
+                     uint32_t m0, uint32_t n0, uint32_t tm, uint32_t tn, double *C)
+{
+    if (K % 32) return -1;
+    const uint32_t kb = K / 2, ks = K / 32;
+    double *a = (double *)malloc((size_t)tm * K * sizeof(double));
+    double *b = (double *)malloc((size_t)tn * K * sizeof(double));
+    if (!a || !b) { free(a); free(b); return -3; }
+    for (uint32_t i = 0; i < tm; i++)
+        for (uint32_t k = 0; k < K; k++) {
+            const uint8_t byte = A[(size_t)(m0 + i) * kb + k / 2];
+            a[(size_t)i * K + k] = orc_decode(6, (k & 1) ? byte >> 4 : byte & 15) * orc_e8m0(SA[(size_t)(m0 + i) * ks + k / 32]);
+        }
+    for (uint32_t j = 0; j < tn; j++)
+        for (uint32_t k = 0; k < K; k++) {
+            const uint8_t byte = B[(size_t)(n0 + j) * kb + k / 2];
+            b[(size_t)j * K + k] = orc_decode(6, (k & 1) ? byte >> 4 : byte & 15) * orc_e8m0(SB[(size_t)(n0 + j) * ks + k / 32]);
+        }
+    #pragma omp parallel for schedule(static)
+    for (uint32_t i = 0; i < tm; i++)
+        for (uint32_t j = 0; j < tn; j++) {
+            double acc = 0.0;
+            const double *ar = a + (size_t)i * K, *br = b + (size_t)j * K;
+            for (uint32_t k = 0; k < K; k++) acc += ar[k] * br[k];
+            C[(size_t)i * tn + j] = acc;
+        }
+    free(a);
+    free(b);
+    return 0;
+}
+
+/* dst[i] = lo + below(word(seed, stream, first+i), span): uniform bytes, as the device fill. */
+void orc_fill_bytes(uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream, uint32_t lo, uint32_t span, uint64_t first)
+{
+    for (uint64_t i = 0; i < n; i++) dst[i] = (uint8_t)(lo + orc_below(seed, stream, first + i, span));
+}
+
 /* ------------------------------------------------------------------------- */
 /* Seeded operand builders (inputs of the matrix tests)                        */
 /* ------------------------------------------------------------------------- */

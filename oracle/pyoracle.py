@@ -138,6 +138,25 @@ def gemm_tile2(fmt_a, fmt_b, A, B, K, lda, ldb, m0, n0, tm, tn, scale=1.0):
 FMT_I8 = 7
 
 
+def gemm_mx_tile(A, B, SA, SB, K, m0, n0, tm, tn):
+    out = np.empty((tm, tn), dtype=np.float64)
+    L = lib()
+    L.orc_gemm_mx_tile.argtypes = [C.c_void_p] * 4 + [C.c_uint32] * 5 + [C.c_void_p]
+    L.orc_gemm_mx_tile.restype = C.c_int
+    rc = L.orc_gemm_mx_tile(A.ctypes.data, B.ctypes.data, SA.ctypes.data, SB.ctypes.data, K, m0, n0, tm, tn, out.ctypes.data)
+    assert rc == 0, rc
+    return out
+
+
+def fill_bytes(n, seed, stream, lo, span, first=0):
+    out = np.empty(n, dtype=np.uint8)
+    L = lib()
+    L.orc_fill_bytes.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint64]
+    L.orc_fill_bytes.restype = None
+    L.orc_fill_bytes(out.ctypes.data, n, seed, stream, lo, span, first)
+    return out
+
+
 def fill_fmt(fmt, n, seed, stream, dist, scale=1.0, first=0):
     out = np.empty(n, dtype=np.uint16 if fmt <= FMT_BF16 else np.uint8)
     L = lib()

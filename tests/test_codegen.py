@@ -27,16 +27,20 @@ def device_asm(tmp_path, source):
 
 
 def kernel_metadata(asm):
-    """{kernel name: {field: int}} from the amdhsa.kernels metadata block."""
-    meta, cur = {}, None
+    """{kernel name: {field: int}} from the amdhsa.kernels metadata block (one YAML list item per kernel)."""
+    meta, item = {}, None
+    fields = r"(vgpr_count|vgpr_spill_count|sgpr_spill_count|agpr_count|private_segment_fixed_size|group_segment_fixed_size)"
     for line in asm.splitlines():
-        m = re.match(r"\s+\.name:\s+(\S+)", line)
+        if re.match(r"  - \.\w+:", line):               # "  - .key: value" at list depth opens the next kernel's item
+            item = {}
+        if item is None:
+            continue
+        m = re.match(r"\s+(?:-\s+)?\." + fields + r":\s+(\d+)", line)
+        if m:
+            item[m.group(1)] = int(m.group(2))
+        m = re.match(r"\s+(?:-\s+)?\.name:\s+(\S+)", line)
         if m and "kernel" in m.group(1):
-            cur = meta.setdefault(m.group(1), {})
-        m = re.match(r"\s+\.(vgpr_count|vgpr_spill_count|sgpr_spill_count|agpr_count|"
-                     r"private_segment_fixed_size|group_segment_fixed_size):\s+(\d+)", line)
-        if m and cur is not None:
-            cur[m.group(1)] = int(m.group(2))
+            meta[m.group(1)] = item
     return meta
 
 
@@ -83,3 +87,27 @@ def test_peak_loops_do_not_spill(tmp_path, source):
     for name, m in meta.items():
         assert m.get("vgpr_spill_count", 0) == 0, (name, m)
         assert m.get("private_segment_fixed_size", 0) == 0, (name, m)
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_gemm_mxfp4_keeps_asynchronous_results_out_of_scratch(tmp_path):
+    """One wave per SIMD: 256 accumulation registers for the 64 tiles and the vector registers for fragments
+    and scales.  A few lane-index values may spill around the loop; nothing inside the loops may, because
+    the fragment and scale registers are written asynchronously by the loads."""
+    asm = device_asm(tmp_path, "gemm_mxfp4.hip")
+    meta = kernel_metadata(asm)
+    name = next(k for k in meta if "gemm_mxfp4_kernel" in k)
+    m = meta[name]
+    assert m["agpr_count"] == 256 and m["vgpr_count"] <= 512, m
+    body = kernel_body(asm, name)
+    assert body.count("v_mfma_scale_f32_16x16x128_f8f6f4") == 256      # two instances of the 128-instruction step
+    # every loop body (from a loop header label to its backward branch) is free of scratch traffic
+    lines = body.split("\n")
+    labels = {l.split(":")[0]: n for n, l in enumerate(lines) if l.startswith(".LBB")}
+    loops = 0
+    for n, l in enumerate(lines):
+        mt = re.search(r"s_cbranch_\w+ (\.LBB\w+)", l)
+        if mt and mt.group(1) in labels and labels[mt.group(1)] < n:
+            loops += 1
+            assert not any("scratch_" in x for x in lines[labels[mt.group(1)]:n]), mt.group(1)
+    assert loops >= 2

@@ -164,3 +164,55 @@ def test_gemm_other_types_8192_sampled_tiles(dev, kind):
     rng = np.random.default_rng(3)
     tiles = [(int(m) * 128, int(n) * 128) for m, n in zip(rng.integers(0, 64, 12), rng.integers(0, 64, 12))]
     _check_kind(dev, kind, 8192, 8192, 8192, tiles)
+
+
+# --- block-scaled FP4 ----------------------------------------------------------------------------------
+def _check_mx(dev, M, N, K, tiles, tile=128):
+    dA, dB = dev.alloc(M * K // 2), dev.alloc(N * K // 2)
+    dSA, dSB = dev.alloc(M * K // 32), dev.alloc(N * K // 32)
+    dC = dev.alloc(M * N * 2)
+    dev.memset(dC, 0xff)
+    dev.fill_bytes(dA, M * K // 2, SEED, wl.STREAM_GEMM_A, 0, 256)        # two uniformly random e2m1 codes per byte
+    dev.fill_bytes(dB, N * K // 2, SEED, wl.STREAM_GEMM_B, 0, 256)
+    dev.fill_bytes(dSA, M * K // 32, SEED, wl.STREAM_SCALE_A, 123, 9)       # 2^-4 .. 2^4
+    dev.fill_bytes(dSB, N * K // 32, SEED, wl.STREAM_SCALE_B, 123, 9)
+    dev.gemm_mxfp4(dA, dB, dSA, dSB, dC, M, N, K)
+    for (m0, n0) in tiles:
+        a = dA.download(np.uint8, tile * K // 2, offset_bytes=m0 * K // 2)
+        b = dB.download(np.uint8, tile * K // 2, offset_bytes=n0 * K // 2)
+        sa = dSA.download(np.uint8, tile * K // 32, offset_bytes=m0 * K // 32)
+        sb = dSB.download(np.uint8, tile * K // 32, offset_bytes=n0 * K // 32)
+        ref = orc.gemm_mx_tile(a, b, sa, sb, K, 0, 0, tile, tile)
+        got = np.empty((tile, tile), dtype=np.float64)
+        for i in range(tile):
+            row = dC.download(np.uint16, tile, offset_bytes=((m0 + i) * N + n0) * 2)
+            got[i] = (row.astype(np.uint32) << 16).view(np.float32)
+        rms = float(np.sqrt((ref ** 2).mean()))
+        err = np.abs(got - ref)
+        assert np.all(np.isfinite(got)), (m0, n0)
+        assert np.all(err <= 1e-2 * np.abs(ref) + 1e-2 * rms), (m0, n0, float(err.max()), rms)
+    for b in (dA, dB, dSA, dSB, dC):
+        b.free()
+
+
+def test_fill_bytes_bit_exact(dev):
+    n = (1 << 16) + 3
+    buf = dev.alloc(n)
+    for lo, span in ((0, 256), (123, 9), (7, 1)):
+        dev.fill_bytes(buf, n, SEED, wl.STREAM_SCALE_A, lo, span)
+        got = buf.download(np.uint8, n)
+        assert np.array_equal(got, orc.fill_bytes(n, SEED, wl.STREAM_SCALE_A, lo, span))
+        assert got.min() >= lo and got.max() < lo + span
+    buf.free()
+
+
+@pytest.mark.parametrize("steps", [1, 2, 3, 4, 5, 9])
+def test_gemm_mxfp4_short_walks(dev, steps):
+    _check_mx(dev, 256, 256, steps * 256, [(0, 0), (0, 128), (128, 0), (128, 128)])
+
+
+def test_gemm_mxfp4_grids_and_full_size(dev):
+    _check_mx(dev, 768, 512, 1024, [(m, n) for m in range(0, 768, 128) for n in range(0, 512, 128)])
+    rng = np.random.default_rng(4)
+    tiles = [(int(m) * 128, int(n) * 128) for m, n in zip(rng.integers(0, 64, 8), rng.integers(0, 64, 8))]
+    _check_mx(dev, 8192, 8192, 8192, tiles)

@@ -84,7 +84,7 @@ def test_full_run_row_contract_and_xml(tmp_path):
         assert cat == CATEGORY_OF_UNIT[unit]
     # measured values carry exactly 4 decimals
     vals = [m[2] for _, _, _, ms in rows for m in ms if m[1] is None]
-    assert len(vals) == 46 and all(re.fullmatch(r"-?\d+\.\d{4}", v) for v in vals)
+    assert len(vals) == 47 and all(re.fullmatch(r"-?\d+\.\d{4}", v) for v in vals)
     # rows that are deliberate skips keep the reference's status
     status = {(t, m[0]): m[1] for _, t, _, ms in rows for m in ms}
     assert status[("kernel_launch_latency", "dispatch")] == "unsupported"
@@ -143,7 +143,7 @@ def test_device_selection(tmp_path):
 
 @pytest.mark.parametrize("entry,tag,metric", [("mfma_dense", "mfma_bf16", "mfma_bf16"), ("gemm_bf16", "rocblas-fp", "bf16"),
                                               ("gemm_f16", "rocblas-fp", "fp16"), ("fill_i8", "rocblas-int", "int8"),
-                                              ("gemm_fp8_e5m2", "hipblaslt-fp8", "fp8_e5m2"),
+                                              ("gemm_fp8_e5m2", "hipblaslt-fp8", "fp8_e5m2"), ("gemm_mxfp4", "hipblaslt-fp8", "mxf4_e2m1"),
                                               ("local_bandwidth", "local_memory_bandwidth", "float2"),
                                               ("host_alloc", "transfer_bandwidth", "h2d_pinned"),
                                               ("copy_async", "transfer_bandwidth", "d2h_pinned"),
