@@ -48,7 +48,7 @@ def timed(dev, launch, min_us=300e3, warm_us=300e3, max_iters=10000):
 
 def bench_rows(dev, quick, only):
     from clpeak_amd import capi
-    from oracle import workloads as wl
+    from clpeak_amd import workloads as wl
     rows = []
     budget = dict(min_us=100e3, warm_us=100e3) if quick else {}
 
@@ -66,7 +66,9 @@ def bench_rows(dev, quick, only):
         us = dev.launch_roundtrip(2, 10000)
         add("kernel_launch_latency", "roundtrip", us, "us", us)
     if "mfma" in only or "smfmac" in only:
-        _matrix_rows(dev, wl, add, budget, only)
+        _matrix_rows(dev, wl, add, budget, only, zero=False)
+    if "matrix_zero" in only:
+        _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=True)
     if "gemm" in only:
         _gemm_rows(dev, capi, wl, add, budget, constant=False)
     if "gemm_const" in only:
@@ -124,21 +126,27 @@ def _mad_rows(dev, capi, add, budget):
     out.free()
 
 
-def _matrix_rows(dev, wl, add, budget, only):
+def _matrix_rows(dev, wl, add, budget, only, zero):
     # --- dense MFMA / SMFMAC: 2048 waves x 4 chains x 4096 iterations ------------------------
+    # zero: the same launches on all-zero operands.  Nothing toggles in the multipliers, the part holds
+    # its boost clock, and the row shows the issue rate of the loop itself (the seeded rows show what the
+    # part sustains under the power that random operands draw).
     waves, iters = 2048, 4096
+    tail = " zero operands" if zero else ""
     clk = dev.alloc(16)
     peaks = {0: "f16", 1: "bf16", 2: "f16", 3: "bf16", 4: "int8", 5: "fp8", 6: "fp8", 7: "fp6", 8: "fp6", 9: "fp4"}
     for kind in sorted(wl.DENSE) if "mfma" in only else []:
         s = wl.DENSE[kind]
         A, B, sA, sB = wl.dense_inputs(kind, waves, SEED)
+        if zero:
+            A, B = np.zeros_like(A), np.zeros_like(B)
         bufs = [dev.from_host(A), dev.from_host(B), dev.from_host(sA) if sA is not None else None,
                 dev.from_host(sB) if sB is not None else None]
         o = dev.alloc(waves * 4 * s["M"] * s["N"] * 4)
         us, _ = timed(dev, lambda: dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], o, waves, iters, clk), **budget)
         c = clk.download(np.uint64, 2)
-        unit = "tops" if s["fmt"] is None else "tflops"
-        add(s["name"], s["name"], wl.dense_flops(kind, waves, iters) / us / 1e6, unit, us, PEAK[peaks[kind]],
+        unit = "tops" if s["fmt"] == wl.I8 else "tflops"
+        add(s["name"], s["name"] + tail, wl.dense_flops(kind, waves, iters) / us / 1e6, unit, us, PEAK[peaks[kind]],
             shape=s["shape"], sclk_mhz=round(float(c[0]) / max(float(c[1]), 1.0) * 100.0, 0))
         for b in bufs + [o]:
             if b is not None:
@@ -147,12 +155,14 @@ def _matrix_rows(dev, wl, add, budget, only):
     for kind in sorted(wl.SPARSE) if "smfmac" in only else []:
         s = wl.SPARSE[kind]
         Ac, meta, B = wl.sparse_inputs(kind, waves, SEED)
+        if zero:
+            Ac, B = np.zeros_like(Ac), np.zeros_like(B)
         bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
         o = dev.alloc(waves * 4 * 256 * 4)
         us, _ = timed(dev, lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk), **budget)
         c = clk.download(np.uint64, 2)
-        unit = "tops" if s["fmt"] is None else "tflops"
-        add(s["name"], s["name"], wl.sparse_flops(kind, waves, iters) / us / 1e6, unit, us, 2 * PEAK[speaks[kind]],
+        unit = "tops" if s["fmt"] == wl.I8 else "tflops"
+        add(s["name"], s["name"] + tail, wl.sparse_flops(kind, waves, iters) / us / 1e6, unit, us, 2 * PEAK[speaks[kind]],
             shape=s["shape"], sclk_mhz=round(float(c[0]) / max(float(c[1]), 1.0) * 100.0, 0))
         for b in bufs + [o]:
             b.free()
@@ -314,15 +324,15 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel over 1 GiB (20 launches): under rocprofv3 --pmc this "
                          "gives what FETCH_SIZE / WRITE_SIZE read for a transfer of known size")
-    ap.add_argument("--only", default="mad,latency,mfma,smfmac,gemm,gemm_const,lds,transfer",
-                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,gemm,gemm_const,lds,transfer")
+    ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_zero,gemm,gemm_const,lds,transfer",
+                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_zero,gemm,gemm_const,lds,transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; the hot path has no multi-GPU step "
                  "(every kernel is independent per device), run with --gpus 1")
 
     from clpeak_amd import capi
-    from oracle import workloads as wl
+    from clpeak_amd import workloads as wl
     dev = capi.Device(0)
 
     if args.calibrate_copy:

@@ -42,10 +42,18 @@
 // transposed 16x16 tile: a lane then holds 4 consecutive N elements of one C row and
 // stores them as one 8-byte word.
 //
-// Workgroup -> tile mapping.  Workgroups are dealt round-robin to the 8 XCDs, each
-// with its own L2.  The mapping hands every XCD a contiguous band of tile rows, so
-// the A rows a band needs are fetched into one L2 only, and walks each band in
-// column-major order of 4-row groups so that B slabs are reused while still hot.
+// Workgroups are persistent: one per CU (the ring takes the whole LDS), each walking the
+// tiles id, id + grid, id + 2*grid, ...  The ring does not stop at a tile boundary: slabs are
+// numbered through all tiles of the workgroup, so while the last steps of one tile compute, the
+// first slabs of the next tile are already being fetched, and the only time the matrix pipe is
+// not fed between two tiles is the time it takes to convert and store the accumulators.  After
+// its last tile a workgroup keeps fetching (the slabs of its first tile again, which nobody
+// reads) so that every step is the same code; those loads are waited for before the wave ends.
+//
+// Tile id -> tile mapping.  Workgroups are dealt round-robin to the 8 XCDs, each
+// with its own L2, and id + k*grid stays on the XCD of id.  The mapping hands every XCD a
+// contiguous band of tile rows, so the A rows a band needs are fetched into one L2 only, and
+// walks each band in column-major order of 4-row groups so that B slabs are reused while hot.
 #include "internal.h"
 #include "mfma_common.h"
 #include "numeric_formats.h"
@@ -101,9 +109,9 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
 
 // Operand types of the kernel that walks a slab as two K halves (16 bytes per lane and half):
 // bf16 and f16 (K=32 per instruction, fp32 accumulate) and int8 (K=64, int32 accumulate).
-enum { kBf16 = 0, kF16 = 1, kI8 = 2 };
+enum { kBf16 = 0, kF16 = 1, kI8 = 2, kScaledBf16 = 3 };   // kScaledBf16: output type of the fp8 kernels only
 
-// State of one wave's walk along K that the step function advances.
+// State of one wave's walk along K that the step function reads.
 struct GemmWalk {
   uint32_t a_cur, b_cur, a_nxt, b_nxt;   // LDS byte addresses of this lane's first A / B fragment, both buffers
   uint32_t dst_a, dst_b;                 // LDS destinations of the wave's 32 A rows / 32 B rows to fetch
@@ -112,17 +120,163 @@ struct GemmWalk {
   uint32_t row8;                         // bytes between rows r and r+8 (load q reads from base + q*row8)
 };
 
+// The tiles one workgroup owns: ids first, first + stride, ... (`mine` of them) out of tiles_m x tiles_n.
+struct TileGrid {
+  uint32_t tiles_m, tiles_n, total, first, stride, mine;
+};
+
+__device__ __forceinline__ void tile_at(const TileGrid &g, uint32_t round, uint32_t &tm, uint32_t &tn) {
+  const uint32_t id = g.first + round * g.stride;
+  uint32_t lin = id;
+  if (g.total % 8u == 0u) lin = (id % 8u) * (g.total / 8u) + id / 8u;   // tiles of one XCD are consecutive
+  // consecutive tiles walk down a group of 4 tile rows, then move one column right
+  const uint32_t per_group = 4u * g.tiles_n;
+  const uint32_t group = lin / per_group, in_group = lin - group * per_group;
+  const uint32_t rows_here = g.tiles_m - group * 4u;
+  if (rows_here >= 4u) {
+    tm = group * 4u + (in_group & 3u);
+    tn = in_group >> 2;
+  } else {
+    tm = group * 4u + in_group % rows_here;
+    tn = in_group / rows_here;
+  }
+}
+
+__device__ __forceinline__ TileGrid tiles_of_workgroup(uint32_t tiles_m, uint32_t tiles_n) {
+  TileGrid g;
+  g.tiles_m = tiles_m; g.tiles_n = tiles_n; g.total = tiles_m * tiles_n;
+  g.first = blockIdx.x; g.stride = gridDim.x;
+  g.mine = (g.total - g.first + g.stride - 1u) / g.stride;   // the host launches at most `total` workgroups
+  return g;
+}
+
+// The LDS ring of one wave and the two fetch streams (A rows three slabs ahead of the slab being
+// multiplied, B rows two ahead) through all tiles of the workgroup.  Slabs are numbered through the
+// tiles: slab g has its A rows in slot 2g mod 5 and its B rows in slot (2g+1) mod 5.
+struct GemmRing {
+  GemmWalk w;
+  TileGrid grid;
+  uint64_t a_origin, b_origin;   // A / B plus this wave's 32 rows within a tile (uniform)
+  uint32_t k_bytes, steps;
+  uint32_t lane_a, lane_b;       // this lane's first A / B fragment within a slot
+  uint32_t dst_wave;             // this wave's 4 KiB within a slot
+  uint32_t k0;                   // slot of the current slab's A rows
+  uint32_t a_round, a_left, b_round, b_left;   // tile (as a round of the workgroup) and steps left in it, per stream
+
+  __device__ __forceinline__ static uint32_t slot_off(uint32_t k) { return (k >= 5u ? k - 5u : k) * (uint32_t)kSlabBytes; }
+
+  __device__ __forceinline__ uint64_t a_rows(uint32_t round) const {
+    uint32_t tm, tn;
+    tile_at(grid, round, tm, tn);
+    return a_origin + (uint64_t)tm * kTile * k_bytes;
+  }
+  __device__ __forceinline__ uint64_t b_rows(uint32_t round) const {
+    uint32_t tm, tn;
+    tile_at(grid, round, tm, tn);
+    return b_origin + (uint64_t)tn * kTile * k_bytes;
+  }
+  __device__ __forceinline__ void place() {
+    w.a_cur = lane_a + slot_off(k0);      w.b_cur = lane_b + slot_off(k0 + 1u);
+    w.a_nxt = lane_a + slot_off(k0 + 2u); w.b_nxt = lane_b + slot_off(k0 + 3u);
+    w.dst_b = dst_wave + slot_off(k0);        // B rows two slabs ahead take over the current A slot
+    w.dst_a = dst_wave + slot_off(k0 + 1u);   // A rows three slabs ahead take over the current B slot
+  }
+  // Move a stream to its next slab: 128 bytes along K, or on to the first slab of the workgroup's next
+  // tile (after the last tile: of its first tile again, a fetch nobody reads).
+  __device__ __forceinline__ void next_a() {
+    if (--a_left == 0u) {
+      a_round = a_round + 1u == grid.mine ? 0u : a_round + 1u;
+      w.ga = a_rows(a_round);
+      a_left = steps;
+    } else {
+      w.ga += kRowBytes;
+    }
+  }
+  __device__ __forceinline__ void next_b() {
+    if (--b_left == 0u) {
+      b_round = b_round + 1u == grid.mine ? 0u : b_round + 1u;
+      w.gb = b_rows(b_round);
+      b_left = steps;
+    } else {
+      w.gb += kRowBytes;
+    }
+  }
+  __device__ __forceinline__ void fetch(uint64_t rows, uint32_t slot) const {
+#pragma unroll
+    for (uint32_t q = 0; q < 4; q++) MI355_LOAD_LDS(w.voff, rows + (uint64_t)q * w.row8, dst_wave + slot_off(slot) + q * 1024u);
+  }
+  // Fill the ring (A and B rows of slabs 0 and 1, A rows of slab 2), wait for it, and stand on slab 0.
+  __device__ __forceinline__ void start(const uint8_t *A, const uint8_t *B, uint32_t k_bytes_, uint32_t lds_base,
+                                        uint32_t wave, uint32_t lane, const TileGrid &g) {
+    const uint32_t wm = wave / 4, wn = wave % 4;
+    grid = g;
+    k_bytes = k_bytes_;
+    steps = k_bytes / kRowBytes;
+    a_origin = (uint64_t)(uintptr_t)(A + (size_t)wave * 32u * k_bytes);
+    b_origin = (uint64_t)(uintptr_t)(B + (size_t)wave * 32u * k_bytes);
+    // global -> LDS: instruction q of a wave fills rows [(wave*4+q)*8, +8) of a slab; lane i is position
+    // i%8 of row i/8, which holds logical chunk (i%8) ^ (row & 7) = (i%8) ^ (i/8).
+    const uint32_t lchunk = (lane % 8u) ^ (lane / 8u);
+    w.voff = (lane / 8u) * k_bytes + lchunk * 16u;
+    w.row8 = 8u * k_bytes;
+    dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 4096u);
+    // LDS -> fragments: row (lane%16) of the wave's sub-tile, logical chunk lane/16 (+4 for the second K
+    // half, i.e. the address with bit 6 flipped), swizzled with row&7 = lane&7.
+    const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
+    lane_a = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
+    lane_b = lds_base + (wn * 64u + lane % 16u) * kRowBytes + swz0;
+
+    a_round = b_round = 0;
+    a_left = b_left = steps;
+    w.ga = a_rows(0);
+    w.gb = b_rows(0);
+    fetch(w.ga, 0); next_a();
+    fetch(w.gb, 1); next_b();
+    fetch(w.ga, 2); next_a();
+    fetch(w.gb, 3); next_b();
+    fetch(w.ga, 4); next_a();
+    asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+    k0 = 0;
+    place();
+  }
+  __device__ __forceinline__ void advance() {
+    k0 = k0 + 2u >= 5u ? k0 + 2u - 5u : k0 + 2u;
+    place();
+    next_a();
+    next_b();
+  }
+};
+
+// The barrier of a step: every wave holds all fragments of the step's slab (its two slots are free)
+// and, loads returning in order, with its 4 youngest loads (the A rows three slabs ahead) still
+// allowed in flight, its share of the next slab has landed.  In the first step of a tile that
+// wait was done at the end of the tile before, and the stores issued since must not count.
+#define MI355_STEP_BARRIER(first, lds_wait)                                                        \
+  asm volatile(lds_wait "s_cmp_lg_u32 %0, 0\n s_cbranch_scc1 1f\n s_waitcnt vmcnt(4)\n1:\n s_barrier"  \
+               :: "s"(first) : "memory", "scc")
+
+// What every wave does once its last tile is stored: the fetches that ran ahead of it still write LDS.
+#define MI355_DRAIN_RING() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory")
+
+// Between the last matrix instruction of a tile and the first read of its accumulators: the wait
+// states the compiler cannot know about (the operands tie the youngest results to this point), then
+// the wave's loads but the 4 youngest, before any store joins the queue of outstanding memory
+// operations: the first barrier of the next tile then needs no wait of its own.
+#define MI355_END_OF_TILE(acc)                                                                     \
+  asm volatile("s_nop 15\n s_nop 15\n s_waitcnt vmcnt(4)"                                          \
+               : "+v"(acc[7][0]), "+v"(acc[7][1]), "+v"(acc[7][2]), "+v"(acc[7][3]), "+v"(acc[6][3]) :: "memory")
+
 // One step of K: 64 MFMAs per wave, 32 on fragment set F0 (first K half of the slab) then 32 on
 // F1.  The order written here is the order issued; never more than one memory instruction between
 // two MFMAs, because a ds_read_b128 (about 11 cycles of issue) slips into the 16-cycle shadow of
 // the MFMA before it, while two in a row would stall the matrix pipe.
-// MAIN: a step of the steady state; otherwise `reads` / `loads` are run-time (wave-uniform)
-// switches for the last steps, which have nothing left to prefetch.
-template <bool MAIN, int KIND>
+// `first` (wave-uniform): the first step of a tile, whose barrier needs no wait for loads (the end of
+// the tile before did it, ahead of the stores that are now in the queue).  A step always prefetches:
+// the last step of a tile reads the first fragments of the next tile, which the ring already holds.
+template <int KIND>
 __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8], bf16x8v (&fb0)[4],
-                                          bf16x8v (&fa1)[8], bf16x8v (&fb1)[4], const GemmWalk &w,
-                                          bool reads, bool loads_a, bool loads_b) {
-  const bool READS = MAIN || reads, LOADS_A = MAIN || loads_a, LOADS_B = MAIN || loads_b;
+                                          bf16x8v (&fa1)[8], bf16x8v (&fb1)[4], const GemmWalk &w, uint32_t first) {
+  constexpr bool READS = true;
   const uint32_t a1 = w.a_cur ^ 64u, b1 = w.b_cur ^ 64u;   // second K half of this step
 #define MM(F, i, j)                                                                                \
   do {                                                                                             \
@@ -130,8 +284,8 @@ __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8]
     else if (KIND == kF16) MI355_MFMA_F16(acc[i][j], F##b##_[j], F##a##_[i]);                      \
     else MI355_MFMA_I8(acc[i][j], F##b##_[j], F##a##_[i]);                                         \
   } while (0)
-#define LDA(q) if (LOADS_A) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
-#define LDB(q) if (LOADS_B) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
+#define LDA(q) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
+#define LDB(q) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
   bf16x8v(&x0a_)[8] = fa0; bf16x8v(&x0b_)[4] = fb0; bf16x8v(&x1a_)[8] = fa1; bf16x8v(&x1b_)[4] = fb1;
   // ---- MFMAs 0..12 (on F0); the 12 reads of F1 in the first 6 gaps ------------------------------
   MM(x0, 0, 0); MI355_DS_READ(fb1[0], b1, 0); MI355_DS_READ(fb1[1], b1, 2048);
@@ -148,8 +302,7 @@ __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8]
   // order, so with the 4 A loads of the last step (for the slab three steps ahead) still allowed in
   // flight, this wave's B rows of the next slab and its A rows of the next slab (older still) have
   // landed.
-  if (MAIN) asm volatile("s_waitcnt vmcnt(4)\n s_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+  MI355_STEP_BARRIER(first, "");
   // ---- MFMAs 13..63: B rows of the slab two steps ahead into the freed A slot, then A rows of the slab
   //      three steps ahead into the freed B slot, one load every sixth MFMA so that the fill path sees a
   //      steady stream; from MFMA 40 on (F0 is dead since MFMA 31) the next step's F0 reads ------------
@@ -210,15 +363,51 @@ __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8]
 #undef MM
 }
 
-__device__ inline void tile_of_block(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn) {
-  const uint32_t bid = blockIdx.x, total = tiles_m * tiles_n;
-  uint32_t lin = bid;
-  if (total % 8u == 0u) lin = (bid % 8u) * (total / 8u) + bid / 8u;   // tiles of one XCD are consecutive
-  // consecutive tiles walk down a group of 4 tile rows, then move one column right
-  const uint32_t group = lin / (4u * tiles_n), in_group = lin % (4u * tiles_n);
-  const uint32_t rows_here = (tiles_m - group * 4u) < 4u ? (tiles_m - group * 4u) : 4u;
-  tm = group * 4u + in_group % rows_here;
-  tn = in_group / rows_here;
+// Store a wave's 128x64 accumulators.  A lane holds 4 consecutive N elements of one row per 16x16 tile
+// (8 bytes of bf16 / f16, 16 bytes of int32), lane group g = lane/16 the 4 elements 4g..4g+3.  Stored as
+// they are, the four groups of a 16-bit row would write 32 contiguous bytes per instruction, a quarter of a
+// cache line; with every workgroup of the part storing its tile at the same moment that pattern reaches
+// 4.7 TB/s where 64-byte pieces reach 7.0 TB/s.  So two neighbouring tiles (j, j+1) first trade halves:
+// v_permlane16_swap exchanges the odd lane groups of tile j with the even groups of tile j+1, after which
+// groups 0,2 hold columns 0..7 and 8..15 of tile j and groups 1,3 those of tile j+1, 16 bytes per lane,
+// 64 contiguous bytes per row and instruction.
+template <int KIND>
+__device__ __forceinline__ void store_tile(const f32x4v (&acc)[8][4], void *__restrict__ Cout, uint32_t N, uint32_t row0,
+                                           uint32_t col0, uint32_t lane, float scale) {
+  if (KIND == kI8) {
+    const uint32_t col = col0 + 4u * (lane / 16u);
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        i32x4v bits;
+        __builtin_memcpy(&bits, &acc[i][j], sizeof(bits));
+        *reinterpret_cast<i32x4v *>(static_cast<int32_t *>(Cout) + (size_t)(row0 + i * 16u) * N + col + j * 16u) = bits;
+      }
+    return;
+  }
+  const uint32_t g = lane / 16u;
+  const uint32_t col = col0 + 16u * (g & 1u) + 8u * (g >> 1);   // of the pair (0,1); the pair (2,3) is 32 further
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int jp = 0; jp < 4; jp += 2) {
+      uint32_t p[2][2];   // [tile of the pair][elements 0,1 | 2,3]
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          float lo = acc[i][jp + t][2 * h], hi = acc[i][jp + t][2 * h + 1];
+          if (KIND == kScaledBf16) { lo *= scale; hi *= scale; }
+          p[t][h] = KIND == kF16 ? mi355_pack_f16x2(lo, hi) : mi355_pack_bf16x2(lo, hi);
+        }
+      // q[0]: this group's elements 0..1 (even groups: of tile jp, odd groups: of tile jp+1), q[1]: the next
+      // group's elements 0..1 of the same tile, i.e. elements 4..5 of the 8 contiguous ones
+      const auto q01 = __builtin_amdgcn_permlane16_swap(p[0][0], p[1][0], false, false);
+      const auto q23 = __builtin_amdgcn_permlane16_swap(p[0][1], p[1][1], false, false);
+      const uint4 packed = make_uint4(q01[0], q23[0], q01[1], q23[1]);
+      *reinterpret_cast<uint4 *>(static_cast<uint16_t *>(Cout) + (size_t)(row0 + i * 16u) * N + col + jp * 16u) = packed;
+    }
 }
 
 template <int KIND>
@@ -229,32 +418,11 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
   const uint32_t tid = threadIdx.x, lane = tid % 64;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);   // wave-uniform, and known to be
   const uint32_t wm = wave / 4, wn = wave % 4;
-  uint32_t tm, tn;
-  tile_of_block(tiles_m, tiles_n, tm, tn);
+  const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
 
-  // --- global -> LDS: this lane's source pointers and this wave's destinations -------------
-  // instruction q of a wave fills rows [(wave*4+q)*8, +8) of a slab; lane i is position i%8 of
-  // row i/8, which holds logical chunk (i%8) ^ (row & 7) = (i%8) ^ (i/8).
-  const uint32_t lrow = wave * 32u + lane / 8u, lchunk = (lane % 8u) ^ (lane / 8u);
-  const uint8_t *ga = A + ((size_t)tm * kTile + lrow) * k_bytes + lchunk * 16u;
-  const uint8_t *gb = B + ((size_t)tn * kTile + lrow) * k_bytes + lchunk * 16u;
-  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-  const uint32_t dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 4096u);
-  // LDS is a ring of five 32 KiB slots; the A rows of slab t live in slot 2t mod 5, its B rows in slot
-  // (2t+1) mod 5.  Two and a half slabs are resident or in flight at any time.
-  auto slot_off = [](uint32_t k) { return (k >= 5u ? k - 5u : k) * (uint32_t)kSlabBytes; };
-  auto fetch_rows = [&](const uint8_t *g, uint32_t step, uint32_t slot) {
-    const size_t kb = (size_t)step * kRowBytes;
-#pragma unroll
-    for (uint32_t q = 0; q < 4; q++) load_to_lds(g + kb + (size_t)q * 8u * k_bytes, dst_wave + slot * kSlabBytes + q * 1024u);
-  };
-
-  // --- LDS -> fragments: byte addresses of this lane's first A / B fragment within a slot ----------
-  // row (lane%16) of the wave's sub-tile, logical chunk ks*4 + lane/16, swizzled with row&7 = lane&7;
-  // the second K half differs by bit 2 of the chunk index, i.e. by 64 bytes.
-  const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
-  const uint32_t lane_a = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
-  const uint32_t lane_b = lds_base + (wn * 64u + lane % 16u) * kRowBytes + swz0;
+  GemmRing ring;
+  ring.start(A, B, k_bytes, (uint32_t)(uintptr_t)lds, wave, lane, grid);
+  const uint32_t steps = ring.steps;
 
   f32x4v acc[8][4];
 #pragma unroll
@@ -262,62 +430,30 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
   bf16x8v fa0[8], fb0[4], fa1[8], fb1[4];
-
-  const uint32_t steps = k_bytes / kRowBytes;
-  fetch_rows(ga, 0, 0);
-  fetch_rows(gb, 0, 1);
-  if (steps > 1) { fetch_rows(ga, 1, 2); fetch_rows(gb, 1, 3); }
-  if (steps > 2) fetch_rows(ga, 2, 4);
-  asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-
-  // The loads inside the loop take the scalar-base form (uniform 64-bit base + this lane's 32-bit
-  // offset), which costs no vector ALU work: load q of the wave covers rows 8q..8q+7 of its 32.
-  GemmWalk w;
-  uint32_t k0 = 0;   // slot of the current slab's A rows
-  auto place = [&]() {
-    w.a_cur = lane_a + slot_off(k0);     w.b_cur = lane_b + slot_off(k0 + 1u);
-    w.a_nxt = lane_a + slot_off(k0 + 2u); w.b_nxt = lane_b + slot_off(k0 + 3u);
-    w.dst_b = dst_wave + slot_off(k0);   // B rows two slabs ahead take over the current A slot
-    w.dst_a = dst_wave + slot_off(k0 + 1u);   // A rows three slabs ahead take over the current B slot
-  };
-  place();
-  MI355_READ_FRAGS(fa0, fb0, w.a_cur, w.b_cur);
+  MI355_READ_FRAGS(fa0, fb0, ring.w.a_cur, ring.w.b_cur);
   MI355_WAIT_FRAGS(fa0, fb0);
-  w.voff = (lane / 8u) * k_bytes + lchunk * 16u;
-  w.row8 = 8u * k_bytes;
-  w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kTile + wave * 32u) * k_bytes + 3 * (size_t)kRowBytes);
-  w.gb = (uint64_t)(uintptr_t)(B + ((size_t)tn * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
-  auto advance = [&]() {
-    k0 = k0 + 2u >= 5u ? k0 + 2u - 5u : k0 + 2u;
-    place();
-    w.ga += kRowBytes;
-    w.gb += kRowBytes;
-  };
-  uint32_t s = 0;
-  for (; s + 3 < steps; s++) { gemm_step<true, KIND>(acc, fa0, fb0, fa1, fb1, w, true, true, true); advance(); }
-  for (; s < steps; s++) { gemm_step<false, KIND>(acc, fa0, fb0, fa1, fb1, w, s + 1 < steps, false, s + 2 < steps); advance(); }
-  // wait states the compiler cannot know about, before the accumulators are read
-  asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
-  // --- epilogue: 4 consecutive N elements per lane; bf16 / f16 rounded from fp32, int32 as it is ----
-  const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 64u + 4u * (lane / 16u);
+  // one loop over the steps of all tiles of the workgroup
+  uint32_t round = 0, left = steps, first = 1;
+  for (uint32_t g = grid.mine * steps; g > 0; g--) {
+    gemm_step<KIND>(acc, fa0, fb0, fa1, fb1, ring.w, first);
+    ring.advance();
+    first = 0;
+    if (--left == 0) {
+      MI355_END_OF_TILE(acc);
+      uint32_t tm, tn;
+      tile_at(grid, round, tm, tn);
+      store_tile<KIND>(acc, Cout, N, tm * kTile + wm * 128u + lane % 16u, tn * kTile + wn * 64u, lane, 1.0f);
 #pragma unroll
-  for (int i = 0; i < 8; i++)
+      for (int i = 0; i < 8; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const size_t at = (size_t)(row0 + i * 16u) * N + col0 + j * 16u;
-      if (KIND == kI8) {
-        i32x4v bits;
-        __builtin_memcpy(&bits, &acc[i][j], sizeof(bits));
-        *reinterpret_cast<i32x4v *>(static_cast<int32_t *>(Cout) + at) = bits;
-      } else {
-        uint16_t h[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) h[r] = KIND == kBf16 ? mi355_f32_to_bf16(acc[i][j][r]) : mi355_f32_to_f16(acc[i][j][r]);
-        const uint2 packed = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
-        *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(Cout) + at) = packed;
-      }
+        for (int j = 0; j < 4; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
+      round++;
+      left = steps;
+      first = 1;
     }
+  }
+  MI355_DRAIN_RING();
 }
 
 // ---- fp8 e4m3 ------------------------------------------------------------------------------------
@@ -357,14 +493,13 @@ struct Fp8Frags {
   i32x4v a_lo[8], a_hi[8], b_lo[4], b_hi[4];
 };
 
-template <bool MAIN, bool E5M2>
-__device__ __forceinline__ void gemm_fp8_step(f32x4v (&acc)[8][4], Fp8Frags &f, const GemmWalk &w, bool reads,
-                                              bool loads_a, bool loads_b) {
-  const bool READS = MAIN || reads, LOADS_A = MAIN || loads_a, LOADS_B = MAIN || loads_b;
+template <bool E5M2>
+__device__ __forceinline__ void gemm_fp8_step(f32x4v (&acc)[8][4], Fp8Frags &f, const GemmWalk &w, uint32_t first) {
+  constexpr bool READS = true;
   const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u, an_hi = w.a_nxt ^ 64u, bn_hi = w.b_nxt ^ 64u;
 #define MM(i, j) MI355_MFMA_FP8(E5M2, acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i])
-#define LDA(q) if (LOADS_A) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
-#define LDB(q) if (LOADS_B) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
+#define LDA(q) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
+#define LDB(q) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
 #define RD_A_NEXT(i, off)                                                                          \
   if (READS) { MI355_DS_READ(f.a_lo[i], w.a_nxt, off); MI355_DS_READ(f.a_hi[i], an_hi, off); }
 #define RD_B_NEXT(j, off)                                                                          \
@@ -384,8 +519,7 @@ __device__ __forceinline__ void gemm_fp8_step(f32x4v (&acc)[8][4], Fp8Frags &f, 
   MM(4, 0); MM(4, 1);
   // every read of this step's slab has returned (its two slots are free); with the 4 A loads of the
   // last step still allowed in flight, this wave's share of the next slab has landed
-  if (MAIN) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n s_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier" ::: "memory");
+  MI355_STEP_BARRIER(first, "s_waitcnt lgkmcnt(0)\n");
   MM(5, 0); LDB(0);
   MM(5, 1);
   MM(6, 0); LDB(1);
@@ -423,27 +557,12 @@ gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, ui
   const uint32_t tid = threadIdx.x, lane = tid % 64;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const uint32_t wm = wave / 4, wn = wave % 4;
-  uint32_t tm, tn;
-  tile_of_block(tiles_m, tiles_n, tm, tn);
+  const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
 
-  // global -> LDS, exactly as in the bf16 kernel (rows are 128 bytes in both)
-  const uint32_t lrow = wave * 32u + lane / 8u, lchunk = (lane % 8u) ^ (lane / 8u);
-  const uint8_t *ga = A + ((size_t)tm * kTile + lrow) * k_bytes + lchunk * 16u;
-  const uint8_t *gb = B + ((size_t)tn * kTile + lrow) * k_bytes + lchunk * 16u;
-  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-  const uint32_t dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 4096u);
-  auto slot_off = [](uint32_t k) { return (k >= 5u ? k - 5u : k) * (uint32_t)kSlabBytes; };
-  auto fetch_rows = [&](const uint8_t *g, uint32_t step, uint32_t slot) {
-    const size_t kb = (size_t)step * kRowBytes;
-#pragma unroll
-    for (uint32_t q = 0; q < 4; q++) load_to_lds(g + kb + (size_t)q * 8u * k_bytes, dst_wave + slot * kSlabBytes + q * 1024u);
-  };
-
-  // LDS -> fragments: chunk lane/16 of row lane%16 (low half of the operand); the high half is
-  // chunk lane/16 + 4, i.e. the address with bit 6 flipped.
-  const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
-  const uint32_t lane_a = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
-  const uint32_t lane_b = lds_base + (wn * 64u + lane % 16u) * kRowBytes + swz0;
+  // ring, loads and fragment addresses exactly as in the bf16 kernel (rows are 128 bytes in both)
+  GemmRing ring;
+  ring.start(A, B, k_bytes, (uint32_t)(uintptr_t)lds, wave, lane, grid);
+  const uint32_t steps = ring.steps;
 
   f32x4v acc[8][4];
 #pragma unroll
@@ -451,25 +570,9 @@ gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, ui
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
   Fp8Frags f;
-
-  const uint32_t steps = k_bytes / kRowBytes;
-  fetch_rows(ga, 0, 0);
-  fetch_rows(gb, 0, 1);
-  if (steps > 1) { fetch_rows(ga, 1, 2); fetch_rows(gb, 1, 3); }
-  if (steps > 2) fetch_rows(ga, 2, 4);
-  asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-
-  GemmWalk w;
-  uint32_t k0 = 0;   // slot of the current slab's A rows (the ring of the bf16 kernel)
-  auto place = [&]() {
-    w.a_cur = lane_a + slot_off(k0);      w.b_cur = lane_b + slot_off(k0 + 1u);
-    w.a_nxt = lane_a + slot_off(k0 + 2u); w.b_nxt = lane_b + slot_off(k0 + 3u);
-    w.dst_b = dst_wave + slot_off(k0);
-    w.dst_a = dst_wave + slot_off(k0 + 1u);
-  };
-  place();
   // what a step expects in flight on entry: B fragments 0,1 then A fragments 0..6
   {
+    const GemmWalk &w = ring.w;
     const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u;
     MI355_DS_READ(f.b_lo[0], w.b_cur, 0); MI355_DS_READ(f.b_hi[0], b_hi, 0);
     MI355_DS_READ(f.b_lo[1], w.b_cur, 2048); MI355_DS_READ(f.b_hi[1], b_hi, 2048);
@@ -482,31 +585,27 @@ gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, ui
     MI355_DS_READ(f.a_lo[6], w.a_cur, 12288); MI355_DS_READ(f.a_hi[6], a_hi, 12288);
   }
 
-  w.voff = (lane / 8u) * k_bytes + lchunk * 16u;
-  w.row8 = 8u * k_bytes;
-  w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kTile + wave * 32u) * k_bytes + 3 * (size_t)kRowBytes);
-  w.gb = (uint64_t)(uintptr_t)(B + ((size_t)tn * kTile + wave * 32u) * k_bytes + 2 * (size_t)kRowBytes);
-  auto advance = [&]() {
-    k0 = k0 + 2u >= 5u ? k0 + 2u - 5u : k0 + 2u;
-    place();
-    w.ga += kRowBytes;
-    w.gb += kRowBytes;
-  };
-  uint32_t s = 0;
-  for (; s + 3 < steps; s++) { gemm_fp8_step<true, E5M2>(acc, f, w, true, true, true); advance(); }
-  for (; s < steps; s++) { gemm_fp8_step<false, E5M2>(acc, f, w, s + 1 < steps, false, s + 2 < steps); advance(); }
-  asm volatile("s_nop 15\n s_nop 15" ::: "memory");
-
-  const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 64u + 4u * (lane / 16u);
+  // one loop over the steps of all tiles of the workgroup
+  uint32_t round = 0, left = steps, first = 1;
+  for (uint32_t g = grid.mine * steps; g > 0; g--) {
+    gemm_fp8_step<E5M2>(acc, f, ring.w, first);
+    ring.advance();
+    first = 0;
+    if (--left == 0) {
+      MI355_END_OF_TILE(acc);
+      uint32_t tm, tn;
+      tile_at(grid, round, tm, tn);
+      store_tile<kScaledBf16>(acc, C, N, tm * kTile + wm * 128u + lane % 16u, tn * kTile + wn * 64u, lane, scale);
 #pragma unroll
-  for (int i = 0; i < 8; i++)
+      for (int i = 0; i < 8; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const uint16_t h0 = mi355_f32_to_bf16(acc[i][j][0] * scale), h1 = mi355_f32_to_bf16(acc[i][j][1] * scale);
-      const uint16_t h2 = mi355_f32_to_bf16(acc[i][j][2] * scale), h3 = mi355_f32_to_bf16(acc[i][j][3] * scale);
-      const uint2 packed = make_uint2((uint32_t)h0 | ((uint32_t)h1 << 16), (uint32_t)h2 | ((uint32_t)h3 << 16));
-      *reinterpret_cast<uint2 *>(C + (size_t)(row0 + i * 16u) * N + col0 + j * 16u) = packed;
+        for (int j = 0; j < 4; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
+      round++;
+      left = steps;
+      first = 1;
     }
+  }
+  MI355_DRAIN_RING();
 }
 
 int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, uint32_t M, uint32_t N, uint32_t K,
@@ -521,6 +620,12 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
 
 constexpr size_t kRingBytes = 5 * (size_t)kSlabBytes;   // five 32 KiB slots: all 160 KiB of a CU
 
+// One persistent workgroup per CU (a workgroup takes the whole LDS of one), never more than tiles.
+uint32_t workgroups(const mi355_dev *dev, uint32_t tiles) {
+  const uint32_t cus = dev->props.num_cus > 0 ? (uint32_t)dev->props.num_cus : 1u;
+  return tiles < cus ? tiles : cus;
+}
+
 template <int KIND>
 int launch_halves(mi355_dev *dev, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N,
                   uint32_t K, uint32_t elem) {
@@ -532,7 +637,7 @@ int launch_halves(mi355_dev *dev, const char *what, const void *A, const void *B
     attr_set = true;
   }
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_bf16_kernel<KIND><<<tiles_m * tiles_n, kThreads, kRingBytes, dev->stream>>>(
+  gemm_bf16_kernel<KIND><<<workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
       (const uint8_t *)A, (const uint8_t *)B, C, N, K * elem, tiles_m, tiles_n);
   MI355_LAUNCH_CHECK(dev, what);
   return MI355_OK;
@@ -549,7 +654,7 @@ int launch_fp8(mi355_dev *dev, const char *what, const uint8_t *A, const uint8_t
     attr_set = true;
   }
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_fp8_kernel<E5M2><<<tiles_m * tiles_n, kThreads, kRingBytes, dev->stream>>>(A, B, C, N, K, scale, tiles_m, tiles_n);
+  gemm_fp8_kernel<E5M2><<<workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(A, B, C, N, K, scale, tiles_m, tiles_n);
   MI355_LAUNCH_CHECK(dev, what);
   return MI355_OK;
 }

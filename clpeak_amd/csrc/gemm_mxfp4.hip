@@ -346,15 +346,20 @@ gemm_mxfp4_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, 
   for (; s < steps; s++) { mx_step<false>(acc, f, w, s + 1 < steps, false, s + 2 < steps); advance(); }
   asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
-  const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 128u + 4u * (lane / 16u);
+  // A lane holds 4 consecutive N elements per 16x16 tile.  Two neighbouring tiles (j, j+1) trade halves
+  // first (v_permlane16_swap: the odd lane groups of tile j against the even groups of tile j+1), so that a
+  // lane stores 8 consecutive bf16 and an instruction 64 contiguous bytes per row instead of 32.
+  const uint32_t g = lane / 16u;
+  const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 128u + 16u * (g & 1u) + 8u * (g >> 1);
 #pragma unroll
   for (int i = 0; i < 8; i++)
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const uint16_t h0 = mi355_f32_to_bf16(acc[i][j][0]), h1 = mi355_f32_to_bf16(acc[i][j][1]);
-      const uint16_t h2 = mi355_f32_to_bf16(acc[i][j][2]), h3 = mi355_f32_to_bf16(acc[i][j][3]);
-      const uint2 packed = make_uint2((uint32_t)h0 | ((uint32_t)h1 << 16), (uint32_t)h2 | ((uint32_t)h3 << 16));
-      *reinterpret_cast<uint2 *>(C + (size_t)(row0 + i * 16u) * N + col0 + j * 16u) = packed;
+    for (int jp = 0; jp < 8; jp += 2) {
+      const uint32_t p00 = mi355_pack_bf16x2(acc[i][jp][0], acc[i][jp][1]), p01 = mi355_pack_bf16x2(acc[i][jp][2], acc[i][jp][3]);
+      const uint32_t p10 = mi355_pack_bf16x2(acc[i][jp + 1][0], acc[i][jp + 1][1]), p11 = mi355_pack_bf16x2(acc[i][jp + 1][2], acc[i][jp + 1][3]);
+      const auto q01 = __builtin_amdgcn_permlane16_swap(p00, p10, false, false);
+      const auto q23 = __builtin_amdgcn_permlane16_swap(p01, p11, false, false);
+      *reinterpret_cast<uint4 *>(C + (size_t)(row0 + i * 16u) * N + col0 + jp * 16u) = make_uint4(q01[0], q23[0], q01[1], q23[1]);
     }
 }
 

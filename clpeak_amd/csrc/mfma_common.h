@@ -56,3 +56,23 @@ __device__ inline V load_bytes(const uint8_t *p) {
   __builtin_memcpy(&v, p, sizeof(V));
   return v;
 }
+
+// Two fp32 values rounded to nearest even and packed, `lo` in bits 0..15: one instruction each on
+// gfx950 (v_cvt_pk_bf16_f32, v_cvt_pk_f16_f32).  Same results as the bit-level routines of
+// numeric_formats.h for every finite input (bf16: every fp32 value; f16: gradual underflow, overflow
+// to infinity), which cost ten instructions and a branch per value.
+typedef float f32x2v __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t mi355_pack_bf16x2(float lo, float hi) {
+  typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+  const bf16x2v r = __builtin_convertvector((f32x2v){lo, hi}, bf16x2v);
+  uint32_t u;
+  __builtin_memcpy(&u, &r, sizeof(u));
+  return u;
+}
+__device__ inline uint32_t mi355_pack_f16x2(float lo, float hi) {
+  typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+  const half2v r = __builtin_convertvector((f32x2v){lo, hi}, half2v);
+  uint32_t u;
+  __builtin_memcpy(&u, &r, sizeof(u));
+  return u;
+}

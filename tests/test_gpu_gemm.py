@@ -34,7 +34,7 @@ def _rows(buf, fp8, row0, rows, K):
     return buf.download(np.uint8 if fp8 else np.uint16, rows * K, offset_bytes=row0 * K * eb)
 
 
-def _check_tiles(dev, fp8, M, N, K, tiles, tile=128):
+def _check_tiles(dev, fp8, M, N, K, tiles, tile=128, whole_output_finite=False):
     dA, dB = _operands(dev, fp8, M, N, K)
     dC = dev.alloc(M * N * 2)
     dev._check(dev.lib.mi355_memset(dev.h, dC.ptr, 0xff, M * N * 2))   # NaN pattern: unwritten output shows
@@ -44,6 +44,9 @@ def _check_tiles(dev, fp8, M, N, K, tiles, tile=128):
         dev.gemm_bf16(dA, dB, dC, M, N, K)
     fmt = orc.FMT_E4M3 if fp8 else orc.FMT_BF16
     scale = 1.0 / (FP8_SCALE * FP8_SCALE) if fp8 else 1.0
+    if whole_output_finite:
+        c = dC.download(np.uint16, M * N)
+        assert not np.any((c & 0x7f80) == 0x7f80), "an element of C was never written"
     worst = 0.0
     for (m0, n0) in tiles:
         a = _rows(dA, fp8, m0, tile, K)
@@ -85,9 +88,9 @@ def test_gemm_8192_sampled_tiles(dev, fp8):
 @pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("steps", [1, 2, 3, 4, 5, 6, 7, 11])
 def test_gemm_every_short_k_walk(dev, fp8, steps):
-    """K walks of 1..7 and 11 steps of 128 bytes: the prologue fills up to five ring slots, the
-    steady-state step needs four or more steps, and the last three steps each prefetch less; every
-    combination of those paths has its own K here.  One 256x256 tile, all four 128x128 quarters."""
+    """K walks of 1..7 and 11 steps of 128 bytes: the start fills five ring slots, which with fewer than
+    three steps already run into the workgroup's next tile (here: wrap to its only tile), and the first
+    step of a tile takes the barrier without a load wait.  One 256x256 tile, all four 128x128 quarters."""
     K = steps * (128 if fp8 else 64)
     _check_tiles(dev, fp8, 256, 256, K, [(0, 0), (0, 128), (128, 0), (128, 128)])
 
@@ -100,6 +103,19 @@ def test_gemm_non_square_grid_visits_every_tile_once(dev, fp8):
     for M, N in ((768, 1280), (2048, 512)):
         tiles = [(m, n) for m in range(0, M, 256) for n in range(0, N, 256)]
         _check_tiles(dev, fp8, M, N, 512, tiles)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("steps", [1, 2, 5])
+def test_gemm_workgroups_walk_several_tiles(dev, fp8, steps):
+    """17 x 16 = 272 tiles on a 256-CU part: workgroups are persistent, 16 of them own two tiles and the
+    ring runs through the tile boundary (with 1 and 2 steps per tile the fetch streams are a whole tile
+    or more ahead of the tile being multiplied).  Every 256x256 tile is checked on one 128x128 quarter,
+    and no element of C keeps the NaN pattern it started with."""
+    M, N, K = 17 * 256, 16 * 256, steps * (128 if fp8 else 64)
+    assert (M // 256) * (N // 256) > dev.props.num_cus
+    tiles = [(m + 128 * ((m // 256 + n // 256) % 2), n + 128 * ((m // 256) % 2)) for m in range(0, M, 256) for n in range(0, N, 256)]
+    _check_tiles(dev, fp8, M, N, K, tiles, whole_output_finite=True)
 
 
 # --- the other operand types of the same two kernels -------------------------------------------------

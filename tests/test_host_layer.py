@@ -253,3 +253,22 @@ def test_host_int8_scales_and_sparse_metadata_match_oracle(host):
     assert np.array_equal(buf, orc.fill_e8m0(seed, wl.STREAM_SCALE_A, n))
     host.clpeak_host_seeded_bytes(1, seed, wl.STREAM_SPARSE, n, buf.ctypes.data)
     assert np.array_equal(buf, orc.fill_sparse_meta(seed, wl.STREAM_SPARSE, n))
+
+
+def test_backend_workloads_equal_oracle_workloads():
+    """clpeak_amd.workloads (what bench.py hands the kernels) and oracle.workloads (what the parity tests
+    hand the kernels and the oracle) describe the same kinds and build the same bytes."""
+    from clpeak_amd import workloads as pw
+    assert sorted(pw.DENSE) == sorted(wl.DENSE) and sorted(pw.SPARSE) == sorted(wl.SPARSE)
+    for kind in pw.DENSE:
+        for key in ("name", "shape", "M", "N", "K", "scaled"):
+            assert pw.DENSE[kind][key] == wl.DENSE[kind][key]
+        for got, ref in zip(pw.dense_inputs(kind, 8), wl.dense_inputs(kind, 8)):
+            assert (got is None and ref is None) or np.array_equal(got, ref.view(np.uint8))
+        assert pw.dense_flops(kind, 2048, 4096) == wl.dense_flops(kind, 2048, 4096)
+    for kind in pw.SPARSE:
+        assert pw.SPARSE[kind]["name"] == wl.SPARSE[kind]["name"] and pw.SPARSE[kind]["K"] == wl.SPARSE[kind]["K"]
+        for got, ref in zip(pw.sparse_inputs(kind, 8), wl.sparse_inputs(kind, 8)):
+            assert np.array_equal(got, ref.view(np.uint8))
+        assert pw.sparse_flops(kind, 2048, 4096) == wl.sparse_flops(kind, 2048, 4096)
+    assert [getattr(pw, n) for n in dir(pw) if n.startswith("STREAM_")] == [getattr(wl, n) for n in dir(pw) if n.startswith("STREAM_")]
