@@ -56,31 +56,12 @@
 // walks each band in column-major order of 4-row groups so that B slabs are reused while hot.
 #include "internal.h"
 #include "mfma_common.h"
-#include "numeric_formats.h"
+#include "gemm_ring.h"
 
 namespace {
 
-constexpr int kTile = 256;        // C tile edge
-constexpr int kRowBytes = 128;    // bytes of K per step, per row
-constexpr int kThreads = 512;
-constexpr int kSlabBytes = kTile * kRowBytes;   // 32 KiB per operand per step
-
-typedef __attribute__((address_space(3))) void *lds_void_ptr;
-typedef const __attribute__((address_space(1))) void *global_void_ptr;
-
-// 16 bytes per lane from global memory straight into LDS; lane i lands at lds_dst + 16*i.
-__device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
-  __builtin_amdgcn_global_load_lds((global_void_ptr)gptr, (lds_void_ptr)(uintptr_t)lds_dst, 16, 0, 0);
-}
-
-// The same as instructions in the hand-scheduled loop: scalar base + per-lane 32-bit offset (no
-// vector ALU work per load), LDS destination through M0 (one wait state after writing it).
-#define MI355_LOAD_LDS(voff, sbase, m0val)                                                         \
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"                     \
-               :: "v"(voff), "s"(sbase), "s"(m0val) : "memory", "m0")
-
-#define MI355_DS_READ(dst, addr, off) \
-  asm volatile("ds_read_b128 %0, %1 offset:" #off : "=v"(dst) : "v"(addr))
+constexpr int kThreads = 512;   // 8 waves, 2 (M) x 4 (N), 128x64 of C each
+using Ring = GemmRing<2, 4>;
 
 // 8 A fragments (rows i*16.., 2 KiB apart) and 4 B fragments from the given LDS addresses.
 #define MI355_READ_FRAGS(fa, fb, a_addr, b_addr)                                                   \
@@ -111,142 +92,6 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
 // bf16 and f16 (K=32 per instruction, fp32 accumulate) and int8 (K=64, int32 accumulate).
 enum { kBf16 = 0, kF16 = 1, kI8 = 2, kScaledBf16 = 3 };   // kScaledBf16: output type of the fp8 kernels only
 
-// State of one wave's walk along K that the step function reads.
-struct GemmWalk {
-  uint32_t a_cur, b_cur, a_nxt, b_nxt;   // LDS byte addresses of this lane's first A / B fragment, both buffers
-  uint32_t dst_a, dst_b;                 // LDS destinations of the wave's 32 A rows / 32 B rows to fetch
-  uint64_t ga, gb;                       // uniform global addresses of those A / B rows in the next slab to fetch
-  uint32_t voff;                         // this lane's byte offset from ga / gb within a group of 8 rows
-  uint32_t row8;                         // bytes between rows r and r+8 (load q reads from base + q*row8)
-};
-
-// The tiles one workgroup owns: ids first, first + stride, ... (`mine` of them) out of tiles_m x tiles_n.
-struct TileGrid {
-  uint32_t tiles_m, tiles_n, total, first, stride, mine;
-};
-
-__device__ __forceinline__ void tile_at(const TileGrid &g, uint32_t round, uint32_t &tm, uint32_t &tn) {
-  const uint32_t id = g.first + round * g.stride;
-  uint32_t lin = id;
-  if (g.total % 8u == 0u) lin = (id % 8u) * (g.total / 8u) + id / 8u;   // tiles of one XCD are consecutive
-  // consecutive tiles walk down a group of 4 tile rows, then move one column right
-  const uint32_t per_group = 4u * g.tiles_n;
-  const uint32_t group = lin / per_group, in_group = lin - group * per_group;
-  const uint32_t rows_here = g.tiles_m - group * 4u;
-  if (rows_here >= 4u) {
-    tm = group * 4u + (in_group & 3u);
-    tn = in_group >> 2;
-  } else {
-    tm = group * 4u + in_group % rows_here;
-    tn = in_group / rows_here;
-  }
-}
-
-__device__ __forceinline__ TileGrid tiles_of_workgroup(uint32_t tiles_m, uint32_t tiles_n) {
-  TileGrid g;
-  g.tiles_m = tiles_m; g.tiles_n = tiles_n; g.total = tiles_m * tiles_n;
-  g.first = blockIdx.x; g.stride = gridDim.x;
-  g.mine = (g.total - g.first + g.stride - 1u) / g.stride;   // the host launches at most `total` workgroups
-  return g;
-}
-
-// The LDS ring of one wave and the two fetch streams (A rows three slabs ahead of the slab being
-// multiplied, B rows two ahead) through all tiles of the workgroup.  Slabs are numbered through the
-// tiles: slab g has its A rows in slot 2g mod 5 and its B rows in slot (2g+1) mod 5.
-struct GemmRing {
-  GemmWalk w;
-  TileGrid grid;
-  uint64_t a_origin, b_origin;   // A / B plus this wave's 32 rows within a tile (uniform)
-  uint32_t k_bytes, steps;
-  uint32_t lane_a, lane_b;       // this lane's first A / B fragment within a slot
-  uint32_t dst_wave;             // this wave's 4 KiB within a slot
-  uint32_t k0;                   // slot of the current slab's A rows
-  uint32_t a_round, a_left, b_round, b_left;   // tile (as a round of the workgroup) and steps left in it, per stream
-
-  __device__ __forceinline__ static uint32_t slot_off(uint32_t k) { return (k >= 5u ? k - 5u : k) * (uint32_t)kSlabBytes; }
-
-  __device__ __forceinline__ uint64_t a_rows(uint32_t round) const {
-    uint32_t tm, tn;
-    tile_at(grid, round, tm, tn);
-    return a_origin + (uint64_t)tm * kTile * k_bytes;
-  }
-  __device__ __forceinline__ uint64_t b_rows(uint32_t round) const {
-    uint32_t tm, tn;
-    tile_at(grid, round, tm, tn);
-    return b_origin + (uint64_t)tn * kTile * k_bytes;
-  }
-  __device__ __forceinline__ void place() {
-    w.a_cur = lane_a + slot_off(k0);      w.b_cur = lane_b + slot_off(k0 + 1u);
-    w.a_nxt = lane_a + slot_off(k0 + 2u); w.b_nxt = lane_b + slot_off(k0 + 3u);
-    w.dst_b = dst_wave + slot_off(k0);        // B rows two slabs ahead take over the current A slot
-    w.dst_a = dst_wave + slot_off(k0 + 1u);   // A rows three slabs ahead take over the current B slot
-  }
-  // Move a stream to its next slab: 128 bytes along K, or on to the first slab of the workgroup's next
-  // tile (after the last tile: of its first tile again, a fetch nobody reads).
-  __device__ __forceinline__ void next_a() {
-    if (--a_left == 0u) {
-      a_round = a_round + 1u == grid.mine ? 0u : a_round + 1u;
-      w.ga = a_rows(a_round);
-      a_left = steps;
-    } else {
-      w.ga += kRowBytes;
-    }
-  }
-  __device__ __forceinline__ void next_b() {
-    if (--b_left == 0u) {
-      b_round = b_round + 1u == grid.mine ? 0u : b_round + 1u;
-      w.gb = b_rows(b_round);
-      b_left = steps;
-    } else {
-      w.gb += kRowBytes;
-    }
-  }
-  __device__ __forceinline__ void fetch(uint64_t rows, uint32_t slot) const {
-#pragma unroll
-    for (uint32_t q = 0; q < 4; q++) MI355_LOAD_LDS(w.voff, rows + (uint64_t)q * w.row8, dst_wave + slot_off(slot) + q * 1024u);
-  }
-  // Fill the ring (A and B rows of slabs 0 and 1, A rows of slab 2), wait for it, and stand on slab 0.
-  __device__ __forceinline__ void start(const uint8_t *A, const uint8_t *B, uint32_t k_bytes_, uint32_t lds_base,
-                                        uint32_t wave, uint32_t lane, const TileGrid &g) {
-    const uint32_t wm = wave / 4, wn = wave % 4;
-    grid = g;
-    k_bytes = k_bytes_;
-    steps = k_bytes / kRowBytes;
-    a_origin = (uint64_t)(uintptr_t)(A + (size_t)wave * 32u * k_bytes);
-    b_origin = (uint64_t)(uintptr_t)(B + (size_t)wave * 32u * k_bytes);
-    // global -> LDS: instruction q of a wave fills rows [(wave*4+q)*8, +8) of a slab; lane i is position
-    // i%8 of row i/8, which holds logical chunk (i%8) ^ (row & 7) = (i%8) ^ (i/8).
-    const uint32_t lchunk = (lane % 8u) ^ (lane / 8u);
-    w.voff = (lane / 8u) * k_bytes + lchunk * 16u;
-    w.row8 = 8u * k_bytes;
-    dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 4096u);
-    // LDS -> fragments: row (lane%16) of the wave's sub-tile, logical chunk lane/16 (+4 for the second K
-    // half, i.e. the address with bit 6 flipped), swizzled with row&7 = lane&7.
-    const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
-    lane_a = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
-    lane_b = lds_base + (wn * 64u + lane % 16u) * kRowBytes + swz0;
-
-    a_round = b_round = 0;
-    a_left = b_left = steps;
-    w.ga = a_rows(0);
-    w.gb = b_rows(0);
-    fetch(w.ga, 0); next_a();
-    fetch(w.gb, 1); next_b();
-    fetch(w.ga, 2); next_a();
-    fetch(w.gb, 3); next_b();
-    fetch(w.ga, 4); next_a();
-    asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-    k0 = 0;
-    place();
-  }
-  __device__ __forceinline__ void advance() {
-    k0 = k0 + 2u >= 5u ? k0 + 2u - 5u : k0 + 2u;
-    place();
-    next_a();
-    next_b();
-  }
-};
-
 // The barrier of a step: every wave holds all fragments of the step's slab (its two slots are free)
 // and, loads returning in order, with its 4 youngest loads (the A rows three slabs ahead) still
 // allowed in flight, its share of the next slab has landed.  In the first step of a tile that
@@ -254,9 +99,6 @@ struct GemmRing {
 #define MI355_STEP_BARRIER(first, lds_wait)                                                        \
   asm volatile(lds_wait "s_cmp_lg_u32 %0, 0\n s_cbranch_scc1 1f\n s_waitcnt vmcnt(4)\n1:\n s_barrier"  \
                :: "s"(first) : "memory", "scc")
-
-// What every wave does once its last tile is stored: the fetches that ran ahead of it still write LDS.
-#define MI355_DRAIN_RING() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory")
 
 // Between the last matrix instruction of a tile and the first read of its accumulators: the wait
 // states the compiler cannot know about (the operands tie the youngest results to this point), then
@@ -420,7 +262,7 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
   const uint32_t wm = wave / 4, wn = wave % 4;
   const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
 
-  GemmRing ring;
+  Ring ring;
   ring.start(A, B, k_bytes, (uint32_t)(uintptr_t)lds, wave, lane, grid);
   const uint32_t steps = ring.steps;
 
@@ -560,7 +402,7 @@ gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, ui
   const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
 
   // ring, loads and fragment addresses exactly as in the bf16 kernel (rows are 128 bytes in both)
-  GemmRing ring;
+  Ring ring;
   ring.start(A, B, k_bytes, (uint32_t)(uintptr_t)lds, wave, lane, grid);
   const uint32_t steps = ring.steps;
 
@@ -618,14 +460,6 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
   return MI355_OK;
 }
 
-constexpr size_t kRingBytes = 5 * (size_t)kSlabBytes;   // five 32 KiB slots: all 160 KiB of a CU
-
-// One persistent workgroup per CU (a workgroup takes the whole LDS of one), never more than tiles.
-uint32_t workgroups(const mi355_dev *dev, uint32_t tiles) {
-  const uint32_t cus = dev->props.num_cus > 0 ? (uint32_t)dev->props.num_cus : 1u;
-  return tiles < cus ? tiles : cus;
-}
-
 template <int KIND>
 int launch_halves(mi355_dev *dev, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N,
                   uint32_t K, uint32_t elem) {
@@ -637,7 +471,7 @@ int launch_halves(mi355_dev *dev, const char *what, const void *A, const void *B
     attr_set = true;
   }
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_bf16_kernel<KIND><<<workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
+  gemm_bf16_kernel<KIND><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
       (const uint8_t *)A, (const uint8_t *)B, C, N, K * elem, tiles_m, tiles_n);
   MI355_LAUNCH_CHECK(dev, what);
   return MI355_OK;
@@ -654,7 +488,7 @@ int launch_fp8(mi355_dev *dev, const char *what, const uint8_t *A, const uint8_t
     attr_set = true;
   }
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_fp8_kernel<E5M2><<<workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(A, B, C, N, K, scale, tiles_m, tiles_n);
+  gemm_fp8_kernel<E5M2><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(A, B, C, N, K, scale, tiles_m, tiles_n);
   MI355_LAUNCH_CHECK(dev, what);
   return MI355_OK;
 }

@@ -21,30 +21,17 @@
 // a wave issues its 2 scale loads first, then 8 loads of B rows and 8 of A rows into LDS.  On entry to
 // the next step "at most 16 outstanding" means the scales are there; at its barrier "at most 8
 // outstanding" means the B rows (and everything older) have landed.
+// Workgroups are persistent and the ring runs through tile boundaries, as in gemm.hip; the scale bytes
+// are a third stream, one step ahead of the slab being multiplied.  At the end of a tile a wave waits for
+// its loads but the 8 youngest before its stores join the queue; the first step of the next tile then
+// takes neither the wait for its scale bytes nor the one at its barrier (both would count the stores).
 #include "internal.h"
 #include "mfma_common.h"
-#include "numeric_formats.h"
+#include "gemm_ring.h"
 
 namespace {
 
-constexpr int kTile = 256;
-constexpr int kRowBytes = 128;
-constexpr int kThreads = 256;
-constexpr int kSlabBytes = kTile * kRowBytes;
-constexpr size_t kRingBytes = 5 * (size_t)kSlabBytes;
-
-typedef __attribute__((address_space(3))) void *lds_void_ptr;
-typedef const __attribute__((address_space(1))) void *global_void_ptr;
-
-__device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
-  __builtin_amdgcn_global_load_lds((global_void_ptr)gptr, (lds_void_ptr)(uintptr_t)lds_dst, 16, 0, 0);
-}
-
-#define MI355_LOAD_LDS(voff, sbase, m0val)                                                         \
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"                     \
-               :: "v"(voff), "s"(sbase), "s"(m0val) : "memory", "m0")
-#define MI355_DS_READ(dst, addr, off) \
-  asm volatile("ds_read_b128 %0, %1 offset:" #off : "=v"(dst) : "v"(addr))
+constexpr int kThreads = 256;   // 4 waves, 2 (M) x 2 (N), 128x128 of C each
 #define MI355_WAIT_FRAGS16(fa, fb)                                                                 \
   asm volatile("s_waitcnt lgkmcnt(0)"                                                              \
                : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]),     \
@@ -60,14 +47,42 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
                ",0] cbsz:4 blgp:4"                                                                 \
                : "+a"(acc) : "v"(fb), "v"(fa), "v"(sb), "v"(sa))
 
-struct MxWalk {
-  uint32_t a_cur, b_cur, a_nxt, b_nxt;   // LDS byte addresses of this lane's first A / B fragment, this and the next slab
-  uint32_t dst_a, dst_b;                 // LDS destinations of the wave's 64 A rows / 64 B rows to fetch
-  uint64_t ga, gb;                       // uniform global addresses of those rows (A three slabs ahead, B two)
-  uint32_t voff, row8;                   // lane offset within a group of 8 rows; bytes between rows r and r+8
-  uint64_t sa_next, sb_next;             // uniform addresses of the next step's 1 KiB of lane-ordered scale bytes
-  uint32_t soff;                         // this lane's offset there (16 * lane)
+// The ring of the 16-bit GEMM plus the stream of lane-ordered scale bytes, one step ahead: 1 KiB per
+// block of 128 rows and step, steps of one block consecutive.
+struct MxRing : GemmRing<2, 2> {
+  const uint8_t *sal, *sbl;      // lane-ordered scales of A / B
+  uint32_t wm, wn;
+  uint64_t sa_next, sb_next;     // uniform addresses of the next step's 1 KiB per operand
+  uint32_t soff;                 // this lane's offset there (16 * lane)
+  uint32_t s_round, s_left;
+
+  __device__ __forceinline__ void scales_of(uint32_t round) {
+    uint32_t tm, tn;
+    tile_at(grid, round, tm, tn);
+    sa_next = (uint64_t)(uintptr_t)(sal + (size_t)(tm * 2u + wm) * steps * 1024u);
+    sb_next = (uint64_t)(uintptr_t)(sbl + (size_t)(tn * 2u + wn) * steps * 1024u);
+  }
+  __device__ __forceinline__ void next_scales() {
+    if (--s_left == 0u) {
+      s_round = s_round + 1u == grid.mine ? 0u : s_round + 1u;
+      scales_of(s_round);
+      s_left = steps;
+    } else {
+      sa_next += 1024;
+      sb_next += 1024;
+    }
+  }
+  __device__ __forceinline__ void advance_all() {
+    advance();
+    next_scales();
+  }
 };
+
+// The same starting a fresh accumulator tile (C = 0): what the first K half of a tile's first step issues.
+#define MI355_MFMA_MX0(H, JB, IB, acc, fb, fa, sb, sa)                                             \
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel:[" #H "," #H ",0] op_sel_hi:[" #JB "," #IB \
+               ",0] cbsz:4 blgp:4"                                                                 \
+               : "=a"(acc) : "v"(fb), "v"(fa), "v"(sb), "v"(sa))
 
 struct MxFrags {
   i32x4v a0[8], b0[8], a1[8], b1[8];     // fragment sets of the two K halves
@@ -76,26 +91,30 @@ struct MxFrags {
 };
 
 // One step of K: 128 instructions per wave, 64 on the first K half then 64 on the second.
-template <bool MAIN>
-__device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const MxWalk &w, bool reads, bool loads_a,
-                                        bool loads_b) {
-  const bool READS = MAIN || reads, LOADS_A = MAIN || loads_a, LOADS_B = MAIN || loads_b;
+// FIRST: the first step of a tile.  Its first K half starts the accumulators from zero, and it takes no
+// counted wait for loads: every outstanding load that matters was waited for at the end of the tile before,
+// and the stores issued since must not be counted.
+template <bool FIRST>
+__device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const MxRing &ring) {
+  const GemmWalk &w = ring.w;
   const uint32_t a1 = w.a_cur ^ 64u, b1 = w.b_cur ^ 64u;
   i32x4v(&fa0)[8] = f.a0; i32x4v(&fb0)[8] = f.b0; i32x4v(&fa1)[8] = f.a1; i32x4v(&fb1)[8] = f.b1;
   // the scale bytes of this step were requested a step ago, before the 16 loads into LDS
-  if (MAIN) asm volatile("s_waitcnt vmcnt(16)" : "+v"(f.sa_n), "+v"(f.sb_n));
-  else asm volatile("s_waitcnt vmcnt(0)" : "+v"(f.sa_n), "+v"(f.sb_n));
+  if (!FIRST) asm volatile("s_waitcnt vmcnt(16)" : "+v"(f.sa_n), "+v"(f.sb_n));
   f.sa = f.sa_n;
   f.sb = f.sb_n;
   // the copies are ordinary vector moves; the matrix instruction that reads one as a scale must not issue
   // right behind it, and the compiler cannot see into the assembly to space them
   asm volatile("s_nop 7" : "+v"(f.sa), "+v"(f.sb));
-#define MM(H, i, j, JB, IB) \
-  MI355_MFMA_MX(H, JB, IB, acc[i][j], (H ? fb1 : fb0)[j], (H ? fa1 : fa0)[i], f.sb[(j) / 2], f.sa[(i) / 2])
-#define LDA(q) if (LOADS_A) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
-#define LDB(q) if (LOADS_B) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
-#define SCL_A() if (READS) MI355_SCALE16(f.sa_n, w.soff, w.sa_next)
-#define SCL_B() if (READS) MI355_SCALE16(f.sb_n, w.soff, w.sb_next)
+#define MM(H, i, j, JB, IB)                                                                        \
+  do {                                                                                             \
+    if (FIRST && H == 0) MI355_MFMA_MX0(H, JB, IB, acc[i][j], fb0[j], fa0[i], f.sb[(j) / 2], f.sa[(i) / 2]); \
+    else MI355_MFMA_MX(H, JB, IB, acc[i][j], (H ? fb1 : fb0)[j], (H ? fa1 : fa0)[i], f.sb[(j) / 2], f.sa[(i) / 2]); \
+  } while (0)
+#define LDA(q) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
+#define LDB(q) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
+#define SCL_A() MI355_SCALE16(f.sa_n, ring.soff, ring.sa_next)
+#define SCL_B() MI355_SCALE16(f.sb_n, ring.soff, ring.sb_next)
   MM(0, 0, 0, 0, 0); MI355_DS_READ(fb1[0], b1, 0);
   MM(0, 0, 1, 1, 0); MI355_DS_READ(fb1[1], b1, 2048);
   MM(0, 0, 2, 0, 0); MI355_DS_READ(fb1[2], b1, 4096);
@@ -123,8 +142,8 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   MI355_WAIT_FRAGS16(fa1, fb1);
   // every read of this step's slab has returned (its two slots are free); only the 8 youngest loads, the A
   // rows three steps ahead, may still be in flight: this wave's B rows of the next slab have landed
-  if (MAIN) asm volatile("s_waitcnt vmcnt(8)\n s_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+  if (FIRST) asm volatile("s_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(8)\n s_barrier" ::: "memory");
   MM(0, 3, 0, 0, 1); SCL_B();
   MM(0, 3, 1, 1, 1); SCL_A();
   MM(0, 3, 2, 0, 1);
@@ -166,37 +185,37 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   MM(0, 7, 6, 0, 1);
   MM(0, 7, 7, 1, 1);
   MM(1, 0, 0, 0, 0); LDB(2);
-  MM(1, 0, 1, 1, 0); if (READS) MI355_DS_READ(fb0[0], w.b_nxt, 0);
+  MM(1, 0, 1, 1, 0); MI355_DS_READ(fb0[0], w.b_nxt, 0);
   MM(1, 0, 2, 0, 0);
-  MM(1, 0, 3, 1, 0); if (READS) MI355_DS_READ(fb0[1], w.b_nxt, 2048);
+  MM(1, 0, 3, 1, 0); MI355_DS_READ(fb0[1], w.b_nxt, 2048);
   MM(1, 0, 4, 0, 0); LDB(3);
-  MM(1, 0, 5, 1, 0); if (READS) MI355_DS_READ(fb0[2], w.b_nxt, 4096);
+  MM(1, 0, 5, 1, 0); MI355_DS_READ(fb0[2], w.b_nxt, 4096);
   MM(1, 0, 6, 0, 0);
-  MM(1, 0, 7, 1, 0); if (READS) MI355_DS_READ(fb0[3], w.b_nxt, 6144);
+  MM(1, 0, 7, 1, 0); MI355_DS_READ(fb0[3], w.b_nxt, 6144);
   MM(1, 1, 0, 0, 1); LDB(4);
-  MM(1, 1, 1, 1, 1); if (READS) MI355_DS_READ(fb0[4], w.b_nxt, 8192);
+  MM(1, 1, 1, 1, 1); MI355_DS_READ(fb0[4], w.b_nxt, 8192);
   MM(1, 1, 2, 0, 1);
-  MM(1, 1, 3, 1, 1); if (READS) MI355_DS_READ(fb0[5], w.b_nxt, 10240);
+  MM(1, 1, 3, 1, 1); MI355_DS_READ(fb0[5], w.b_nxt, 10240);
   MM(1, 1, 4, 0, 1); LDB(5);
-  MM(1, 1, 5, 1, 1); if (READS) MI355_DS_READ(fb0[6], w.b_nxt, 12288);
+  MM(1, 1, 5, 1, 1); MI355_DS_READ(fb0[6], w.b_nxt, 12288);
   MM(1, 1, 6, 0, 1);
-  MM(1, 1, 7, 1, 1); if (READS) MI355_DS_READ(fb0[7], w.b_nxt, 14336);
+  MM(1, 1, 7, 1, 1); MI355_DS_READ(fb0[7], w.b_nxt, 14336);
   MM(1, 2, 0, 0, 0); LDB(6);
-  MM(1, 2, 1, 1, 0); if (READS) MI355_DS_READ(fa0[0], w.a_nxt, 0);
+  MM(1, 2, 1, 1, 0); MI355_DS_READ(fa0[0], w.a_nxt, 0);
   MM(1, 2, 2, 0, 0);
-  MM(1, 2, 3, 1, 0); if (READS) MI355_DS_READ(fa0[1], w.a_nxt, 2048);
+  MM(1, 2, 3, 1, 0); MI355_DS_READ(fa0[1], w.a_nxt, 2048);
   MM(1, 2, 4, 0, 0); LDB(7);
-  MM(1, 2, 5, 1, 0); if (READS) MI355_DS_READ(fa0[2], w.a_nxt, 4096);
+  MM(1, 2, 5, 1, 0); MI355_DS_READ(fa0[2], w.a_nxt, 4096);
   MM(1, 2, 6, 0, 0);
-  MM(1, 2, 7, 1, 0); if (READS) MI355_DS_READ(fa0[3], w.a_nxt, 6144);
+  MM(1, 2, 7, 1, 0); MI355_DS_READ(fa0[3], w.a_nxt, 6144);
   MM(1, 3, 0, 0, 1); LDA(0);
-  MM(1, 3, 1, 1, 1); if (READS) MI355_DS_READ(fa0[4], w.a_nxt, 8192);
+  MM(1, 3, 1, 1, 1); MI355_DS_READ(fa0[4], w.a_nxt, 8192);
   MM(1, 3, 2, 0, 1);
-  MM(1, 3, 3, 1, 1); if (READS) MI355_DS_READ(fa0[5], w.a_nxt, 10240);
+  MM(1, 3, 3, 1, 1); MI355_DS_READ(fa0[5], w.a_nxt, 10240);
   MM(1, 3, 4, 0, 1); LDA(1);
-  MM(1, 3, 5, 1, 1); if (READS) MI355_DS_READ(fa0[6], w.a_nxt, 12288);
+  MM(1, 3, 5, 1, 1); MI355_DS_READ(fa0[6], w.a_nxt, 12288);
   MM(1, 3, 6, 0, 1);
-  MM(1, 3, 7, 1, 1); if (READS) MI355_DS_READ(fa0[7], w.a_nxt, 14336);
+  MM(1, 3, 7, 1, 1); MI355_DS_READ(fa0[7], w.a_nxt, 14336);
   MM(1, 4, 0, 0, 0); LDA(2);
   MM(1, 4, 1, 1, 0);
   MM(1, 4, 2, 0, 0);
@@ -237,13 +256,18 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
 #undef SCL_B
 }
 
-// Pre-pass: scales of one operand from row-major [rows][k32] to the per-lane order the main loop loads.
-// One wave per (block of 128 rows, K step); lane (r,g) gathers its 16 bytes and stores them as one word.
+// Pre-pass: scales from row-major [rows][k32] to the per-lane order the main loop loads, both operands
+// in one launch.  One wave per (block of 128 rows, K step); lane (r,g) gathers its 16 bytes and stores them
+// as one word.
 __global__ void __launch_bounds__(256)
-mx_scale_layout_kernel(const uint8_t *__restrict__ S, uint8_t *__restrict__ out, uint32_t k32, uint32_t steps,
-                       uint32_t units) {
-  const uint32_t unit = blockIdx.x * (blockDim.x / 64u) + threadIdx.x / 64u, lane = threadIdx.x % 64u;
-  if (unit >= units) return;
+mx_scale_layout_kernel(const uint8_t *__restrict__ SA, const uint8_t *__restrict__ SB, uint8_t *__restrict__ out_a,
+                       uint8_t *__restrict__ out_b, uint32_t k32, uint32_t steps, uint32_t units_a, uint32_t units_b) {
+  uint32_t unit = blockIdx.x * (blockDim.x / 64u) + threadIdx.x / 64u;
+  const uint32_t lane = threadIdx.x % 64u;
+  if (unit >= units_a + units_b) return;
+  const uint8_t *S = SA;
+  uint8_t *out = out_a;
+  if (unit >= units_a) { unit -= units_a; S = SB; out = out_b; }
   const uint32_t rb = unit / steps, s = unit % steps, r = lane % 16u, g = lane / 16u;
   uint32_t word[4];
 #pragma unroll
@@ -256,16 +280,6 @@ mx_scale_layout_kernel(const uint8_t *__restrict__ S, uint8_t *__restrict__ out,
   *reinterpret_cast<uint4 *>(out + ((size_t)unit * 64u + lane) * 16u) = make_uint4(word[0], word[1], word[2], word[3]);
 }
 
-__device__ inline void tile_of_block(uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm, uint32_t &tn) {
-  const uint32_t bid = blockIdx.x, total = tiles_m * tiles_n;
-  uint32_t lin = bid;
-  if (total % 8u == 0u) lin = (bid % 8u) * (total / 8u) + bid / 8u;   // tiles of one XCD are consecutive
-  const uint32_t group = lin / (4u * tiles_n), in_group = lin % (4u * tiles_n);
-  const uint32_t rows_here = (tiles_m - group * 4u) < 4u ? (tiles_m - group * 4u) : 4u;
-  tm = group * 4u + in_group % rows_here;
-  tn = in_group / rows_here;
-}
-
 __global__ void __launch_bounds__(kThreads)
 gemm_mxfp4_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const uint8_t *__restrict__ SAl,
                   const uint8_t *__restrict__ SBl, uint16_t *__restrict__ C, uint32_t N, uint32_t k_bytes,
@@ -274,93 +288,63 @@ gemm_mxfp4_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, 
   const uint32_t tid = threadIdx.x, lane = tid % 64;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const uint32_t wm = wave / 2, wn = wave % 2;
-  uint32_t tm, tn;
-  tile_of_block(tiles_m, tiles_n, tm, tn);
+  const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
 
-  // global -> LDS: wave w fills rows [64w, 64w+64) of an A slab and of a B slab, 8 rows per instruction
-  const uint32_t lchunk = (lane % 8u) ^ (lane / 8u);
-  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-  const uint32_t dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 8192u);
-  MxWalk w;
-  w.voff = (lane / 8u) * k_bytes + lchunk * 16u;
-  w.row8 = 8u * k_bytes;
-  const uint8_t *ga0 = A + ((size_t)tm * kTile + wave * 64u) * k_bytes, *gb0 = B + ((size_t)tn * kTile + wave * 64u) * k_bytes;
-  auto slot_off = [](uint32_t k) { return (k >= 5u ? k - 5u : k) * (uint32_t)kSlabBytes; };
-  auto fetch_rows = [&](const uint8_t *g, uint32_t step, uint32_t slot) {
-    const size_t kb = (size_t)step * kRowBytes;
-#pragma unroll
-    for (uint32_t q = 0; q < 8; q++) load_to_lds(g + w.voff + kb + (size_t)q * w.row8, dst_wave + slot * kSlabBytes + q * 1024u);
-  };
-  const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
-  const uint32_t lane_a = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
-  const uint32_t lane_b = lds_base + (wn * 128u + lane % 16u) * kRowBytes + swz0;
+  MxRing ring;
+  MxFrags f;
+  // the scale bytes of the first step go out first; the start of the ring waits for every load
+  ring.grid = grid;
+  ring.steps = k_bytes / kRowBytes;
+  ring.sal = SAl; ring.sbl = SBl; ring.wm = wm; ring.wn = wn;
+  ring.soff = lane * 16u;
+  ring.s_round = 0;
+  ring.s_left = ring.steps;
+  ring.scales_of(0);
+  MI355_SCALE16(f.sa_n, ring.soff, ring.sa_next);
+  MI355_SCALE16(f.sb_n, ring.soff, ring.sb_next);
+  ring.next_scales();
+  ring.start(A, B, k_bytes, (uint32_t)(uintptr_t)lds, wave, lane, grid);
+  const uint32_t steps = ring.steps;
 
   f32x4v acc[8][8];
 #pragma unroll
-  for (int i = 0; i < 8; i++)
+  for (int j = 0; j < 8; j++) asm volatile("ds_read_b128 %0, %1" : "=v"(f.b0[j]) : "v"(ring.w.b_cur + j * 2048u));
 #pragma unroll
-    for (int j = 0; j < 8; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
-  MxFrags f;
-
-  // scales in lane order (see mx_scale_layout_kernel): 1 KiB per block of 128 rows and step
-  const uint32_t steps = k_bytes / kRowBytes;
-  w.soff = lane * 16u;
-  w.sa_next = (uint64_t)(uintptr_t)(SAl + (size_t)(tm * 2u + wm) * steps * 1024u);
-  w.sb_next = (uint64_t)(uintptr_t)(SBl + (size_t)(tn * 2u + wn) * steps * 1024u);
-  MI355_SCALE16(f.sa_n, w.soff, w.sa_next);
-  MI355_SCALE16(f.sb_n, w.soff, w.sb_next);
-  w.sa_next += 1024;
-  w.sb_next += 1024;
-
-  fetch_rows(ga0, 0, 0);
-  fetch_rows(gb0, 0, 1);
-  if (steps > 1) { fetch_rows(ga0, 1, 2); fetch_rows(gb0, 1, 3); }
-  if (steps > 2) fetch_rows(ga0, 2, 4);
-  asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
-
-  uint32_t k0 = 0;   // slot of the current slab's A rows
-  auto place = [&]() {
-    w.a_cur = lane_a + slot_off(k0);      w.b_cur = lane_b + slot_off(k0 + 1u);
-    w.a_nxt = lane_a + slot_off(k0 + 2u); w.b_nxt = lane_b + slot_off(k0 + 3u);
-    w.dst_b = dst_wave + slot_off(k0);
-    w.dst_a = dst_wave + slot_off(k0 + 1u);
-  };
-  place();
-#pragma unroll
-  for (int j = 0; j < 8; j++) asm volatile("ds_read_b128 %0, %1" : "=v"(f.b0[j]) : "v"(w.b_cur + j * 2048u));
-#pragma unroll
-  for (int i = 0; i < 8; i++) asm volatile("ds_read_b128 %0, %1" : "=v"(f.a0[i]) : "v"(w.a_cur + i * 2048u));
+  for (int i = 0; i < 8; i++) asm volatile("ds_read_b128 %0, %1" : "=v"(f.a0[i]) : "v"(ring.w.a_cur + i * 2048u));
   MI355_WAIT_FRAGS16(f.a0, f.b0);
-  w.ga = (uint64_t)(uintptr_t)(ga0 + 3 * (size_t)kRowBytes);
-  w.gb = (uint64_t)(uintptr_t)(gb0 + 2 * (size_t)kRowBytes);
-  auto advance = [&]() {
-    k0 = k0 + 2u >= 5u ? k0 + 2u - 5u : k0 + 2u;
-    place();
-    w.ga += kRowBytes;
-    w.gb += kRowBytes;
-    w.sa_next += 1024;
-    w.sb_next += 1024;
-  };
-  uint32_t s = 0;
-  for (; s + 3 < steps; s++) { mx_step<true>(acc, f, w, true, true, true); advance(); }
-  for (; s < steps; s++) { mx_step<false>(acc, f, w, s + 1 < steps, false, s + 2 < steps); advance(); }
-  asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
   // A lane holds 4 consecutive N elements per 16x16 tile.  Two neighbouring tiles (j, j+1) trade halves
   // first (v_permlane16_swap: the odd lane groups of tile j against the even groups of tile j+1), so that a
   // lane stores 8 consecutive bf16 and an instruction 64 contiguous bytes per row instead of 32.
   const uint32_t g = lane / 16u;
-  const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 128u + 16u * (g & 1u) + 8u * (g >> 1);
-#pragma unroll
-  for (int i = 0; i < 8; i++)
-#pragma unroll
-    for (int jp = 0; jp < 8; jp += 2) {
-      const uint32_t p00 = mi355_pack_bf16x2(acc[i][jp][0], acc[i][jp][1]), p01 = mi355_pack_bf16x2(acc[i][jp][2], acc[i][jp][3]);
-      const uint32_t p10 = mi355_pack_bf16x2(acc[i][jp + 1][0], acc[i][jp + 1][1]), p11 = mi355_pack_bf16x2(acc[i][jp + 1][2], acc[i][jp + 1][3]);
-      const auto q01 = __builtin_amdgcn_permlane16_swap(p00, p10, false, false);
-      const auto q23 = __builtin_amdgcn_permlane16_swap(p01, p11, false, false);
-      *reinterpret_cast<uint4 *>(C + (size_t)(row0 + i * 16u) * N + col0 + jp * 16u) = make_uint4(q01[0], q23[0], q01[1], q23[1]);
+  const uint32_t row_in_tile = wm * 128u + lane % 16u, col_in_tile = wn * 128u + 16u * (g & 1u) + 8u * (g >> 1);
+
+  for (uint32_t round = 0; round < grid.mine; round++) {
+    mx_step<true>(acc, f, ring);
+    ring.advance_all();
+    for (uint32_t s = 1; s < steps; s++) {
+      mx_step<false>(acc, f, ring);
+      ring.advance_all();
     }
+    // wait states the compiler cannot know about before the accumulators are read (the operands tie the
+    // youngest results to this point), then this wave's loads but the 8 youngest before any store
+    asm volatile("s_nop 15\n s_nop 15\n s_waitcnt vmcnt(8)"
+                 : "+a"(acc[7][4]), "+a"(acc[7][5]), "+a"(acc[7][6]), "+a"(acc[7][7]) :: "memory");
+    uint32_t tm, tn;
+    tile_at(grid, round, tm, tn);
+    const uint32_t row0 = tm * kTile + row_in_tile, col0 = tn * kTile + col_in_tile;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int jp = 0; jp < 8; jp += 2) {
+        const uint32_t p00 = mi355_pack_bf16x2(acc[i][jp][0], acc[i][jp][1]), p01 = mi355_pack_bf16x2(acc[i][jp][2], acc[i][jp][3]);
+        const uint32_t p10 = mi355_pack_bf16x2(acc[i][jp + 1][0], acc[i][jp + 1][1]), p11 = mi355_pack_bf16x2(acc[i][jp + 1][2], acc[i][jp + 1][3]);
+        const auto q01 = __builtin_amdgcn_permlane16_swap(p00, p10, false, false);
+        const auto q23 = __builtin_amdgcn_permlane16_swap(p01, p11, false, false);
+        *reinterpret_cast<uint4 *>(C + (size_t)(row0 + i * 16u) * N + col0 + jp * 16u) = make_uint4(q01[0], q23[0], q01[1], q23[1]);
+      }
+  }
+  MI355_DRAIN_RING();
 }
 
 }  // namespace
@@ -394,11 +378,10 @@ extern "C" int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t 
   }
   uint8_t *sal = static_cast<uint8_t *>(dev->mx_scratch), *sbl = sal + sa_bytes;
   const uint32_t units_a = M / 128u * steps, units_b = N / 128u * steps;
-  mx_scale_layout_kernel<<<(units_a + 3) / 4, 256, 0, dev->stream>>>(scale_a, sal, k32, steps, units_a);
-  mx_scale_layout_kernel<<<(units_b + 3) / 4, 256, 0, dev->stream>>>(scale_b, sbl, k32, steps, units_b);
+  mx_scale_layout_kernel<<<(units_a + units_b + 3) / 4, 256, 0, dev->stream>>>(scale_a, scale_b, sal, sbl, k32, steps, units_a, units_b);
   MI355_LAUNCH_CHECK(dev, "mx_scale_layout");
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_mxfp4_kernel<<<tiles_m * tiles_n, kThreads, kRingBytes, dev->stream>>>(A, B, sal, sbl, C, N, K / 2u, tiles_m, tiles_n);
+  gemm_mxfp4_kernel<<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(A, B, sal, sbl, C, N, K / 2u, tiles_m, tiles_n);
   MI355_LAUNCH_CHECK(dev, "gemm_mxfp4");
   return MI355_OK;
 }

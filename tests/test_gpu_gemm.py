@@ -183,7 +183,7 @@ def test_gemm_other_types_8192_sampled_tiles(dev, kind):
 
 
 # --- block-scaled FP4 ----------------------------------------------------------------------------------
-def _check_mx(dev, M, N, K, tiles, tile=128):
+def _check_mx(dev, M, N, K, tiles, tile=128, whole_output_finite=False):
     dA, dB = dev.alloc(M * K // 2), dev.alloc(N * K // 2)
     dSA, dSB = dev.alloc(M * K // 32), dev.alloc(N * K // 32)
     dC = dev.alloc(M * N * 2)
@@ -193,6 +193,9 @@ def _check_mx(dev, M, N, K, tiles, tile=128):
     dev.fill_bytes(dSA, M * K // 32, SEED, wl.STREAM_SCALE_A, 123, 9)       # 2^-4 .. 2^4
     dev.fill_bytes(dSB, N * K // 32, SEED, wl.STREAM_SCALE_B, 123, 9)
     dev.gemm_mxfp4(dA, dB, dSA, dSB, dC, M, N, K)
+    if whole_output_finite:
+        c = dC.download(np.uint16, M * N)
+        assert not np.any((c & 0x7f80) == 0x7f80), "an element of C was never written"
     for (m0, n0) in tiles:
         a = dA.download(np.uint8, tile * K // 2, offset_bytes=m0 * K // 2)
         b = dB.download(np.uint8, tile * K // 2, offset_bytes=n0 * K // 2)
@@ -232,3 +235,13 @@ def test_gemm_mxfp4_grids_and_full_size(dev):
     rng = np.random.default_rng(4)
     tiles = [(int(m) * 128, int(n) * 128) for m, n in zip(rng.integers(0, 64, 8), rng.integers(0, 64, 8))]
     _check_mx(dev, 8192, 8192, 8192, tiles)
+
+
+@pytest.mark.parametrize("steps", [1, 2, 5])
+def test_gemm_mxfp4_workgroups_walk_several_tiles(dev, steps):
+    """272 tiles on a 256-CU part (see test_gemm_workgroups_walk_several_tiles): the A, B and scale streams
+    each cross the tile boundary at their own distance ahead of the tile being multiplied."""
+    M, N, K = 17 * 256, 16 * 256, steps * 256
+    assert (M // 256) * (N // 256) > dev.props.num_cus
+    tiles = [(m + 128 * ((m // 256 + n // 256) % 2), n + 128 * ((m // 256) % 2)) for m in range(0, M, 256) for n in range(0, N, 256)]
+    _check_mx(dev, M, N, K, tiles, whole_output_finite=True)
