@@ -32,7 +32,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # MI355X dense peaks (TFLOP/s or TOP/s); 2:4 sparse peaks are twice the dense ones.
 PEAK = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "fp6": 10100.0, "fp4": 10100.0,
-        "fp32_vec": 157.3, "fp64_vec": 78.6}
+        "fp32_vec": 157.3, "fp64_vec": 78.6, "fp32_mat": 157.3, "fp64_mat": 78.6}
 SEED = 0x5EEDC1BEA4D355
 
 
@@ -173,7 +173,9 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
     # --- GEMM 8192^3: (test, metric, bytes per element, bytes per output, peak key, unit, constant fill byte) ----
     M = N = K = 8192
     s43, s52 = 448.0, 57344.0
-    kinds = [("rocblas-fp", "fp16", 2, 2, "f16", "tflops", 0x3c),
+    kinds = [("rocblas-fp", "fp32", 4, 4, "fp32_mat", "tflops", 0x3f),
+             ("rocblas-fp", "fp64", 8, 8, "fp64_mat", "tflops", 0x3f),
+             ("rocblas-fp", "fp16", 2, 2, "f16", "tflops", 0x3c),
              ("rocblas-fp", "bf16", 2, 2, "bf16", "tflops", 0x3f),
              ("hipblaslt-fp8", "fp8_e4m3", 1, 2, "fp8", "tflops", 0x38),
              ("hipblaslt-fp8", "fp8_e5m2", 1, 2, "fp8", "tflops", 0x38),
@@ -190,6 +192,12 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
             if constant:
                 dev.memset(dSA, 0x7f); dev.memset(dSB, 0x7f)
             fn = lambda: dev.gemm_mxfp4(dA, dB, dSA, dSB, dC, M, N, K)
+        elif metric == "fp32":
+            dev.fill_f32(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_f32(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            fn = lambda: dev.gemm_f32(dA, dB, dC, M, N, K)
+        elif metric == "fp64":
+            dev.fill_f64(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_f64(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            fn = lambda: dev.gemm_f64(dA, dB, dC, M, N, K)
         elif metric == "fp16":
             dev.fill_f16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_f16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
             fn = lambda: dev.gemm_f16(dA, dB, dC, M, N, K)

@@ -22,6 +22,7 @@ SYMBOLS = [
     "mi355_gemm_bf16", "mi355_gemm_fp8_e4m3",
     "mi355_local_bandwidth", "mi355_host_alloc", "mi355_host_free", "mi355_copy_async",
     "mi355_fill_f16", "mi355_fill_fp8_e5m2", "mi355_fill_i8", "mi355_gemm_f16", "mi355_gemm_i8", "mi355_gemm_fp8_e5m2",
+    "mi355_gemm_f32", "mi355_gemm_f64", "mi355_fill_f64",
     "mi355_gemm_mxfp4", "mi355_fill_bytes",
 ]
 
@@ -90,6 +91,9 @@ def load_library(path=LIB_PATH):
     lib.mi355_fill_i8.argtypes = [vp, vp, u64, u64, u32]
     lib.mi355_gemm_f16.argtypes = [vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_gemm_i8.argtypes = [vp, vp, vp, vp, u32, u32, u32]
+    lib.mi355_gemm_f32.argtypes = [vp, vp, vp, vp, u32, u32, u32]
+    lib.mi355_gemm_f64.argtypes = [vp, vp, vp, vp, u32, u32, u32]
+    lib.mi355_fill_f64.argtypes = [vp, vp, u64, u64, u32, i32]
     lib.mi355_gemm_fp8_e5m2.argtypes = [vp, vp, vp, vp, u32, u32, u32, C.c_float, C.c_float]
     lib.mi355_gemm_mxfp4.argtypes = [vp, vp, vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_fill_bytes.argtypes = [vp, vp, u64, u64, u32, u32, u32]
@@ -263,6 +267,15 @@ class Device:
 
     def gemm_i8(self, A, B, Cbuf, M, N, K):
         self._check(self.lib.mi355_gemm_i8(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K))
+
+    def gemm_f32(self, A, B, Cbuf, M, N, K):
+        self._check(self.lib.mi355_gemm_f32(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K))
+
+    def gemm_f64(self, A, B, Cbuf, M, N, K):
+        self._check(self.lib.mi355_gemm_f64(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K))
+
+    def fill_f64(self, buf, n, seed, stream, dist):
+        self._check(self.lib.mi355_fill_f64(self.h, buf.ptr, n, seed, stream, dist))
 
     def gemm_fp8_e5m2(self, A, B, Cbuf, M, N, K, scale_a, scale_b):
         self._check(self.lib.mi355_gemm_fp8_e5m2(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K, scale_a, scale_b))

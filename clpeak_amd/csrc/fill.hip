@@ -19,6 +19,12 @@ __global__ void fill_f32_kernel(float *dst, uint64_t n, uint64_t seed, uint32_t 
     dst[i] = draw(seed, stream, i, dist);
 }
 
+__global__ void fill_f64_kernel(double *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    dst[i] = (double)draw(seed, stream, i, dist);
+}
+
 __global__ void fill_bf16_kernel(uint16_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist) {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
@@ -84,6 +90,15 @@ extern "C" int mi355_fill_f32(mi355_dev *dev, float *dst, uint64_t n, uint64_t s
   if (int rc = check_fill(dev, dst, n, dist)) return rc;
   fill_f32_kernel<<<fill_grid(n), kFillBlock, 0, dev->stream>>>(dst, n, seed, stream, dist);
   MI355_LAUNCH_CHECK(dev, "fill_f32");
+  return MI355_OK;
+}
+
+extern "C" int mi355_fill_f64(mi355_dev *dev, double *dst, uint64_t n, uint64_t seed, uint32_t stream,
+                              int dist) {
+  MI355_ENTER(dev);
+  if (int rc = check_fill(dev, dst, n, dist)) return rc;
+  fill_f64_kernel<<<fill_grid(n), kFillBlock, 0, dev->stream>>>(dst, n, seed, stream, dist);
+  MI355_LAUNCH_CHECK(dev, "fill_f64");
   return MI355_OK;
 }
 

@@ -57,6 +57,7 @@
 #include "internal.h"
 #include "mfma_common.h"
 #include "gemm_ring.h"
+#include <utility>
 
 namespace {
 
@@ -298,6 +299,102 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
   MI355_DRAIN_RING();
 }
 
+// ---- fp32 ----------------------------------------------------------------------------------------
+// Same tiling, ring, loads and LDS layout; a 128-byte row segment is 32 floats.  The fp32 matrix
+// instruction is 16x16x4 with ONE float per lane and operand (row lane%16, k = lane/16).  A lane's
+// 16-byte fragment read is chunk lane/16 of its row, i.e. floats 4*(lane/16) .. +3; register t of it,
+// used as the operand of the t-th of four instructions, makes lane group g supply k = 4g + t: the four
+// instructions together cover the 16 floats of a K half, in an order that is the same for A and B.
+// 256 instructions of 32 cycles per wave and step: the matrix pipe has four times as long per slab as
+// in the 16-bit kernel, so the memory instructions need no careful placement, only an order: the 12
+// reads of the second K half in the first 6 gaps, the barrier after instruction 7, the wave's B loads
+// then its A loads one every 16 instructions, the next step's first-half reads from instruction 208.
+template <int E>
+__device__ __forceinline__ void f32_read_fragment(f32x4v (&fa)[8], f32x4v (&fb)[4], uint32_t a_addr, uint32_t b_addr) {
+  if constexpr (E < 4) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[E]) : "v"(b_addr), "i"(2048 * E));
+  else asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[E - 4]) : "v"(a_addr), "i"(2048 * (E - 4)));
+}
+
+template <int M>
+__device__ __forceinline__ void f32_slot(f32x4v (&acc)[8][4], f32x4v (&fa0)[8], f32x4v (&fb0)[4], f32x4v (&fa1)[8],
+                                         f32x4v (&fb1)[4], const GemmWalk &w, uint32_t first, uint32_t a1, uint32_t b1) {
+  constexpr int half = M / 128, t = (M / 32) % 4, i = (M / 4) % 8, j = M % 4;
+  if constexpr (half == 0)
+    asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(fb0[j][t]), "v"(fa0[i][t]));
+  else
+    asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(fb1[j][t]), "v"(fa1[i][t]));
+  if constexpr (M < 6) {
+    f32_read_fragment<2 * M>(fa1, fb1, a1, b1);
+    f32_read_fragment<2 * M + 1>(fa1, fb1, a1, b1);
+  }
+  if constexpr (M == 7) {
+    MI355_WAIT_FRAGS(fa1, fb1);
+    MI355_STEP_BARRIER(first, "");
+  }
+  if constexpr (M >= 16 && M < 80 && M % 16 == 0)
+    MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)((M - 16) / 16) * w.row8, w.dst_b + ((M - 16) / 16) * 1024u);
+  if constexpr (M >= 136 && M < 200 && (M - 136) % 16 == 0)
+    MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)((M - 136) / 16) * w.row8, w.dst_a + ((M - 136) / 16) * 1024u);
+  if constexpr (M >= 208 && (M - 208) % 4 == 0) f32_read_fragment<(M - 208) / 4>(fa0, fb0, w.a_nxt, w.b_nxt);
+}
+
+template <int... Ms>
+__device__ __forceinline__ void f32_step(std::integer_sequence<int, Ms...>, f32x4v (&acc)[8][4], f32x4v (&fa0)[8],
+                                         f32x4v (&fb0)[4], f32x4v (&fa1)[8], f32x4v (&fb1)[4], const GemmWalk &w,
+                                         uint32_t first) {
+  const uint32_t a1 = w.a_cur ^ 64u, b1 = w.b_cur ^ 64u;   // second K half of this step
+  (f32_slot<Ms>(acc, fa0, fb0, fa1, fb1, w, first, a1, b1), ...);
+  MI355_WAIT_FRAGS(fa0, fb0);
+}
+
+__global__ void __launch_bounds__(kThreads)
+gemm_f32_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, float *__restrict__ C, uint32_t N,
+                uint32_t k_bytes, uint32_t tiles_m, uint32_t tiles_n) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t tid = threadIdx.x, lane = tid % 64;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const uint32_t wm = wave / 4, wn = wave % 4;
+  const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
+
+  Ring ring;
+  ring.start(A, B, k_bytes, (uint32_t)(uintptr_t)lds, wave, lane, grid);
+  const uint32_t steps = ring.steps;
+
+  f32x4v acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
+  f32x4v fa0[8], fb0[4], fa1[8], fb1[4];
+  MI355_READ_FRAGS(fa0, fb0, ring.w.a_cur, ring.w.b_cur);
+  MI355_WAIT_FRAGS(fa0, fb0);
+
+  uint32_t round = 0, left = steps, first = 1;
+  for (uint32_t g = grid.mine * steps; g > 0; g--) {
+    f32_step(std::make_integer_sequence<int, 256>{}, acc, fa0, fb0, fa1, fb1, ring.w, first);
+    ring.advance();
+    first = 0;
+    if (--left == 0) {
+      MI355_END_OF_TILE(acc);
+      uint32_t tm, tn;
+      tile_at(grid, round, tm, tn);
+      // 4 consecutive N elements per lane, 16 bytes: the four lane groups write 64 contiguous bytes per row
+      const uint32_t row0 = tm * kTile + wm * 128u + lane % 16u, col0 = tn * kTile + wn * 64u + 4u * (lane / 16u);
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          *reinterpret_cast<f32x4v *>(C + (size_t)(row0 + i * 16u) * N + col0 + j * 16u) = acc[i][j];
+          acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
+        }
+      round++;
+      left = steps;
+      first = 1;
+    }
+  }
+  MI355_DRAIN_RING();
+}
+
 // ---- fp8 e4m3 ------------------------------------------------------------------------------------
 // Same tiling, LDS layout, loads and barrier discipline as above; a slab of 128 bytes per row is
 // exactly one K=128 matrix instruction per 16x16 tile, 32 instructions of 32 cycles per wave and step.
@@ -505,6 +602,23 @@ extern "C" int mi355_gemm_f16(mi355_dev *dev, const uint16_t *A, const uint16_t 
                               uint32_t N, uint32_t K) {
   MI355_ENTER(dev);
   return launch_halves<kF16>(dev, "gemm_f16", A, B, C, M, N, K, 2);
+}
+
+extern "C" int mi355_gemm_f32(mi355_dev *dev, const float *A, const float *B, float *C, uint32_t M, uint32_t N,
+                              uint32_t K) {
+  MI355_ENTER(dev);
+  if (int rc = check_shapes(dev, A, B, C, M, N, K, 4)) return rc;
+  static bool attr_set = false;
+  if (!attr_set) {
+    MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f32_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
+    attr_set = true;
+  }
+  const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
+  gemm_f32_kernel<<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
+      (const uint8_t *)A, (const uint8_t *)B, C, N, K * 4, tiles_m, tiles_n);
+  MI355_LAUNCH_CHECK(dev, "gemm_f32");
+  return MI355_OK;
 }
 
 extern "C" int mi355_gemm_i8(mi355_dev *dev, const int8_t *A, const int8_t *B, int32_t *C, uint32_t M, uint32_t N,

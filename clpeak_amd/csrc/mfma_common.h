@@ -11,6 +11,9 @@
 //   B operand: lane l holds column (l % 32), same K range.
 //   C/D:       register r (0..15) of lane l is element
 //              (row 8*(r/4) + 4*(l/32) + r%4, column l % 32).
+// 16x16x4 f32 / f64 (one element per lane and operand): lane l holds row (l % 16), k = l / 16.  C/D of
+//   the f32 shape as above; of the f64 shape register r (a pair) of lane l is element
+//   (row 4*r + l/16, column l % 16): rows interleave over the lane groups.
 // f8f6f4, 16x16x128.  6-bit and 4-bit codes follow the rule above (lane l holds the 32
 //   consecutive K elements of block l/16).  8-bit codes do not: the 32 bytes of lane l
 //   are K elements [ 16*(l/16), +16 ) followed by [ 64 + 16*(l/16), +16 ), i.e. two

@@ -40,6 +40,9 @@ struct Mi355Api {
   decltype(&mi355_gemm_fp8_e5m2) gemm_fp8_e5m2;
   decltype(&mi355_gemm_mxfp4) gemm_mxfp4;
   decltype(&mi355_fill_bytes) fill_bytes;
+  decltype(&mi355_fill_f64) fill_f64;
+  decltype(&mi355_gemm_f32) gemm_f32;
+  decltype(&mi355_gemm_f64) gemm_f64;
 };
 
 const Mi355Api &mi355_real_api();   // the entry points of libclpeak_mi355.so

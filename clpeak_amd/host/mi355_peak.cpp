@@ -397,13 +397,22 @@ void Mi355Peak::runGemmRow(logger::TestScope &test, const char *metric, const ch
 
 void Mi355Peak::runGemmFp() {
   auto test = device_->beginTest({"rocblas-fp", "rocBLAS GEMM peak", "tflops", Category::Unknown,
-                                  "Square GEMM.  The fp16 and bf16 rows are this backend's hand-written MFMA kernel "
-                                  "(256x256 tiles, LDS ring, K contiguous in both operands), not a vendor library."});
-  const char *notBuilt = "No hand-written kernel for this type in the MI355X backend (no vendor BLAS is used)";
-  test.skip("fp32", ResultStatus::Unsupported, notBuilt);
-  test.skip("fp64", ResultStatus::Unsupported, notBuilt);
+                                  "Square GEMM on this backend's hand-written MFMA kernels (LDS-tiled, K contiguous in both "
+                                  "operands), not a vendor library."});
   const uint32_t D = workload.gemmDim;
   const uint64_t n = (uint64_t)D * D;
+  runGemmRow(test, "fp32", "fp32 inputs, accumulation and output, on the fp32 matrix instruction; A row-major, B column-major.", 4, 4,
+             [&](void *a, void *b) {
+               const int rc = api_.fill_f32(dev_, (float *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
+               return rc != MI355_OK ? rc : api_.fill_f32(dev_, (float *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
+             },
+             [&](void *a, void *b, void *c) { return api_.gemm_f32(dev_, (const float *)a, (const float *)b, (float *)c, D, D, D); });
+  runGemmRow(test, "fp64", "fp64 inputs, accumulation and output, on the fp64 matrix instruction; A row-major, B column-major.", 8, 8,
+             [&](void *a, void *b) {
+               const int rc = api_.fill_f64(dev_, (double *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
+               return rc != MI355_OK ? rc : api_.fill_f64(dev_, (double *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
+             },
+             [&](void *a, void *b, void *c) { return api_.gemm_f64(dev_, (const double *)a, (const double *)b, (double *)c, D, D, D); });
   runGemmRow(test, "fp16", "IEEE half inputs, fp32 accumulation, half output; A row-major, B column-major.", 2, 2,
              [&](void *a, void *b) {
                const int rc = api_.fill_f16(dev_, (uint16_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);

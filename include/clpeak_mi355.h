@@ -89,6 +89,8 @@ int mi355_timer_stop(mi355_dev *dev, float *elapsed_us);
 #define MI355_DIST_U01   0
 #define MI355_DIST_UPM1  1
 int mi355_fill_f32(mi355_dev *dev, float *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist);
+/* The same fp32 values widened to fp64 (operands of the fp64 GEMM). */
+int mi355_fill_f64(mi355_dev *dev, double *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist);
 /* Same values rounded to nearest-even bf16 (GEMM operands). */
 int mi355_fill_bf16(mi355_dev *dev, uint16_t *dst, uint64_t n, uint64_t seed, uint32_t stream, int dist);
 /* Same values multiplied by `scale` (fp32) then rounded to nearest-even OCP
@@ -253,6 +255,15 @@ int mi355_gemm_i8(mi355_dev *dev, const int8_t *A, const int8_t *B, int32_t *C,
                   uint32_t M, uint32_t N, uint32_t K);
 int mi355_gemm_fp8_e5m2(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C,
                         uint32_t M, uint32_t N, uint32_t K, float scale_a, float scale_b);
+/*   "fp32" of runRocblas (src/rocm/rocblas.cpp:246-254, rocblas_sgemm): fp32 operands, accumulation
+ *          and output, on the fp32 matrix instruction; K a multiple of 32;
+ *   "fp64" of runRocblas (src/rocm/rocblas.cpp:256-263, rocblas_dgemm): all fp64, on the fp64 matrix
+ *          instruction; M, N multiples of 128, K a multiple of 16, buffers 32-byte aligned.
+ *          Same operand layout as the rows above (K contiguous in A and in B). */
+int mi355_gemm_f32(mi355_dev *dev, const float *A, const float *B, float *C,
+                   uint32_t M, uint32_t N, uint32_t K);
+int mi355_gemm_f64(mi355_dev *dev, const double *A, const double *B, double *C,
+                   uint32_t M, uint32_t N, uint32_t K);
 
 /*   "mxf4_e2m1" of runHipblasLt (src/rocm/hipblaslt_gemm.cpp:398-512: block-scaled FP4, one
  *          UE8M0 scale per 32 elements along K, fp32 accumulate, bf16 output).  A[M][K/2] and

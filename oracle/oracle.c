@@ -527,12 +527,20 @@ int orc_smfmac(int kind, const void *Ac, const uint8_t *meta, const void *B, voi
 /* ------------------------------------------------------------------------- */
 /* C[m][n] = scale * sum_k A[m][k]*B[n][k] for m in [m0,m0+tm), n in [n0,n0+tn), summed
  * in double, returned as double (the test rounds / compares).  Operand formats: 0 f16, 1 bf16,
- * 2 e4m3fn, 3 e5m2, 7 int8 (two's complement); A and B may differ. */
-static int gemm_elem_bytes(int fmt) { return fmt == 0 || fmt == 1 ? 2 : (fmt == 2 || fmt == 3 || fmt == 7 ? 1 : 0); }
+ * 2 e4m3fn, 3 e5m2, 7 int8 (two's complement), 8 IEEE fp32, 9 IEEE fp64; A and B may differ.  The sum runs
+ * in long double so that it also stands above an fp64 product. */
+static int gemm_elem_bytes(int fmt)
+{
+    if (fmt == 8) return 4;
+    if (fmt == 9) return 8;
+    return fmt == 0 || fmt == 1 ? 2 : (fmt == 2 || fmt == 3 || fmt == 7 ? 1 : 0);
+}
 
 static double gemm_elem(int fmt, const uint8_t *p)
 {
     if (fmt == 7) return (double)(int8_t)p[0];
+    if (fmt == 8) { float f; memcpy(&f, p, 4); return (double)f; }
+    if (fmt == 9) { double d; memcpy(&d, p, 8); return d; }
     return orc_decode(fmt, gemm_elem_bytes(fmt) == 2 ? (uint32_t)(p[0] | (p[1] << 8)) : p[0]);
 }
 
@@ -554,10 +562,10 @@ int orc_gemm_tile2(int fmt_a, int fmt_b, const void *A, const void *B, uint32_t 
     #pragma omp parallel for schedule(static)
     for (uint32_t i = 0; i < tm; i++)
         for (uint32_t j = 0; j < tn; j++) {
-            double acc = 0.0;
+            long double acc = 0.0L;
             const double *ar = a + (size_t)i * K, *br = b + (size_t)j * K;
-            for (uint32_t k = 0; k < K; k++) acc += ar[k] * br[k];
-            C[(size_t)i * tn + j] = acc * scale;
+            for (uint32_t k = 0; k < K; k++) acc += (long double)ar[k] * (long double)br[k];
+            C[(size_t)i * tn + j] = (double)(acc * (long double)scale);
         }
     free(a);
     free(b);

@@ -125,7 +125,7 @@ def gemm_tile(fmt, A, B, K, lda, ldb, m0, n0, tm, tn, scale=1.0):
 
 
 def gemm_tile2(fmt_a, fmt_b, A, B, K, lda, ldb, m0, n0, tm, tn, scale=1.0):
-    """fmt: FMT_F16 / FMT_BF16 / FMT_E4M3 / FMT_E5M2 or FMT_I8; A and B may differ."""
+    """fmt: FMT_F16 / FMT_BF16 / FMT_E4M3 / FMT_E5M2, FMT_I8, FMT_F32 or FMT_F64; A and B may differ."""
     out = np.empty((tm, tn), dtype=np.float64)
     L = lib()
     L.orc_gemm_tile2.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p] + [C.c_uint32] * 7 + [C.c_double, C.c_void_p]
@@ -136,6 +136,8 @@ def gemm_tile2(fmt_a, fmt_b, A, B, K, lda, ldb, m0, n0, tm, tn, scale=1.0):
 
 
 FMT_I8 = 7
+FMT_F32 = 8
+FMT_F64 = 9
 
 
 def gemm_mx_tile(A, B, SA, SB, K, m0, n0, tm, tn):

@@ -182,6 +182,70 @@ def test_gemm_other_types_8192_sampled_tiles(dev, kind):
     _check_kind(dev, kind, 8192, 8192, 8192, tiles)
 
 
+# --- fp32 and fp64: the accumulation type is the operand type ---------------------------------------------
+def _check_wide(dev, kind, M, N, K, tiles, tile=128):
+    """kind in f32 / f64.  Bar: |gpu - ref| <= 4 sqrt(K) eps (|ref| + rms(ref tile)), eps = 2^-24 / 2^-53: K
+    roundings of a running sum of the size of the result, adding up like a random walk, times four.  The
+    reference sum runs in long double."""
+    eb, dt, eps = (4, np.float32, 2.0 ** -24) if kind == "f32" else (8, np.float64, 2.0 ** -53)
+    dA, dB, dC = dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * eb)
+    dev.memset(dC, 0xff)
+    if kind == "f32":
+        dev.fill_f32(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1)
+        dev.fill_f32(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+        dev.gemm_f32(dA, dB, dC, M, N, K)
+    else:
+        dev.fill_f64(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1)
+        dev.fill_f64(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+        dev.gemm_f64(dA, dB, dC, M, N, K)
+    fmt = orc.FMT_F32 if kind == "f32" else orc.FMT_F64
+    worst = 0.0
+    for (m0, n0) in tiles:
+        a = dA.download(dt, tile * K, offset_bytes=m0 * K * eb)
+        b = dB.download(dt, tile * K, offset_bytes=n0 * K * eb)
+        ref = orc.gemm_tile2(fmt, fmt, a, b, K, K, K, 0, 0, tile, tile, 1.0)
+        got = np.empty((tile, tile), dtype=np.float64)
+        for i in range(tile):
+            got[i] = dC.download(dt, tile, offset_bytes=((m0 + i) * N + n0) * eb)
+        assert np.all(np.isfinite(got)), (m0, n0)
+        rms = float(np.sqrt((ref ** 2).mean()))
+        err = np.abs(got - ref)
+        bound = 4.0 * np.sqrt(K) * eps * (np.abs(ref) + rms)
+        assert np.all(err <= bound), (m0, n0, float((err / bound).max()))
+        worst = max(worst, float((err / bound).max()))
+    for b in (dA, dB, dC):
+        b.free()
+    return worst
+
+
+def test_fill_f64_is_the_fp32_stream_widened(dev):
+    n = (1 << 16) + 5
+    buf = dev.alloc(n * 8)
+    for dist in (capi.DIST_U01, capi.DIST_UPM1):
+        dev.fill_f64(buf, n, SEED, wl.STREAM_GEMM_A, dist)
+        got = buf.download(np.float64, n)
+        assert np.array_equal(got, orc.fill_f32(n, SEED, wl.STREAM_GEMM_A, dist).astype(np.float64))
+    buf.free()
+
+
+@pytest.mark.parametrize("kind", ["f32", "f64"])
+@pytest.mark.parametrize("steps", [1, 2, 3, 4, 5, 9])
+def test_gemm_wide_types_short_walks(dev, kind, steps):
+    K = steps * (32 if kind == "f32" else 16)
+    _check_wide(dev, kind, 256, 256, K, [(0, 0), (0, 128), (128, 0), (128, 128)])
+
+
+@pytest.mark.parametrize("kind", ["f32", "f64"])
+def test_gemm_wide_types_grids_and_full_size(dev, kind):
+    """Non-square tile grids (every tile checked), more tiles than CUs with a short K, and 8192^3 on sampled tiles."""
+    for M, N in ((768, 1280), (2048, 512)):
+        _check_wide(dev, kind, M, N, 256, [(m, n) for m in range(0, M, 128) for n in range(0, N, 128)])
+    _check_wide(dev, kind, 17 * 256, 16 * 256, 64, [(m, n + 128 * ((m // 256) % 2)) for m in range(0, 17 * 256, 256) for n in range(0, 16 * 256, 256)])
+    rng = np.random.default_rng(5)
+    tiles = [(int(m) * 128, int(n) * 128) for m, n in zip(rng.integers(0, 64, 8), rng.integers(0, 64, 8))]
+    _check_wide(dev, kind, 8192, 8192, 8192, tiles)
+
+
 # --- block-scaled FP4 ----------------------------------------------------------------------------------
 def _check_mx(dev, M, N, K, tiles, tile=128, whole_output_finite=False):
     dA, dB = dev.alloc(M * K // 2), dev.alloc(N * K // 2)

@@ -84,13 +84,13 @@ def test_full_run_row_contract_and_xml(tmp_path):
         assert cat == CATEGORY_OF_UNIT[unit]
     # measured values carry exactly 4 decimals
     vals = [m[2] for _, _, _, ms in rows for m in ms if m[1] is None]
-    assert len(vals) == 47 and all(re.fullmatch(r"-?\d+\.\d{4}", v) for v in vals)
+    assert len(vals) == 49 and all(re.fullmatch(r"-?\d+\.\d{4}", v) for v in vals)
     # rows that are deliberate skips keep the reference's status
     status = {(t, m[0]): m[1] for _, t, _, ms in rows for m in ms}
     assert status[("kernel_launch_latency", "dispatch")] == "unsupported"
     assert status[("image_memory_bandwidth", "float4")] == "unsupported"
     assert status[("wmma_fp16", "wmma_fp16")] == "unsupported"
-    assert status[("rocblas-fp", "bf16")] is None and status[("rocblas-fp", "fp32")] == "unsupported"
+    assert status[("rocblas-fp", "bf16")] is None and status[("rocblas-fp", "fp32")] is None and status[("rocblas-fp", "fp64")] is None
     assert status[("hipblaslt-fp8", "fp8_e4m3")] is None
 
 

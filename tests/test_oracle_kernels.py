@@ -355,3 +355,29 @@ def test_generic_fill_matches_library_roundings():
     # beyond the largest finite value the fill saturates (torch would give inf there)
     sat = orc.fill_fmt(orc.FMT_E5M2, n, wl.DEFAULT_SEED, wl.STREAM_GEMM_A, 1, 1e6)
     assert set(np.unique(sat & 0x7f)) <= set(range(0x7c)) and (sat & 0x7f).max() == 0x7b
+
+
+def test_gemm_tile2_fp32_and_fp64_against_exact_sums():
+    """fp32 / fp64 operands.  The tile sums run in long double: against math.fsum of the exact products
+    (products of two fp32 values are exact in double; for fp64 operands the test uses values with 20-bit
+    mantissas so that theirs are too) the result is the correctly rounded sum, or next to it."""
+    import math
+    rng = np.random.default_rng(7)
+    a = rng.standard_normal((5, 96)).astype(np.float32)
+    b = rng.standard_normal((4, 96)).astype(np.float32)
+    got = orc.gemm_tile2(orc.FMT_F32, orc.FMT_F32, a, b, 96, 96, 96, 1, 0, 3, 4)
+    want = np.array([[math.fsum(float(x) * float(y) for x, y in zip(a[1 + i], b[j])) for j in range(4)] for i in range(3)])
+    assert np.allclose(got, want, rtol=4e-16, atol=0)
+    # fp64 with a cancellation a double-only sum gets visibly wrong: 2^40 + (terms with 20 fraction bits) - 2^40
+    da = np.round(rng.standard_normal((2, 64)) * 2 ** 10) / 2 ** 10
+    db = np.round(rng.standard_normal((3, 64)) * 2 ** 10) / 2 ** 10
+    da[:, 0] = 2.0 ** 20; db[:, 0] = 2.0 ** 20; da[:, 63] = -(2.0 ** 20); db[:, 63] = 2.0 ** 20
+    got = orc.gemm_tile2(orc.FMT_F64, orc.FMT_F64, da, db, 64, 64, 64, 0, 0, 2, 3, 0.25)
+    want = np.array([[0.25 * math.fsum(float(x) * float(y) for x, y in zip(da[i], db[j])) for j in range(3)] for i in range(2)])
+    assert np.array_equal(got, want)
+    plain = 0.25 * np.array([[sum(float(x) * float(y) for x, y in zip(da[i], db[j])) for j in range(3)] for i in range(2)])
+    assert not np.array_equal(plain, want)          # the case does tell a double sum from a wider one
+    # transposition or a wrong leading dimension shows: a non-square tile out of a larger matrix
+    big_a = rng.standard_normal((8, 32)); big_b = rng.standard_normal((6, 32))
+    got = orc.gemm_tile2(orc.FMT_F64, orc.FMT_F64, big_a, big_b, 32, 32, 32, 2, 1, 4, 3)
+    assert np.allclose(got, big_a[2:6] @ big_b[1:4].T, rtol=1e-13, atol=1e-13)
