@@ -130,3 +130,25 @@ def test_gemm_mxfp4_keeps_asynchronous_results_out_of_scratch(tmp_path):
     assert inner and any(sum("v_mfma_scale" in x for x in lines[a:b]) == 128 for a, b in inner)
     for a, b in inner:
         assert not any("scratch_" in x for x in lines[a:b]), (a, b)
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_gemm_fp32_and_fp64_kernels(tmp_path):
+    """fp32: the ring kernel with four 16x16x4 instructions per 16-byte fragment read, 256 per step.
+    fp64: 64 instructions per step, two 32 KiB buffers (64 KiB static LDS, two workgroups per CU)."""
+    asm = device_asm(tmp_path, "gemm.hip")
+    meta = kernel_metadata(asm)
+    name = next(k for k in meta if "gemm_f32_kernel" in k)
+    assert meta[name]["vgpr_spill_count"] == 0 and meta[name]["private_segment_fixed_size"] == 0 and meta[name]["vgpr_count"] <= 256
+    body = kernel_body(asm, name)
+    assert body.count("v_mfma_f32_16x16x4_f32") == 256 and "ds_write" not in body
+    asm = device_asm(tmp_path, "gemm_f64.hip")
+    meta = kernel_metadata(asm)
+    name = next(k for k in meta if "gemm_f64_kernel" in k)
+    assert meta[name]["vgpr_spill_count"] == 0 and meta[name]["private_segment_fixed_size"] == 0 and meta[name]["vgpr_count"] <= 256
+    assert meta[name]["group_segment_fixed_size"] == 65536
+    body = kernel_body(asm, name)
+    assert body.count("v_mfma_f64_16x16x4_f64") == 64 and "ds_write" not in body
+    # the step's matrix instructions stay ahead of the wait for the next slab's loads
+    loop = body[body.index("v_mfma_f64_16x16x4_f64"):]
+    assert loop.rindex("v_mfma_f64_16x16x4_f64") < loop.index("s_barrier")
