@@ -561,12 +561,7 @@ template <int KIND>
 int launch_halves(mi355_dev *dev, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N,
                   uint32_t K, uint32_t elem) {
   if (int rc = check_shapes(dev, A, B, C, M, N, K, elem)) return rc;
-  static bool attr_set = false;
-  if (!attr_set) {
-    MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_bf16_kernel<KIND>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
-    attr_set = true;
-  }
+  if (int rc = allow_full_lds(dev, &gemm_bf16_kernel<KIND>, KIND == kBf16 ? kLdsBf16 : KIND == kF16 ? kLdsF16 : kLdsI8)) return rc;
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
   gemm_bf16_kernel<KIND><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
       (const uint8_t *)A, (const uint8_t *)B, C, N, K * elem, tiles_m, tiles_n);
@@ -578,12 +573,7 @@ template <bool E5M2>
 int launch_fp8(mi355_dev *dev, const char *what, const uint8_t *A, const uint8_t *B, uint16_t *C, uint32_t M,
                uint32_t N, uint32_t K, float scale) {
   if (int rc = check_shapes(dev, A, B, C, M, N, K, 1)) return rc;
-  static bool attr_set = false;
-  if (!attr_set) {
-    MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_fp8_kernel<E5M2>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
-    attr_set = true;
-  }
+  if (int rc = allow_full_lds(dev, &gemm_fp8_kernel<E5M2>, E5M2 ? kLdsFp8E5m2 : kLdsFp8E4m3)) return rc;
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
   gemm_fp8_kernel<E5M2><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(A, B, C, N, K, scale, tiles_m, tiles_n);
   MI355_LAUNCH_CHECK(dev, what);
@@ -608,12 +598,7 @@ extern "C" int mi355_gemm_f32(mi355_dev *dev, const float *A, const float *B, fl
                               uint32_t K) {
   MI355_ENTER(dev);
   if (int rc = check_shapes(dev, A, B, C, M, N, K, 4)) return rc;
-  static bool attr_set = false;
-  if (!attr_set) {
-    MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f32_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
-    attr_set = true;
-  }
+  if (int rc = allow_full_lds(dev, &gemm_f32_kernel, kLdsF32)) return rc;
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
   gemm_f32_kernel<<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
       (const uint8_t *)A, (const uint8_t *)B, C, N, K * 4, tiles_m, tiles_n);

@@ -357,12 +357,7 @@ extern "C" int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t 
   MI355_REQUIRE(dev, M % kTile == 0 && N % kTile == 0, "gemm_mxfp4: M (%u) and N (%u) must be multiples of 256", M, N);
   MI355_REQUIRE(dev, K % 256 == 0, "gemm_mxfp4: K (%u) must be a multiple of 256", K);
   MI355_REQUIRE(dev, (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) == 0, "gemm_mxfp4: buffers must be 16-byte aligned");
-  static bool attr_set = false;
-  if (!attr_set) {
-    MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mxfp4_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRingBytes));
-    attr_set = true;
-  }
+  if (int rc = allow_full_lds(dev, &gemm_mxfp4_kernel, kLdsMxfp4)) return rc;
   // lane-ordered copies of the scales live in a scratch buffer the handle keeps (same size as the scales)
   const uint32_t k32 = K / 32u, steps = K / 256u;
   const size_t sa_bytes = (size_t)M * k32, sb_bytes = (size_t)N * k32;

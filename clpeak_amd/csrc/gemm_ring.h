@@ -172,6 +172,18 @@ struct GemmRing {
 
 constexpr size_t kRingBytes = 5 * (size_t)kSlabBytes;   // five 32 KiB slots: all 160 KiB of a CU
 
+// A kernel that takes the whole LDS must be allowed to, once per device handle (the attribute belongs to
+// the function on the handle's device).  `bit` names the kernel within mi355_dev::full_lds_allowed.
+enum { kLdsBf16 = 0, kLdsF16, kLdsI8, kLdsFp8E4m3, kLdsFp8E5m2, kLdsF32, kLdsMxfp4 };
+template <typename Kernel>
+inline int allow_full_lds(mi355_dev *dev, Kernel kernel, unsigned bit) {
+  if (dev->full_lds_allowed & (1u << bit)) return MI355_OK;
+  MI355_HIP(dev, hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)kRingBytes));
+  dev->full_lds_allowed |= 1u << bit;
+  return MI355_OK;
+}
+
 // One persistent workgroup per CU (a workgroup takes the whole LDS of one), never more than tiles.
 inline uint32_t gemm_workgroups(const mi355_dev *dev, uint32_t tiles) {
   const uint32_t cus = dev->props.num_cus > 0 ? (uint32_t)dev->props.num_cus : 1u;

@@ -16,6 +16,8 @@ struct mi355_dev {
   // scratch owned by the handle: scale bytes of the block-scaled GEMM laid out per lane (grown on demand)
   void        *mx_scratch = nullptr;
   size_t       mx_scratch_bytes = 0;
+  // GEMM kernels that have been allowed the whole LDS of a CU on this device (one bit per kernel)
+  uint32_t     full_lds_allowed = 0;
 };
 
 // Error text for failures that have no handle to hang on (open, device_count).

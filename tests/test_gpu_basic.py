@@ -38,6 +38,19 @@ def test_argument_errors_are_reported_not_launched(dev):
     with pytest.raises(capi.Mi355Error) as e:
         dev.gemm_bf16(out, out, out, 100, 256, 64)
     assert "multiples of 256" in str(e.value)
+    # every GEMM entry point refuses a shape its tiling cannot cover, before anything is launched
+    for call, text in ((lambda: dev.gemm_f16(out, out, out, 256, 256, 96), "multiple of 64"),
+                       (lambda: dev.gemm_i8(out, out, out, 256, 256, 64), "multiple of 128"),
+                       (lambda: dev.gemm_f32(out, out, out, 256, 256, 48), "multiple of 32"),
+                       (lambda: dev.gemm_f32(out, out, out, 128, 256, 64), "multiples of 256"),
+                       (lambda: dev.gemm_f64(out, out, out, 64, 128, 16), "multiples of 128"),
+                       (lambda: dev.gemm_f64(out, out, out, 128, 128, 8), "multiple of 16"),
+                       (lambda: dev.gemm_fp8_e4m3(out, out, out, 256, 256, 100, 1.0, 1.0), "multiple of 128"),
+                       (lambda: dev.gemm_fp8_e5m2(out, out, out, 256, 0, 128, 1.0, 1.0), "empty"),
+                       (lambda: dev.gemm_mxfp4(out, out, out, out, out, 256, 256, 128), "multiple of 256")):
+        with pytest.raises(capi.Mi355Error) as e:
+            call()
+        assert e.value.code == capi.ERR_ARG and text in str(e.value), str(e.value)
     out.free()
 
 
