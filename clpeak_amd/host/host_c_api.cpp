@@ -3,6 +3,7 @@
 #include <cstring>
 #include <sstream>
 #include "mi355_peak.h"
+#include "results.h"
 #include "seeded_inputs.h"
 
 extern "C" {
@@ -33,6 +34,15 @@ void clpeak_host_config_for_device(unsigned type, unsigned long long out[6]) {
   const benchmark_config_t c = benchmark_config_t::forDevice((DeviceType)type);
   out[0] = c.globalBWMaxSize; out[1] = c.computeWgsPerCU; out[2] = c.computeDPWgsPerCU;
   out[3] = c.transferBWMaxSize; out[4] = c.targetTimeUs; out[5] = c.kernelLatencyIters;
+}
+
+// Load a result file (any of the three formats, by extension) and write it out again as `fmt`
+// (0 XML, 1 JSON, 2 CSV).  Returns the number of rows loaded, or -1 when saving failed.
+int clpeak_host_resave(const char *in_path, const char *out_path, int fmt) {
+  DeviceInfoStore devices;
+  const ResultStore store = loadResultFile(in_path, &devices);
+  const bool ok = fmt == 0 ? saveXml(store, out_path, devices) : fmt == 1 ? saveJson(store, out_path, devices) : saveCsv(store, out_path);
+  return ok ? (int)store.size() : -1;
 }
 
 int clpeak_host_cancel_requested(void) { return clpeak::cancelRequested() ? 1 : 0; }

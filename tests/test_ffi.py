@@ -173,3 +173,20 @@ def test_load_result_file_rejects_garbage(ffi, tmp_path):
     bad = tmp_path / "bad.json"
     bad.write_text("{not json")
     assert ffi.clpeak_load_result_file_json(str(bad).encode()) is None
+
+
+def test_loads_a_result_file_the_reference_wrote(ffi):
+    """clpeak_load_result_file_json on a file from the reference's results/ (tests/golden, copied as data):
+    every row arrives with the keys the GUI's model reads, values and skip reasons intact."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_results_amd_threadripper.xml")
+    doc = json.loads(take_string(ffi, ffi.clpeak_load_result_file_json(path.encode())))
+    assert doc["format_version"] == 2 and len(doc["entries"]) == 192
+    first = doc["entries"][0]
+    assert (first["backend"], first["category"], first["test"], first["metric"], first["unit"]) == \
+        ("Vulkan", "fp_compute", "single_precision_compute", "float", "gflops")
+    assert abs(first["value"] - 229.0884) < 1e-3 and "status" not in first      # measured rows carry a value, skipped ones a status
+    assert first["device"] == "llvmpipe (LLVM 22.1.8, 256 bits)" and first["display"] == "Single-precision compute"
+    skipped = [e for e in doc["entries"] if e.get("status") == "unsupported"]
+    assert skipped and all(e["reason"] and "value" not in e for e in skipped)
+    assert any(e["reason"].startswith("VK_KHR_shader_bfloat16") for e in skipped)
+    assert ffi.clpeak_load_result_file_json(b"/nonexistent/file.xml") is None

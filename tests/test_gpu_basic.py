@@ -262,3 +262,29 @@ def test_transfer_batches_time_like_kernels(dev):
         dev.copy_async(dbuf.ptr, hp, nbytes, 7)
     dbuf.free()
     dev.host_free(hp)
+
+
+def test_device_fills_reproduce_the_committed_streams(dev):
+    """The first 16 elements of every device fill against tests/golden/seeded_streams.json (the fixture the
+    oracle and the host generator are held to as well)."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "seeded_streams.json")) as f:
+        g = json.load(f)
+    n, seed = g["count"], g["seed"]
+    buf = dev.alloc(n * 8)
+    dev.fill_f32(buf, n, seed, wl.STREAM_BW, capi.DIST_U01)
+    assert [int(x) for x in buf.download(np.uint32, n)] == g["f32"]["bw_u01"]
+    dev.fill_f32(buf, n, seed, wl.STREAM_GEMM_A, capi.DIST_UPM1)
+    assert [int(x) for x in buf.download(np.uint32, n)] == g["f32"]["gemm_a_upm1"]
+    dev.fill_f64(buf, n, seed, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+    assert [int(x) for x in buf.download(np.float64, n).astype(np.float32).view(np.uint32)] == g["f32"]["gemm_b_upm1"]
+    dev.fill_bf16(buf, n, seed, wl.STREAM_GEMM_A, capi.DIST_UPM1)
+    assert [int(x) for x in buf.download(np.uint16, n)] == g["operands"]["gemm_a_bf16"]
+    dev.fill_fp8_e4m3(buf, n, seed, wl.STREAM_GEMM_A, capi.DIST_UPM1, 448.0)
+    assert [int(x) for x in buf.download(np.uint8, n)] == g["operands"]["gemm_a_e4m3_x448"]
+    dev.fill_bytes(buf, n, seed, wl.STREAM_GEMM_A, 0, 256)
+    assert [int(x) for x in buf.download(np.uint8, n)] == g["bytes"]["gemm_a_fp4_pairs"]
+    dev.fill_bytes(buf, n, seed, wl.STREAM_SCALE_A, 123, 9)
+    assert [int(x) for x in buf.download(np.uint8, n)] == g["bytes"]["gemm_scale_a_123_9"]
+    buf.free()

@@ -2,6 +2,7 @@
 against the stand-in device, so row set, order, gating, degrade paths and the dump formats are
 all exercised; no kernel runs."""
 import ctypes as C
+import json
 import os
 import re
 import subprocess
@@ -272,3 +273,36 @@ def test_backend_workloads_equal_oracle_workloads():
             assert np.array_equal(got, ref.view(np.uint8))
         assert pw.sparse_flops(kind, 2048, 4096) == wl.sparse_flops(kind, 2048, 4096)
     assert [getattr(pw, n) for n in dir(pw) if n.startswith("STREAM_")] == [getattr(wl, n) for n in dir(pw) if n.startswith("STREAM_")]
+
+
+# ---- the reference's own result files (tests/golden/reference_results_*.xml, copied as data from its results/) ----
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+@pytest.mark.parametrize("name,rows", [("reference_results_amd_threadripper.xml", 192),
+                                       ("reference_results_nvidia_rtx5060.xml", 217),
+                                       ("reference_results_apple_m1pro.xml", 212)])
+def test_reference_result_files_survive_load_and_save_byte_for_byte(host, tmp_path, name, rows):
+    """The three result files the reference ships were written by its own result store.  Loading one here
+    and saving it again must give the same bytes, line for line, but for the root element (which names
+    the writing program's version and OS): that pins the loader (every attribute, status, reason, prop,
+    entity) and the writer (order, indentation, escaping, number format) to the reference's at once.
+    The same rows then go through this backend's JSON and come back unchanged."""
+    host.clpeak_host_resave.argtypes = [C.c_char_p, C.c_char_p, C.c_int]
+    src = os.path.join(GOLDEN, name)
+    out = tmp_path / "again.xml"
+    assert host.clpeak_host_resave(src.encode(), str(out).encode(), 0) == rows
+    want, got = open(src, encoding="utf-8").read().split("\n"), out.read_text(encoding="utf-8").split("\n")
+    assert len(want) == len(got)
+    assert want[1].startswith("<clpeak format_version=\"2\"") and got[1].startswith("<clpeak format_version=\"2\"")
+    assert want[:1] + want[2:] == got[:1] + got[2:]
+    # XML -> JSON -> XML
+    js, back = tmp_path / "again.json", tmp_path / "back.xml"
+    assert host.clpeak_host_resave(src.encode(), str(js).encode(), 1) == rows
+    assert host.clpeak_host_resave(str(js).encode(), str(back).encode(), 0) == rows
+    assert back.read_text(encoding="utf-8") == out.read_text(encoding="utf-8")
+    doc = json.loads(js.read_text(encoding="utf-8"))
+    assert doc["format_version"] == 2
+    # CSV keeps every row (it has no device properties)
+    assert host.clpeak_host_resave(src.encode(), str(tmp_path / "again.csv").encode(), 2) == rows
+    assert host.clpeak_host_resave(str(tmp_path / "again.csv").encode(), str(tmp_path / "c.xml").encode(), 0) == rows

@@ -154,3 +154,45 @@ def test_operand_builders():
     c = orc.fill_normal_codes(orc.FMT_F16, 0.01, 9, 2, 20000)
     v = c.view(np.float16).astype(np.float64)
     assert abs(v.std() - 0.01) < 3e-4 and abs(v.mean()) < 3e-4
+
+
+# ---- the committed fixture of the seeded streams ------------------------------------------------------
+def _golden_streams():
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "seeded_streams.json")
+    with open(path) as f:
+        return json.load(f)
+
+
+def test_oracle_reproduces_the_committed_streams():
+    """tests/golden/seeded_streams.json was written once by tests/golden/make_seeded_streams.py; building it
+    again must give the same document, value for value."""
+    import importlib.util
+    import os
+    spec = importlib.util.spec_from_file_location(
+        "make_seeded_streams", os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "make_seeded_streams.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert mod.build() == _golden_streams()
+
+
+def test_host_generator_reproduces_the_committed_streams():
+    """The backend's own host-side generator (what Mi355Peak uploads, what bench.py measures on) against the
+    same fixture, without the oracle in between."""
+    from clpeak_amd import workloads as pw
+    g = _golden_streams()
+    n, seed = g["count"], g["seed"]
+    assert seed == pw.DEFAULT_SEED
+    for name, fmt, sigma in (("f16", pw.F16, 0.01), ("bf16", pw.BF16, 0.01), ("e4m3", pw.E4M3, 1.0), ("e5m2", pw.E5M2, 1.0)):
+        got = pw.operand(fmt, sigma, seed, pw.STREAM_MFMA_A, n)
+        codes = got.view(np.uint16) if fmt in (pw.F16, pw.BF16) else got
+        assert [int(x) for x in codes] == g["operands"][name], name
+    # 6- and 4-bit codes come packed: unpack little-endian bit fields
+    for name, fmt, bits in (("e2m3", pw.E2M3, 6), ("e3m2", pw.E3M2, 6), ("e2m1", pw.E2M1, 4)):
+        packed = pw.operand(fmt, 1.0, seed, pw.STREAM_MFMA_A, n)
+        word = int.from_bytes(bytes(packed), "little")
+        assert [(word >> (bits * i)) & ((1 << bits) - 1) for i in range(n)] == g["operands"][name], name
+    assert [int(x) for x in pw.operand(pw.I8, 0.0, seed, pw.STREAM_MFMA_B, n).view(np.int8)] == g["operands"]["int8"]
+    assert [int(x) for x in pw.e8m0_scales(seed, pw.STREAM_SCALE_A, n)] == g["bytes"]["e8m0_scale_a"]
+    assert [int(x) for x in pw.sparse_meta(seed, pw.STREAM_SPARSE, n)] == g["bytes"]["sparse_meta"]
