@@ -97,6 +97,13 @@ def test_quick_run_streams_events_and_saves_xml(ffi, tmp_path):
     assert metrics and metrics[0]["backend"] == "ROCm"
     assert any(m["status"] == "ok" and m["value"] > 0 for m in metrics)
     assert {"category", "test", "display", "metric", "unit", "value", "status", "reason", "sub", "desc", "minfo"} <= set(metrics[0])
+    # the fields the GUI's event model decodes, and the row key it builds from them (app/test/models_test.dart:107-131)
+    m0 = metrics[0]
+    assert {"backend", "platform", "device", "driver", "category", "test", "display", "metric", "unit", "value", "status",
+            "reason", "sub"} <= set(m0)
+    assert isinstance(m0["sub"], bool) and isinstance(m0["value"], float) and m0["reason"] == ""
+    key = "/".join(m0[k] for k in ("backend", "platform", "device", "category", "test", "metric"))
+    assert key == "ROCm/ROCm/Fake MI355X/fp_compute/single_precision_compute/float"
     # what a test measures arrives on test_begin, a reading's own note rides the row
     begin = next(e for e in events if e["t"] == "test_begin" and e["test"] == "global_memory_bandwidth")
     assert begin["desc"] and begin["unit"] == "gbps" and begin["category"] == "bandwidth"
