@@ -1,5 +1,7 @@
-// Hand-written MFMA GEMM:  C[M][N] (bf16) = scale * A[M][K] . B[N][K]^T, fp32 accumulate.
-// Both operands are K-contiguous ("row-major A, column-major B").
+// Hand-written MFMA GEMM:  C[M][N] = scale * A[M][K] . B[N][K]^T.  Both operands are K-contiguous
+// ("row-major A, column-major B").  Operand types: bf16, f16, fp8 (e4m3, or an e5m2 A against an e4m3 B)
+// with fp32 accumulation and a 16-bit C; int8 with an int32 C; fp32.  The tile walk, the LDS ring and the
+// persistent workgroups live in gemm_ring.h and are shared with gemm_mxfp4.hip.
 //
 // Tiling.  One workgroup of 512 threads (8 waves, 2 per SIMD) owns a 256x256 tile
 // of C and walks K in steps of one 128-byte row segment (64 bf16 or 128 fp8
@@ -39,8 +41,8 @@
 // states of its own: every s_waitcnt below is part of the schedule.
 //
 // The MFMA is issued with the B fragment as the first operand, which produces the
-// transposed 16x16 tile: a lane then holds 4 consecutive N elements of one C row and
-// stores them as one 8-byte word.
+// transposed 16x16 tile: a lane then holds 4 consecutive N elements of one C row (see store_tile for
+// how they leave).
 //
 // Workgroups are persistent: one per CU (the ring takes the whole LDS), each walking the
 // tiles id, id + grid, id + 2*grid, ...  The ring does not stop at a tile boundary: slabs are
