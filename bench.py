@@ -296,9 +296,15 @@ def cpu_baseline(target_us=2_000_000, extra_target_us=1_000_000):
             q = pool.measure(kind, SEED, 2, extra_target_us)
             port[name] = {"ST": round(q.giga_st, 3), "MT": round(q.giga_mt, 3), "unit": unit, "threads": q.threads_mt,
                           "iters_ST": q.iters_st, "iters_MT": q.iters_mt, "sample": what}
+        # the other two rows of the reference's DRAM test, restated (all workers only, as it times them)
+        n_stream, llc = _stream_floats(cores)
+        for name, kind, what in (("global_memory_bandwidth copy", 0, "memcpy of one array into another, 2 x 4 bytes per element"),
+                                 ("global_memory_bandwidth triad", 1, "a[i] = b[i] + 1.5 c[i], 3 x 4 bytes per element")):
+            q, _ = pool.measure_stream(pool.own_populate_ptr(), n_stream, kind, 1, extra_target_us)
+            port[name] = {"MT": round(q.giga_mt, 2), "unit": "GB/s", "threads": q.threads_mt, "iters_MT": q.iters_mt,
+                          "sample": f"{what}; three arrays of {n_stream * 4 >> 20} MiB, per-thread contiguous chunks"}
         reference = None
         if ref is not None:
-            n_stream, llc = _stream_floats(cores)
             rd = pool.measure_read_fn(ref["read_fn"], ref["populate_fn"], n_stream, 2, target_us)
             ch = pool.measure_chain_fn(ref["fp32_fn"], ref["fp32_ops"], 2, extra_target_us)
             reference = {"isa": ref["isa"],

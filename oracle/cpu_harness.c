@@ -501,6 +501,98 @@ int cpuh_measure_read_fn(cpuh_pool *p, cpuh_read_fn fn, cpuh_populate_fn populat
     return 0;
 }
 
+/* The reference's buffer fill, restated (src/common/common.cpp:76-95): xorshift32 from 0xDEADBEEF per
+ * call, bits forced to a finite positive float.  Every chunk a thread fills starts the sequence again. */
+void cpuh_populate(float *p, unsigned long long n)
+{
+    uint32_t state = 0xDEADBEEFu;
+    for (unsigned long long i = 0; i < n; i++) {
+        state ^= state << 13;
+        state ^= state >> 17;
+        state ^= state << 5;
+        const uint32_t bits = (state & 0x7F7FFFFFu) | 0x00800000u;
+        memcpy(&p[i], &bits, sizeof(float));
+    }
+}
+
+/* The other two rows of the reference's DRAM test (src/cpu/bandwidth.cpp:323-352): three arrays of
+ * n_floats, first-touched in parallel, every thread working on its own contiguous chunk.
+ *   copy  (kind 0): memcpy(A + lo, C + lo, chunk), 2 * n_floats * 4 bytes per iteration;
+ *   triad (kind 1): A[i] = B[i] + 1.5f * C[i],      3 * n_floats * 4 bytes per iteration.
+ * Timed at every worker only, as the reference does (ST fields of the result stay 0 / -1). */
+typedef struct {
+    float *a, *b, *c;
+    uint64_t n_floats;
+    int n_threads, kind;
+    cpuh_populate_fn populate;
+} stream_workload;
+
+static void stream_chunk(const stream_workload *w, int tid, uint64_t *lo, uint64_t *hi)
+{
+    const uint64_t per = w->n_floats / (uint64_t)w->n_threads;
+    *lo = (uint64_t)tid * per;
+    *hi = tid == w->n_threads - 1 ? w->n_floats : *lo + per;
+}
+
+static void body_stream_touch(void *c, int tid, uint64_t iters)
+{
+    stream_workload *w = (stream_workload *)c;
+    (void)iters;
+    uint64_t lo, hi;
+    stream_chunk(w, tid, &lo, &hi);
+    w->populate(w->a + lo, hi - lo);
+    w->populate(w->b + lo, hi - lo);
+    w->populate(w->c + lo, hi - lo);
+}
+
+static void body_stream(void *c, int tid, uint64_t iters)
+{
+    stream_workload *w = (stream_workload *)c;
+    uint64_t lo, hi;
+    stream_chunk(w, tid, &lo, &hi);
+    if (w->kind == 0) {
+        for (uint64_t it = 0; it < iters; it++) {
+            memcpy(w->a + lo, w->c + lo, (size_t)(hi - lo) * sizeof(float));
+            __asm__ volatile("" ::: "memory");   /* every pass is done */
+        }
+    } else {
+        const float s = 1.5f;
+        float *restrict a = w->a;
+        const float *restrict b = w->b, *restrict cc = w->c;
+        for (uint64_t it = 0; it < iters; it++) {
+            for (uint64_t i = lo; i < hi; i++) a[i] = b[i] + s * cc[i];
+            __asm__ volatile("" ::: "memory");
+        }
+    }
+}
+
+int cpuh_measure_stream(cpuh_pool *p, cpuh_populate_fn populate, uint64_t n_floats, int kind, unsigned warmup,
+                        unsigned target_us, cpuh_result *r, float *probe_out)
+{
+    if (!populate || !r || n_floats == 0 || (kind != 0 && kind != 1)) return -1;
+    const int n = p->n_max > MAX_T ? MAX_T : p->n_max;
+    stream_workload w;
+    memset(&w, 0, sizeof(w));
+    w.n_floats = n_floats;
+    w.n_threads = n;
+    w.kind = kind;
+    w.populate = populate;
+    w.a = (float *)aligned_alloc(64, (n_floats * sizeof(float) + 63) / 64 * 64);
+    w.b = (float *)aligned_alloc(64, (n_floats * sizeof(float) + 63) / 64 * 64);
+    w.c = (float *)aligned_alloc(64, (n_floats * sizeof(float) + 63) / 64 * 64);
+    if (!w.a || !w.b || !w.c) { free(w.a); free(w.b); free(w.c); return -3; }
+    cpuh_pool_run(p, n, body_stream_touch, &w, 1);
+    memset(r, 0, sizeof(*r));
+    r->us_mt = cpuh_run_workload(p, n, body_stream, &w, warmup, target_us, 0, &r->iters_mt);
+    const double bytes = (kind == 0 ? 2.0 : 3.0) * (double)n_floats * 4.0;
+    finish(p, r, n, bytes, bytes / (double)n);
+    /* a few results, so that a test can check what the pass computed */
+    if (probe_out) { probe_out[0] = w.a[0]; probe_out[1] = w.a[n_floats / 2]; probe_out[2] = w.a[n_floats - 1];
+                     probe_out[3] = w.b[n_floats / 2]; probe_out[4] = w.c[n_floats / 2]; }
+    free(w.a); free(w.b); free(w.c);
+    return 0;
+}
+
 /* Test hook: a body that sleeps `ctx` microseconds per iteration, so the discipline can be checked
  * against a known per-iteration time. */
 static void body_sleep(void *c, int tid, uint64_t iters)

@@ -272,6 +272,7 @@ def _bind_harness():
     L.cpuh_measure.argtypes = [vp, i32, u64, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure.restype = i32
     L.cpuh_measure_chain_fn.argtypes = [vp, vp, dbl, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure_chain_fn.restype = i32
     L.cpuh_measure_read_fn.argtypes = [vp, vp, vp, u64, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure_read_fn.restype = i32
+    L.cpuh_measure_stream.argtypes = [vp, vp, u64, i32, u32, u32, C.POINTER(CpuhResult), vp]; L.cpuh_measure_stream.restype = i32
     L._harness_bound = True
     return L
 
@@ -333,6 +334,21 @@ class CpuPool:
         if rc != 0:
             raise RuntimeError(f"cpuh_measure_read_fn failed: {rc}")
         return r
+
+
+    def own_populate_ptr(self):
+        """Address of the harness's restatement of the reference's populate()."""
+        return C.cast(self.L.cpuh_populate, C.c_void_p).value
+
+    def measure_stream(self, populate_ptr, n_floats, kind, warmup=2, target_us=2_000_000):
+        """The reference's DRAM `copy` (kind 0) / `triad` (kind 1) rows over three shared arrays, all workers.
+        Returns (result, probe) with probe = a[0], a[n/2], a[n-1], b[n/2], c[n/2] after the run."""
+        r = CpuhResult()
+        probe = np.zeros(5, dtype=np.float32)
+        rc = self.L.cpuh_measure_stream(self.h, populate_ptr, n_floats, kind, warmup, target_us, C.byref(r), probe.ctypes.data)
+        if rc != 0:
+            raise RuntimeError(f"cpuh_measure_stream failed: {rc}")
+        return r, probe
 
 
 REF_LIB_PATH = os.path.join(_HERE, "_ref", "libclpeak_ref.so")

@@ -128,3 +128,44 @@ def test_reference_kernels_run_under_the_harness(pool):
     rd = pool.measure_read_fn(ref["read_fn"], ref["populate_fn"], 1 << 24, warmup=1, target_us=50_000)
     assert 1.0 < rd.giga_st < 200.0 and rd.giga_mt > 0.8 * rd.giga_st
     assert rd.units_per_iter_st == (1 << 24) // pool.max_threads * pool.max_threads * 4.0
+
+
+def test_populate_restated_against_the_first_values_and_its_mask():
+    """xorshift32 from 0xDEADBEEF (src/common/common.cpp:76-95): the first states computed here by hand in
+    Python; the mask clears the sign and sets the lowest exponent bit, so every value is positive and normal
+    or, one time in 128, has an all-ones exponent (the reference's comment calls them all finite; they are not)."""
+    import ctypes as C
+    L = orc.lib()
+    n = 1000
+    buf = np.zeros(n, dtype=np.float32)
+    L.cpuh_populate.argtypes = [C.c_void_p, C.c_ulonglong]; L.cpuh_populate.restype = None
+    L.cpuh_populate(buf.ctypes.data, n)
+    state, want = 0xDEADBEEF, []
+    for _ in range(n):
+        state ^= (state << 13) & 0xFFFFFFFF
+        state ^= state >> 17
+        state ^= (state << 5) & 0xFFFFFFFF
+        want.append((state & 0x7F7FFFFF) | 0x00800000)
+    assert [int(x) for x in buf.view(np.uint32)] == want
+    bits = buf.view(np.uint32)
+    assert np.all(bits >> 31 == 0) and np.all((bits >> 23) & 1 == 1)
+    assert 0 < np.count_nonzero(~np.isfinite(buf)) < n // 32
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+def test_stream_copy_and_triad_rows(kind):
+    """copy: A = C; triad: A = B + 1.5 C (src/cpu/bandwidth.cpp:323-352).  All three arrays hold the same
+    populate() sequence per chunk, so after any number of passes A[i] is C[i] or B[i] + 1.5 C[i] = 2.5 C[i];
+    bytes per pass are 2 N x 4 and 3 N x 4."""
+    n = 1 << 20
+    with orc.CpuPool(4) as pool:
+        r, probe = pool.measure_stream(pool.own_populate_ptr(), n, kind, 1, 20_000)
+    a_mid, b_mid, c_mid = probe[1], probe[3], probe[4]
+    assert b_mid.view(np.uint32) == c_mid.view(np.uint32) and np.isfinite(c_mid) and c_mid > 0
+    with np.errstate(over="ignore"):
+        want = c_mid if kind == 0 else np.float32(np.float32(1.5) * c_mid) + b_mid
+    assert a_mid.view(np.uint32) == np.float32(want).view(np.uint32)
+    assert r.iters_mt >= 1 and r.us_mt > 0 and r.threads_mt == 4
+    assert r.units_per_iter_st == (2 if kind == 0 else 3) * n * 4
+    assert abs(r.giga_mt - r.units_per_iter_st / (r.us_mt * 1e3)) <= 1e-6 * r.giga_mt
+    assert r.giga_st == -1.0 and r.iters_st == 0          # all workers only, as the reference times these rows

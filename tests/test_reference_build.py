@@ -92,3 +92,16 @@ def test_cancel_flag_behaves_alike(ref, host):
         assert getattr(lib, get)() == 1
         getattr(lib, reset)()
         assert getattr(lib, get)() == 0
+
+
+def test_restated_populate_is_the_reference_s(ref):
+    """The harness's buffer fill against the reference's compiled populate() (src/common/common.cpp:76-95),
+    bit for bit, over a length that is not a multiple of anything."""
+    n = 100_003
+    ref.ref_populate.argtypes = [C.c_void_p, C.c_ulonglong]; ref.ref_populate.restype = None
+    L = orc.lib()
+    L.cpuh_populate.argtypes = [C.c_void_p, C.c_ulonglong]; L.cpuh_populate.restype = None
+    a, b = np.zeros(n, dtype=np.float32), np.zeros(n, dtype=np.float32)
+    ref.ref_populate(a.ctypes.data, n)
+    L.cpuh_populate(b.ctypes.data, n)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
