@@ -66,9 +66,11 @@ def bench_rows(dev, quick, only):
         us = dev.launch_roundtrip(2, 10000)
         add("kernel_launch_latency", "roundtrip", us, "us", us)
     if "mfma" in only or "smfmac" in only:
-        _matrix_rows(dev, wl, add, budget, only, zero=False)
+        _matrix_rows(dev, wl, add, budget, only, zero=False, one_set=True)
+    if "matrix_distinct" in only:
+        _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=False, one_set=False)
     if "matrix_zero" in only:
-        _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=True)
+        _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=True, one_set=True)
     if "gemm" in only:
         _gemm_rows(dev, capi, wl, add, budget, constant=False)
     if "gemm_const" in only:
@@ -126,13 +128,18 @@ def _mad_rows(dev, capi, add, budget):
     out.free()
 
 
-def _matrix_rows(dev, wl, add, budget, only, zero):
+def _matrix_rows(dev, wl, add, budget, only, zero, one_set):
     # --- dense MFMA / SMFMAC: 2048 waves x 4 chains x 4096 iterations ------------------------
+    # one_set: the four accumulator chains of a wave share one A and one B fragment, held in the same
+    # registers, as the reference's kernels do (src/rocm/rocm_kernels/mfma_bf16.hip:16-30); that is the
+    # workload's "per wave: A/B fragments ... 4 independent accumulator chains" and what the rows report.
+    # Not one_set ("distinct operands per chain"): every chain has fragments of its own, in registers of
+    # its own; same arithmetic, more register reads, a lower clock.
     # zero: the same launches on all-zero operands.  Nothing toggles in the multipliers, the part holds
     # its boost clock, and the row shows the issue rate of the loop itself (the seeded rows show what the
     # part sustains under the power that random operands draw).
     waves, iters = 2048, 4096
-    tail = " zero operands" if zero else ""
+    tail = " zero operands" if zero else ("" if one_set else " distinct operands per chain")
     clk = dev.alloc(16)
     peaks = {0: "f16", 1: "bf16", 2: "f16", 3: "bf16", 4: "int8", 5: "fp8", 6: "fp8", 7: "fp6", 8: "fp6", 9: "fp4"}
     for kind in sorted(wl.DENSE) if "mfma" in only else []:
@@ -143,7 +150,7 @@ def _matrix_rows(dev, wl, add, budget, only, zero):
         bufs = [dev.from_host(A), dev.from_host(B), dev.from_host(sA) if sA is not None else None,
                 dev.from_host(sB) if sB is not None else None]
         o = dev.alloc(waves * 4 * s["M"] * s["N"] * 4)
-        us, _ = timed(dev, lambda: dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], o, waves, iters, clk), **budget)
+        us, _ = timed(dev, lambda: dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], o, waves, iters, clk, one_set=one_set), **budget)
         c = clk.download(np.uint64, 2)
         unit = "tops" if s["fmt"] == wl.I8 else "tflops"
         add(s["name"], s["name"] + tail, wl.dense_flops(kind, waves, iters) / us / 1e6, unit, us, PEAK[peaks[kind]],
@@ -159,7 +166,7 @@ def _matrix_rows(dev, wl, add, budget, only, zero):
             Ac, B = np.zeros_like(Ac), np.zeros_like(B)
         bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
         o = dev.alloc(waves * 4 * 256 * 4)
-        us, _ = timed(dev, lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk), **budget)
+        us, _ = timed(dev, lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk, one_set=one_set), **budget)
         c = clk.download(np.uint64, 2)
         unit = "tops" if s["fmt"] == wl.I8 else "tflops"
         add(s["name"], s["name"] + tail, wl.sparse_flops(kind, waves, iters) / us / 1e6, unit, us, 2 * PEAK[speaks[kind]],
@@ -338,8 +345,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel over 1 GiB (20 launches): under rocprofv3 --pmc this "
                          "gives what FETCH_SIZE / WRITE_SIZE read for a transfer of known size")
-    ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_zero,gemm,gemm_const,lds,transfer",
-                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_zero,gemm,gemm_const,lds,transfer")
+    ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,gemm,gemm_const,lds,transfer",
+                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,gemm,gemm_const,lds,transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; the hot path has no multi-GPU step "

@@ -112,7 +112,9 @@ enum { kBf16 = 0, kF16 = 1, kI8 = 2, kScaledBf16 = 3 };   // kScaledBf16: output
                : "+v"(acc[7][0]), "+v"(acc[7][1]), "+v"(acc[7][2]), "+v"(acc[7][3]), "+v"(acc[6][3]) :: "memory")
 
 // One step of K: 64 MFMAs per wave, 32 on fragment set F0 (first K half of the slab) then 32 on
-// F1.  The order written here is the order issued; never more than one memory instruction between
+// F1, each set walked row by row in alternating directions ((0,0)..(0,3),(1,3)..(1,0),(2,0)..) so that
+// every instruction shares one source register set with the one before it: re-reading the registers the
+// last instruction read costs less power than reading others, and power is what bounds this kernel.  The order written here is the order issued; never more than one memory instruction between
 // two MFMAs, because a ds_read_b128 (about 11 cycles of issue) slips into the 16-cycle shadow of
 // the MFMA before it, while two in a row would stall the matrix pipe.
 // `first` (wave-uniform): the first step of a tile, whose barrier needs no wait for loads (the end of
@@ -137,11 +139,11 @@ __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8]
   MM(x0, 0, 1); MI355_DS_READ(fb1[2], b1, 4096); MI355_DS_READ(fb1[3], b1, 6144);
   MM(x0, 0, 2); MI355_DS_READ(fa1[0], a1, 0); MI355_DS_READ(fa1[1], a1, 2048);
   MM(x0, 0, 3); MI355_DS_READ(fa1[2], a1, 4096); MI355_DS_READ(fa1[3], a1, 6144);
-  MM(x0, 1, 0); MI355_DS_READ(fa1[4], a1, 8192); MI355_DS_READ(fa1[5], a1, 10240);
-  MM(x0, 1, 1); MI355_DS_READ(fa1[6], a1, 12288); MI355_DS_READ(fa1[7], a1, 14336);
-  MM(x0, 1, 2); MM(x0, 1, 3);
+  MM(x0, 1, 3); MI355_DS_READ(fa1[4], a1, 8192); MI355_DS_READ(fa1[5], a1, 10240);
+  MM(x0, 1, 2); MI355_DS_READ(fa1[6], a1, 12288); MI355_DS_READ(fa1[7], a1, 14336);
+  MM(x0, 1, 1); MM(x0, 1, 0);
   MM(x0, 2, 0); MM(x0, 2, 1); MM(x0, 2, 2); MM(x0, 2, 3);
-  MM(x0, 3, 0);
+  MM(x0, 3, 3);
   MI355_WAIT_FRAGS(fa1, fb1);
   // Every wave holds all fragments of this step's slab: its two slots are free.  Loads return in
   // order, so with the 4 A loads of the last step (for the slab three steps ahead) still allowed in
@@ -151,57 +153,57 @@ __device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8]
   // ---- MFMAs 13..63: B rows of the slab two steps ahead into the freed A slot, then A rows of the slab
   //      three steps ahead into the freed B slot, one load every sixth MFMA so that the fill path sees a
   //      steady stream; from MFMA 40 on (F0 is dead since MFMA 31) the next step's F0 reads ------------
-  MM(x0, 3, 1);
-  MM(x0, 3, 2); LDB(0);
-  MM(x0, 3, 3);
+  MM(x0, 3, 2);
+  MM(x0, 3, 1); LDB(0);
+  MM(x0, 3, 0);
   MM(x0, 4, 0);
   MM(x0, 4, 1);
   MM(x0, 4, 2);
   MM(x0, 4, 3);
-  MM(x0, 5, 0); LDB(1);
-  MM(x0, 5, 1);
+  MM(x0, 5, 3); LDB(1);
   MM(x0, 5, 2);
-  MM(x0, 5, 3);
+  MM(x0, 5, 1);
+  MM(x0, 5, 0);
   MM(x0, 6, 0);
   MM(x0, 6, 1);
   MM(x0, 6, 2); LDB(2);
   MM(x0, 6, 3);
-  MM(x0, 7, 0);
-  MM(x0, 7, 1);
-  MM(x0, 7, 2);
   MM(x0, 7, 3);
+  MM(x0, 7, 2);
+  MM(x0, 7, 1);
+  MM(x0, 7, 0);
   MM(x1, 0, 0); LDB(3);
   MM(x1, 0, 1);
   MM(x1, 0, 2);
   MM(x1, 0, 3);
-  MM(x1, 1, 0);
-  MM(x1, 1, 1);
-  MM(x1, 1, 2); LDA(0);
   MM(x1, 1, 3);
+  MM(x1, 1, 2);
+  MM(x1, 1, 1); LDA(0);
+  MM(x1, 1, 0);
   MM(x1, 2, 0); if (READS) MI355_DS_READ(fb0[0], w.b_nxt, 0);
   MM(x1, 2, 1); if (READS) MI355_DS_READ(fb0[1], w.b_nxt, 2048);
   MM(x1, 2, 2); if (READS) MI355_DS_READ(fb0[2], w.b_nxt, 4096);
   MM(x1, 2, 3); if (READS) MI355_DS_READ(fb0[3], w.b_nxt, 6144);
-  MM(x1, 3, 0); LDA(1);
-  MM(x1, 3, 1); if (READS) MI355_DS_READ(fa0[0], w.a_nxt, 0);
-  MM(x1, 3, 2); if (READS) MI355_DS_READ(fa0[1], w.a_nxt, 2048);
-  MM(x1, 3, 3); if (READS) MI355_DS_READ(fa0[2], w.a_nxt, 4096);
+  MM(x1, 3, 3); LDA(1);
+  MM(x1, 3, 2); if (READS) MI355_DS_READ(fa0[0], w.a_nxt, 0);
+  MM(x1, 3, 1); if (READS) MI355_DS_READ(fa0[1], w.a_nxt, 2048);
+  MM(x1, 3, 0); if (READS) MI355_DS_READ(fa0[2], w.a_nxt, 4096);
   MM(x1, 4, 0); if (READS) MI355_DS_READ(fa0[3], w.a_nxt, 6144);
   MM(x1, 4, 1); if (READS) MI355_DS_READ(fa0[4], w.a_nxt, 8192);
   MM(x1, 4, 2); LDA(2);
   MM(x1, 4, 3); if (READS) MI355_DS_READ(fa0[5], w.a_nxt, 10240);
-  MM(x1, 5, 0); if (READS) MI355_DS_READ(fa0[6], w.a_nxt, 12288);
-  MM(x1, 5, 1); if (READS) MI355_DS_READ(fa0[7], w.a_nxt, 14336);
-  MM(x1, 5, 2);
-  MM(x1, 5, 3);
+  MM(x1, 5, 3); if (READS) MI355_DS_READ(fa0[6], w.a_nxt, 12288);
+  MM(x1, 5, 2); if (READS) MI355_DS_READ(fa0[7], w.a_nxt, 14336);
+  MM(x1, 5, 1);
+  MM(x1, 5, 0);
   MM(x1, 6, 0); LDA(3);
   MM(x1, 6, 1);
   MM(x1, 6, 2);
   MM(x1, 6, 3);
-  MM(x1, 7, 0);
-  MM(x1, 7, 1);
-  MM(x1, 7, 2);
   MM(x1, 7, 3);
+  MM(x1, 7, 2);
+  MM(x1, 7, 1);
+  MM(x1, 7, 0);
   MI355_WAIT_FRAGS(fa0, fb0);
 #undef LDA
 #undef LDB

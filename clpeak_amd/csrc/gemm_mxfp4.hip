@@ -90,7 +90,8 @@ struct MxFrags {
   i32x4v sa_n, sb_n;                     // scale bytes being loaded for the next step
 };
 
-// One step of K: 128 instructions per wave, 64 on the first K half then 64 on the second.
+// One step of K: 128 instructions per wave, 64 on the first K half then 64 on the second, each half walked
+// row by row in alternating directions so that consecutive instructions share one operand's registers.
 // FIRST: the first step of a tile.  Its first K half starts the accumulators from zero, and it takes no
 // counted wait for loads: every outstanding load that matters was waited for at the end of the tile before,
 // and the stores issued since must not be counted.
@@ -123,14 +124,14 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   MM(0, 0, 5, 1, 0); MI355_DS_READ(fb1[5], b1, 10240);
   MM(0, 0, 6, 0, 0); MI355_DS_READ(fb1[6], b1, 12288);
   MM(0, 0, 7, 1, 0); MI355_DS_READ(fb1[7], b1, 14336);
-  MM(0, 1, 0, 0, 1); MI355_DS_READ(fa1[0], a1, 0);
-  MM(0, 1, 1, 1, 1); MI355_DS_READ(fa1[1], a1, 2048);
-  MM(0, 1, 2, 0, 1); MI355_DS_READ(fa1[2], a1, 4096);
-  MM(0, 1, 3, 1, 1); MI355_DS_READ(fa1[3], a1, 6144);
-  MM(0, 1, 4, 0, 1); MI355_DS_READ(fa1[4], a1, 8192);
-  MM(0, 1, 5, 1, 1); MI355_DS_READ(fa1[5], a1, 10240);
-  MM(0, 1, 6, 0, 1); MI355_DS_READ(fa1[6], a1, 12288);
-  MM(0, 1, 7, 1, 1); MI355_DS_READ(fa1[7], a1, 14336);
+  MM(0, 1, 7, 1, 1); MI355_DS_READ(fa1[0], a1, 0);
+  MM(0, 1, 6, 0, 1); MI355_DS_READ(fa1[1], a1, 2048);
+  MM(0, 1, 5, 1, 1); MI355_DS_READ(fa1[2], a1, 4096);
+  MM(0, 1, 4, 0, 1); MI355_DS_READ(fa1[3], a1, 6144);
+  MM(0, 1, 3, 1, 1); MI355_DS_READ(fa1[4], a1, 8192);
+  MM(0, 1, 2, 0, 1); MI355_DS_READ(fa1[5], a1, 10240);
+  MM(0, 1, 1, 1, 1); MI355_DS_READ(fa1[6], a1, 12288);
+  MM(0, 1, 0, 0, 1); MI355_DS_READ(fa1[7], a1, 14336);
   MM(0, 2, 0, 0, 0);
   MM(0, 2, 1, 1, 0);
   MM(0, 2, 2, 0, 0);
@@ -144,14 +145,14 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   // rows three steps ahead, may still be in flight: this wave's B rows of the next slab have landed
   if (FIRST) asm volatile("s_barrier" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(8)\n s_barrier" ::: "memory");
-  MM(0, 3, 0, 0, 1); SCL_B();
-  MM(0, 3, 1, 1, 1); SCL_A();
-  MM(0, 3, 2, 0, 1);
-  MM(0, 3, 3, 1, 1);
-  MM(0, 3, 4, 0, 1);
+  MM(0, 3, 7, 1, 1); SCL_B();
+  MM(0, 3, 6, 0, 1); SCL_A();
   MM(0, 3, 5, 1, 1);
-  MM(0, 3, 6, 0, 1);
-  MM(0, 3, 7, 1, 1);
+  MM(0, 3, 4, 0, 1);
+  MM(0, 3, 3, 1, 1);
+  MM(0, 3, 2, 0, 1);
+  MM(0, 3, 1, 1, 1);
+  MM(0, 3, 0, 0, 1);
   MM(0, 4, 0, 0, 0);
   MM(0, 4, 1, 1, 0);
   MM(0, 4, 2, 0, 0);
@@ -160,14 +161,14 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   MM(0, 4, 5, 1, 0);
   MM(0, 4, 6, 0, 0);
   MM(0, 4, 7, 1, 0);
-  MM(0, 5, 0, 0, 1);
-  MM(0, 5, 1, 1, 1);
-  MM(0, 5, 2, 0, 1);
-  MM(0, 5, 3, 1, 1);
-  MM(0, 5, 4, 0, 1);
-  MM(0, 5, 5, 1, 1);
-  MM(0, 5, 6, 0, 1);
   MM(0, 5, 7, 1, 1);
+  MM(0, 5, 6, 0, 1);
+  MM(0, 5, 5, 1, 1);
+  MM(0, 5, 4, 0, 1);
+  MM(0, 5, 3, 1, 1);
+  MM(0, 5, 2, 0, 1);
+  MM(0, 5, 1, 1, 1);
+  MM(0, 5, 0, 0, 1);
   MM(0, 6, 0, 0, 0);
   MM(0, 6, 1, 1, 0);
   MM(0, 6, 2, 0, 0);
@@ -176,14 +177,14 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   MM(0, 6, 5, 1, 0);
   MM(0, 6, 6, 0, 0);
   MM(0, 6, 7, 1, 0);
-  MM(0, 7, 0, 0, 1); LDB(0);
-  MM(0, 7, 1, 1, 1);
-  MM(0, 7, 2, 0, 1);
-  MM(0, 7, 3, 1, 1);
-  MM(0, 7, 4, 0, 1); LDB(1);
-  MM(0, 7, 5, 1, 1);
+  MM(0, 7, 7, 1, 1); LDB(0);
   MM(0, 7, 6, 0, 1);
-  MM(0, 7, 7, 1, 1);
+  MM(0, 7, 5, 1, 1);
+  MM(0, 7, 4, 0, 1);
+  MM(0, 7, 3, 1, 1); LDB(1);
+  MM(0, 7, 2, 0, 1);
+  MM(0, 7, 1, 1, 1);
+  MM(0, 7, 0, 0, 1);
   MM(1, 0, 0, 0, 0); LDB(2);
   MM(1, 0, 1, 1, 0); MI355_DS_READ(fb0[0], w.b_nxt, 0);
   MM(1, 0, 2, 0, 0);
@@ -192,14 +193,14 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   MM(1, 0, 5, 1, 0); MI355_DS_READ(fb0[2], w.b_nxt, 4096);
   MM(1, 0, 6, 0, 0);
   MM(1, 0, 7, 1, 0); MI355_DS_READ(fb0[3], w.b_nxt, 6144);
-  MM(1, 1, 0, 0, 1); LDB(4);
-  MM(1, 1, 1, 1, 1); MI355_DS_READ(fb0[4], w.b_nxt, 8192);
-  MM(1, 1, 2, 0, 1);
-  MM(1, 1, 3, 1, 1); MI355_DS_READ(fb0[5], w.b_nxt, 10240);
-  MM(1, 1, 4, 0, 1); LDB(5);
-  MM(1, 1, 5, 1, 1); MI355_DS_READ(fb0[6], w.b_nxt, 12288);
-  MM(1, 1, 6, 0, 1);
-  MM(1, 1, 7, 1, 1); MI355_DS_READ(fb0[7], w.b_nxt, 14336);
+  MM(1, 1, 7, 1, 1); LDB(4);
+  MM(1, 1, 6, 0, 1); MI355_DS_READ(fb0[4], w.b_nxt, 8192);
+  MM(1, 1, 5, 1, 1);
+  MM(1, 1, 4, 0, 1); MI355_DS_READ(fb0[5], w.b_nxt, 10240);
+  MM(1, 1, 3, 1, 1); LDB(5);
+  MM(1, 1, 2, 0, 1); MI355_DS_READ(fb0[6], w.b_nxt, 12288);
+  MM(1, 1, 1, 1, 1);
+  MM(1, 1, 0, 0, 1); MI355_DS_READ(fb0[7], w.b_nxt, 14336);
   MM(1, 2, 0, 0, 0); LDB(6);
   MM(1, 2, 1, 1, 0); MI355_DS_READ(fa0[0], w.a_nxt, 0);
   MM(1, 2, 2, 0, 0);
@@ -208,14 +209,14 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   MM(1, 2, 5, 1, 0); MI355_DS_READ(fa0[2], w.a_nxt, 4096);
   MM(1, 2, 6, 0, 0);
   MM(1, 2, 7, 1, 0); MI355_DS_READ(fa0[3], w.a_nxt, 6144);
-  MM(1, 3, 0, 0, 1); LDA(0);
-  MM(1, 3, 1, 1, 1); MI355_DS_READ(fa0[4], w.a_nxt, 8192);
-  MM(1, 3, 2, 0, 1);
-  MM(1, 3, 3, 1, 1); MI355_DS_READ(fa0[5], w.a_nxt, 10240);
-  MM(1, 3, 4, 0, 1); LDA(1);
-  MM(1, 3, 5, 1, 1); MI355_DS_READ(fa0[6], w.a_nxt, 12288);
-  MM(1, 3, 6, 0, 1);
-  MM(1, 3, 7, 1, 1); MI355_DS_READ(fa0[7], w.a_nxt, 14336);
+  MM(1, 3, 7, 1, 1); LDA(0);
+  MM(1, 3, 6, 0, 1); MI355_DS_READ(fa0[4], w.a_nxt, 8192);
+  MM(1, 3, 5, 1, 1);
+  MM(1, 3, 4, 0, 1); MI355_DS_READ(fa0[5], w.a_nxt, 10240);
+  MM(1, 3, 3, 1, 1); LDA(1);
+  MM(1, 3, 2, 0, 1); MI355_DS_READ(fa0[6], w.a_nxt, 12288);
+  MM(1, 3, 1, 1, 1);
+  MM(1, 3, 0, 0, 1); MI355_DS_READ(fa0[7], w.a_nxt, 14336);
   MM(1, 4, 0, 0, 0); LDA(2);
   MM(1, 4, 1, 1, 0);
   MM(1, 4, 2, 0, 0);
@@ -224,14 +225,14 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   MM(1, 4, 5, 1, 0);
   MM(1, 4, 6, 0, 0);
   MM(1, 4, 7, 1, 0);
-  MM(1, 5, 0, 0, 1); LDA(4);
-  MM(1, 5, 1, 1, 1);
-  MM(1, 5, 2, 0, 1);
-  MM(1, 5, 3, 1, 1);
-  MM(1, 5, 4, 0, 1); LDA(5);
-  MM(1, 5, 5, 1, 1);
+  MM(1, 5, 7, 1, 1); LDA(4);
   MM(1, 5, 6, 0, 1);
-  MM(1, 5, 7, 1, 1);
+  MM(1, 5, 5, 1, 1);
+  MM(1, 5, 4, 0, 1);
+  MM(1, 5, 3, 1, 1); LDA(5);
+  MM(1, 5, 2, 0, 1);
+  MM(1, 5, 1, 1, 1);
+  MM(1, 5, 0, 0, 1);
   MM(1, 6, 0, 0, 0); LDA(6);
   MM(1, 6, 1, 1, 0);
   MM(1, 6, 2, 0, 0);
@@ -240,14 +241,14 @@ __device__ __forceinline__ void mx_step(f32x4v (&acc)[8][8], MxFrags &f, const M
   MM(1, 6, 5, 1, 0);
   MM(1, 6, 6, 0, 0);
   MM(1, 6, 7, 1, 0);
-  MM(1, 7, 0, 0, 1);
-  MM(1, 7, 1, 1, 1);
-  MM(1, 7, 2, 0, 1);
-  MM(1, 7, 3, 1, 1);
-  MM(1, 7, 4, 0, 1);
-  MM(1, 7, 5, 1, 1);
-  MM(1, 7, 6, 0, 1);
   MM(1, 7, 7, 1, 1);
+  MM(1, 7, 6, 0, 1);
+  MM(1, 7, 5, 1, 1);
+  MM(1, 7, 4, 0, 1);
+  MM(1, 7, 3, 1, 1);
+  MM(1, 7, 2, 0, 1);
+  MM(1, 7, 1, 1, 1);
+  MM(1, 7, 0, 0, 1);
   MI355_WAIT_FRAGS16(fa0, fb0);
 #undef MM
 #undef LDA

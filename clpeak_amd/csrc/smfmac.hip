@@ -5,7 +5,8 @@
 // `iters` times, final tiles written row-major.  A arrives compressed (the two kept
 // values of every group of four along K) with one metadata byte per group; each lane
 // packs the metadata of its own K range into the index register once, before the loop.
-// Work is counted with the dense-equivalent K.
+// Work is counted with the dense-equivalent K.  MI355_MFMA_ONE_OPERAND_SET: the four chains take
+// chain 0's A, B and index registers, as the reference's kernels do (src/rocm/rocm_kernels/smfmac_fp16.hip:22-40).
 #include "internal.h"
 #include "mfma_common.h"
 
@@ -51,7 +52,7 @@ MI355_SPARSE_TRAIT(SP_FP8, 128, 1, i32x4v, i32x8v, f32x4v, float, "v_smfmac_f32_
 MI355_SPARSE_TRAIT(SP_BF8, 128, 1, i32x4v, i32x8v, f32x4v, float, "v_smfmac_f32_16x16x128_bf8_bf8")
 MI355_SPARSE_TRAIT(SP_I8, 128, 1, i32x4v, i32x8v, i32x4v, int32_t, "v_smfmac_i32_16x16x128_i8")
 
-template <typename Tr>
+template <typename Tr, bool ONE_SET>
 __global__ void __launch_bounds__(256)
 smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, const uint8_t *__restrict__ B,
               typename Tr::Out *__restrict__ out, uint32_t iters, uint64_t *__restrict__ clocks) {
@@ -67,6 +68,12 @@ smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, 
   int idx[kChains];
 #pragma unroll
   for (int c = 0; c < kChains; c++) {
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc[c][r] = 0;
+    if (ONE_SET && c > 0) {   // the very registers of chain 0
+      a[c] = a[0]; b[c] = b[0]; idx[c] = idx[0];
+      continue;
+    }
     const uint64_t u = wave * kChains + c;
     a[c] = load_bytes<typename Tr::FragA>(Ac + u * 16 * ac_row + (lane % 16) * ac_row + (lane / 16) * (ac_row / 4));
     {  // B: 16 bytes of the first K half and 16 bytes of the second (b_row is 128 for every kind)
@@ -80,8 +87,6 @@ smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, 
 #pragma unroll
     for (int g = 0; g < groups; g++) packed |= (uint32_t)(m[g] & 0xf) << (4 * g);
     idx[c] = (int)packed;
-#pragma unroll
-    for (int r = 0; r < 4; r++) acc[c][r] = 0;
   }
 
   const uint32_t blocks = iters / kBlock, rest = iters % kBlock;
@@ -106,10 +111,14 @@ smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, 
 }
 
 template <typename Tr>
-int launch(mi355_dev *dev, const void *Ac, const uint8_t *meta, const void *B, void *out, uint32_t waves,
+int launch(mi355_dev *dev, bool one_set, const void *Ac, const uint8_t *meta, const void *B, void *out, uint32_t waves,
            uint32_t iters, uint64_t *clocks) {
-  smfmac_kernel<Tr><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)Ac, meta, (const uint8_t *)B,
-                                                       (typename Tr::Out *)out, iters, clocks);
+  if (one_set)
+    smfmac_kernel<Tr, true><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)Ac, meta, (const uint8_t *)B,
+                                                               (typename Tr::Out *)out, iters, clocks);
+  else
+    smfmac_kernel<Tr, false><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)Ac, meta, (const uint8_t *)B,
+                                                                (typename Tr::Out *)out, iters, clocks);
   MI355_LAUNCH_CHECK(dev, "smfmac");
   return MI355_OK;
 }
@@ -122,12 +131,14 @@ extern "C" int mi355_smfmac(mi355_dev *dev, int kind, const void *Ac, const uint
   MI355_REQUIRE(dev, Ac && meta && B && out, "smfmac: null buffer");
   MI355_REQUIRE(dev, waves > 0 && waves % 4 == 0, "smfmac: waves (%u) must be a positive multiple of 4", waves);
   MI355_REQUIRE(dev, (((uintptr_t)Ac | (uintptr_t)B | (uintptr_t)out) & 15u) == 0, "smfmac: buffers must be 16-byte aligned");
+  const bool one_set = (kind & MI355_MFMA_ONE_OPERAND_SET) != 0;
+  kind &= ~MI355_MFMA_ONE_OPERAND_SET;
   switch (kind) {
-    case MI355_SMFMAC_F16_16x16x64:  return launch<SP_F16>(dev, Ac, meta, B, out, waves, iters, clocks);
-    case MI355_SMFMAC_BF16_16x16x64: return launch<SP_BF16>(dev, Ac, meta, B, out, waves, iters, clocks);
-    case MI355_SMFMAC_FP8_16x16x128: return launch<SP_FP8>(dev, Ac, meta, B, out, waves, iters, clocks);
-    case MI355_SMFMAC_BF8_16x16x128: return launch<SP_BF8>(dev, Ac, meta, B, out, waves, iters, clocks);
-    case MI355_SMFMAC_I8_16x16x128:  return launch<SP_I8>(dev, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_F16_16x16x64:  return launch<SP_F16>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_BF16_16x16x64: return launch<SP_BF16>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_FP8_16x16x128: return launch<SP_FP8>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_BF8_16x16x128: return launch<SP_BF8>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_I8_16x16x128:  return launch<SP_I8>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
     default: return mi355_fail(dev, MI355_ERR_ARG, "smfmac: unknown kind %d", kind);
   }
 }

@@ -336,7 +336,7 @@ void Mi355Peak::runMfma(Category phase) {
     }
     const float us = runKernel(
         [&] {
-          return api_.mfma_dense(dev_, m.kind, dA.ptr, dB.ptr, m.scaled ? (const uint8_t *)sA.ptr : nullptr,
+          return api_.mfma_dense(dev_, m.kind | MI355_MFMA_ONE_OPERAND_SET, dA.ptr, dB.ptr, m.scaled ? (const uint8_t *)sA.ptr : nullptr,
                                  m.scaled ? (const uint8_t *)sB.ptr : nullptr, out.ptr, waves, workload.mfmaIters, nullptr);
         },
         targetTimeUs, forceIters ? specifiedIters : 0);
@@ -368,7 +368,7 @@ void Mi355Peak::runSparseMfma(Category phase) {
       continue;
     }
     const float us = runKernel(
-        [&] { return api_.smfmac(dev_, m.kind, dA.ptr, (const uint8_t *)dM.ptr, dB.ptr, out.ptr, waves, workload.mfmaIters, nullptr); },
+        [&] { return api_.smfmac(dev_, m.kind | MI355_MFMA_ONE_OPERAND_SET, dA.ptr, (const uint8_t *)dM.ptr, dB.ptr, out.ptr, waves, workload.mfmaIters, nullptr); },
         targetTimeUs, forceIters ? specifiedIters : 0);
     if (us <= 0.0f) {
       test.skip(m.tag, ResultStatus::Error, "kernel launch failed");

@@ -198,6 +198,11 @@ int mi355_launch_roundtrip(mi355_dev *dev, uint32_t warmup, uint32_t launches, d
 #define MI355_MFMA_MXFP6_E3M2       8
 #define MI355_MFMA_MXFP4_E2M1       9
 #define MI355_MFMA_KIND_COUNT      10
+/* OR into `kind` (here and for mi355_smfmac): every chain of a wave takes the operands (A, B, scales /
+ * index) of its chain 0, from the same registers, as the reference's kernels use one a and one b for all
+ * their accumulator chains (src/rocm/rocm_kernels/mfma_bf16.hip:16-30).  The slots of chains 1..3 in
+ * the operand arrays are then not read; all four output tiles of a wave are equal. */
+#define MI355_MFMA_ONE_OPERAND_SET 0x100
 int mi355_mfma_dense(mi355_dev *dev, int kind, const void *A, const void *B,
                      const uint8_t *scaleA, const uint8_t *scaleB,
                      void *out, uint32_t waves, uint32_t iters, uint64_t *clocks);

@@ -25,7 +25,16 @@ SEED = wl.DEFAULT_SEED
 DOT_TOL = 4e-5   # relative to sum|a_k * b_k|, one instruction
 
 
-def _run_dense(dev, kind, waves, iters, seed=SEED):
+def _chain0_everywhere(x, waves):
+    """What the kernel computes on with MFMA_ONE_OPERAND_SET: every chain of a wave holds chain 0's operand."""
+    if x is None:
+        return None
+    y = np.ascontiguousarray(x).reshape(waves, 4, -1).copy()
+    y[:, 1:, :] = y[:, :1, :]
+    return y.reshape(x.shape)
+
+
+def _run_dense(dev, kind, waves, iters, seed=SEED, one_set=False):
     s = wl.DENSE[kind]
     A, B, sA, sB = wl.dense_inputs(kind, waves, seed)
     dA, dB = dev.from_host(A), dev.from_host(B)
@@ -33,9 +42,11 @@ def _run_dense(dev, kind, waves, iters, seed=SEED):
     dsB = dev.from_host(sB) if sB is not None else None
     n_out = waves * 4 * s["M"] * s["N"]
     out = dev.alloc(n_out * 4)
-    dev.mfma_dense(kind, dA, dB, dsA, dsB, out, waves, iters)
+    dev.mfma_dense(kind, dA, dB, dsA, dsB, out, waves, iters, one_set=one_set)
     is_int = s["fmt"] is None
     got = out.download(np.int32 if is_int else np.float32, n_out)
+    if one_set:   # the device was handed the full arrays; the oracle gets what the flag makes of them
+        A, B, sA, sB = (_chain0_everywhere(x, waves) for x in (A, B, sA, sB))
     ref, ab = orc.mfma_dense(kind, A, B, sA, sB, waves, iters, s["M"] * s["N"], is_int=is_int)
     for b in (dA, dB, dsA, dsB, out):
         if b is not None:
@@ -62,10 +73,23 @@ def test_mfma_dense_parity(dev, kind, iters):
 
 
 @pytest.mark.parametrize("kind", sorted(wl.DENSE))
-def test_mfma_dense_full_launch_sampled(dev, kind):
+@pytest.mark.parametrize("iters", [1, 13, 4096])
+def test_mfma_dense_parity_one_operand_set(dev, kind, iters):
+    """The launch the benchmark rows use: the four chains of a wave take chain 0's fragments from the same
+    registers (one a and one b for all accumulator chains, as in the reference's kernels).  The four tiles of
+    a wave must then be equal among themselves as well as right."""
+    got, ref, ab, is_int = _run_dense(dev, kind, 8, iters, one_set=True)
+    _check(got, ref, ab, is_int, (wl.DENSE[kind]["name"], iters), iters)
+    tiles = got.reshape(8, 4, -1)
+    assert all(np.array_equal(tiles[:, 0], tiles[:, c]) for c in (1, 2, 3))
+
+
+@pytest.mark.parametrize("one_set", [False, True])
+@pytest.mark.parametrize("kind", sorted(wl.DENSE))
+def test_mfma_dense_full_launch_sampled(dev, kind, one_set):
     """The configured launch: 2048 waves x 4 chains x 4096 iterations.  The oracle replays
     every wave (seconds) and the whole output is compared."""
-    got, ref, ab, is_int = _run_dense(dev, kind, 2048, 4096)
+    got, ref, ab, is_int = _run_dense(dev, kind, 2048, 4096, one_set=one_set)
     _check(got, ref, ab, is_int, wl.DENSE[kind]["name"], 4096)
 
 
@@ -76,15 +100,17 @@ def test_mfma_int8_linearity(dev):
     assert np.array_equal(gn.astype(np.int64), g1.astype(np.int64) * 4096)
 
 
-def _run_sparse(dev, kind, waves, iters, seed=SEED):
+def _run_sparse(dev, kind, waves, iters, seed=SEED, one_set=False):
     s = wl.SPARSE[kind]
     Ac, meta, B = wl.sparse_inputs(kind, waves, seed)
     dA, dM, dB = dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)
     n_out = waves * 4 * 256
     out = dev.alloc(n_out * 4)
-    dev.smfmac(kind, dA, dM, dB, out, waves, iters)
+    dev.smfmac(kind, dA, dM, dB, out, waves, iters, one_set=one_set)
     is_int = s["fmt"] is None
     got = out.download(np.int32 if is_int else np.float32, n_out)
+    if one_set:
+        Ac, meta, B = (_chain0_everywhere(x, waves) for x in (Ac, meta, B))
     ref, ab = orc.smfmac(kind, Ac, meta, B, waves, iters, is_int=is_int)
     for b in (dA, dM, dB, out):
         b.free()
@@ -99,6 +125,16 @@ def test_smfmac_parity(dev, kind, iters):
 
 
 @pytest.mark.parametrize("kind", sorted(wl.SPARSE))
-def test_smfmac_full_launch(dev, kind):
-    got, ref, ab, is_int = _run_sparse(dev, kind, 2048, 4096)
+@pytest.mark.parametrize("iters", [1, 13, 4096])
+def test_smfmac_parity_one_operand_set(dev, kind, iters):
+    got, ref, ab, is_int = _run_sparse(dev, kind, 8, iters, one_set=True)
+    _check(got, ref, ab, is_int, (wl.SPARSE[kind]["name"], iters), iters)
+    tiles = got.reshape(8, 4, -1)
+    assert all(np.array_equal(tiles[:, 0], tiles[:, c]) for c in (1, 2, 3))
+
+
+@pytest.mark.parametrize("one_set", [False, True])
+@pytest.mark.parametrize("kind", sorted(wl.SPARSE))
+def test_smfmac_full_launch(dev, kind, one_set):
+    got, ref, ab, is_int = _run_sparse(dev, kind, 2048, 4096, one_set=one_set)
     _check(got, ref, ab, is_int, wl.SPARSE[kind]["name"], 4096)
