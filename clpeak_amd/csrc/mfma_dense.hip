@@ -5,7 +5,7 @@
 // of its 4 chains from the logical A/B matrices once, then issues
 //     acc[c] = MFMA(a[c], b[c], acc[c])        c = 0..3, `iters` times
 // so that 4 independent accumulator tiles are always in flight and a dependent
-// MFMA never waits for its predecessor.  With MI355_MFMA_ONE_OPERAND_SET the four chains
+// MFMA ever waits on a result it cannot have yet.  With MI355_MFMA_ONE_OPERAND_SET the four chains
 // take the fragments of chain 0, from the SAME registers, as the reference's kernels do with
 // their one a and one b (src/rocm/rocm_kernels/mfma_bf16.hip:16-30): an instruction whose
 // sources are the registers its predecessor read costs the part less power than one that reads
@@ -21,40 +21,48 @@ constexpr int kChains = 4;
 
 // The hot loop is written as inline assembly: with the builtins the register
 // allocator rotates the accumulator tiles through copies on every trip, and each
-// copy next to an MFMA costs wait states.  One block = kBlock rounds over the 4
-// chains, accumulating in place (vDst == SrcC), which the matrix pipe executes
-// back to back with no software wait states: the next MFMA that touches the same
-// accumulator is 3 independent MFMAs away.  A block is 128 instructions because the
-// loop branch costs the issuing wave about 20 cycles in which the pipe idles (waves of
-// one SIMD run one after the other here: the oldest always has an MFMA ready and wins
-// arbitration), 4 % at 32 instructions per trip and 1 % at 128.
+// copy next to an MFMA costs wait states.  One block = kBlock iterations of every chain,
+// accumulating in place (vDst == SrcC), ONE CHAIN AFTER THE OTHER: 32 instructions on
+// accumulator 0, then 32 on accumulator 1, and so on.  The matrix pipe forwards an
+// accumulator to the next instruction that names it, so a run of dependent instructions
+// issues back to back exactly like independent ones (97 % pipe utilisation either way), and
+// an instruction that names the registers its predecessor named costs the part less power
+// than one that switches: with the chains interleaved one instruction at a time the same
+// seeded launch holds 1.96 GHz (bf16, 1.95 PFLOP/s), in runs of 2 / 4 / 8 / 16 / 32 it holds
+// 2.14 / 2.26 / 2.29 / 2.33 / 2.33-2.36 GHz (2.17 / 2.29 / 2.35 / 2.39 / 2.42 PFLOP/s).
+// Every chain still performs its `iters` dependent instructions in order, so results do
+// not depend on the run length.  A block is 128 instructions because the loop branch costs
+// the issuing wave about 20 cycles in which the pipe idles (waves of one SIMD run one after
+// the other here: the oldest always has an MFMA ready and wins arbitration), 4 % at 32
+// instructions per trip and 1 % at 128.
 constexpr int kBlock = 32;
 
 #define MI355_REP8(x) x x x x x x x x
 #define MI355_REP32(x) MI355_REP8(x) MI355_REP8(x) MI355_REP8(x) MI355_REP8(x)
 // %0-%3 accumulators, %4-%7 A fragments, %8-%11 B fragments
-#define MI355_ROUND(INSN, TAIL)                \
-  INSN " %0, %4, %8, %0" TAIL "\n"             \
-  INSN " %1, %5, %9, %1" TAIL "\n"             \
-  INSN " %2, %6, %10, %2" TAIL "\n"            \
-  INSN " %3, %7, %11, %3" TAIL "\n"
+#define MI355_CHAINS(REP, INSN, TAIL)          \
+  REP(INSN " %0, %4, %8, %0" TAIL "\n")        \
+  REP(INSN " %1, %5, %9, %1" TAIL "\n")        \
+  REP(INSN " %2, %6, %10, %2" TAIL "\n")       \
+  REP(INSN " %3, %7, %11, %3" TAIL "\n")
 // scaled: %12-%15 scale A, %16-%19 scale B
-#define MI355_ROUND_SCALED(INSN, TAIL)                   \
-  INSN " %0, %4, %8, %0, %12, %16 op_sel_hi:[0,0,0]" TAIL "\n"   \
-  INSN " %1, %5, %9, %1, %13, %17 op_sel_hi:[0,0,0]" TAIL "\n"   \
-  INSN " %2, %6, %10, %2, %14, %18 op_sel_hi:[0,0,0]" TAIL "\n"  \
-  INSN " %3, %7, %11, %3, %15, %19 op_sel_hi:[0,0,0]" TAIL "\n"
+#define MI355_CHAINS_SCALED(REP, INSN, TAIL)                       \
+  REP(INSN " %0, %4, %8, %0, %12, %16 op_sel_hi:[0,0,0]" TAIL "\n")   \
+  REP(INSN " %1, %5, %9, %1, %13, %17 op_sel_hi:[0,0,0]" TAIL "\n")   \
+  REP(INSN " %2, %6, %10, %2, %14, %18 op_sel_hi:[0,0,0]" TAIL "\n")  \
+  REP(INSN " %3, %7, %11, %3, %15, %19 op_sel_hi:[0,0,0]" TAIL "\n")
+#define MI355_ONCE(x) x
 
 #define MI355_DEFINE_STEPS(INSN, TAIL)                                                             \
   __device__ static void block(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&)[4], \
                                const int (&)[4]) {                                                 \
-    asm volatile(MI355_REP32(MI355_ROUND(INSN, TAIL))                                               \
+    asm volatile(MI355_CHAINS(MI355_REP32, INSN, TAIL)                                              \
                  : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
                  : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3])); \
   }                                                                                                \
   __device__ static void single(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&)[4], \
                                 const int (&)[4]) {                                                \
-    asm volatile(MI355_ROUND(INSN, TAIL)                                                           \
+    asm volatile(MI355_CHAINS(MI355_ONCE, INSN, TAIL)                                              \
                  : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
                  : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3])); \
   }
@@ -62,14 +70,14 @@ constexpr int kBlock = 32;
 #define MI355_DEFINE_STEPS_SCALED(INSN, TAIL)                                                      \
   __device__ static void block(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&sa)[4], \
                                const int (&sb)[4]) {                                               \
-    asm volatile(MI355_REP32(MI355_ROUND_SCALED(INSN, TAIL))                                        \
+    asm volatile(MI355_CHAINS_SCALED(MI355_REP32, INSN, TAIL)                                       \
                  : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
                  : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), \
                    "v"(sa[0]), "v"(sa[1]), "v"(sa[2]), "v"(sa[3]), "v"(sb[0]), "v"(sb[1]), "v"(sb[2]), "v"(sb[3])); \
   }                                                                                                \
   __device__ static void single(Acc (&acc)[4], const Frag (&a)[4], const Frag (&b)[4], const int (&sa)[4], \
                                 const int (&sb)[4]) {                                              \
-    asm volatile(MI355_ROUND_SCALED(INSN, TAIL)                                                    \
+    asm volatile(MI355_CHAINS_SCALED(MI355_ONCE, INSN, TAIL)                                       \
                  : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])                          \
                  : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), \
                    "v"(sa[0]), "v"(sa[1]), "v"(sa[2]), "v"(sa[3]), "v"(sb[0]), "v"(sb[1]), "v"(sb[2]), "v"(sb[3])); \
