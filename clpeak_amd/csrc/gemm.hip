@@ -28,17 +28,14 @@
 // one bank group 16 times.  The direct-to-LDS load writes lane i at position i of its
 // 1 KiB destination, so lane i fetches the global chunk that belongs there.
 //
-// Schedule of one bf16 step: 64 MFMAs per wave, 32 on fragment set F0 (first K half of the
-// slab) then 32 on F1 (second half):
-//     MFMA  0..12   the 12 LDS reads of F1, two in each of the first 6 gaps (a 128-bit read takes
-//                   about 8 cycles to issue, two fit in the 16-cycle shadow of an MFMA)
-//     wait F1; wait own loads but the 4 youngest; barrier   <- slab s+1 complete, slab s free
-//     MFMA 13..63   the wave's 8 global->LDS loads, one every sixth MFMA; from MFMA 40 on the
-//                   12 LDS reads of the next step's F0, one per gap
-// One barrier per step, placed as early as the F1 reads allow.
-// The loop body is inline assembly so that this order is the order issued;
-// the compiler knows neither the LDS reads nor the MFMAs and therefore inserts no wait
-// states of its own: every s_waitcnt below is part of the schedule.
+// Schedule of one step (gemm_ring_step): 32 slots per wave, one per 16x16 tile of its 128x64, each slot 32
+// cycles of the matrix pipe: one K=128 fp8 instruction, or two K=32 (bf16, f16) / K=64 (int8) instructions on
+// the two K halves of the slab, back to back on the same accumulator.  There are no registers for a second
+// set of fragments (128 accumulators + 96 fragment registers), so fragments are reloaded in place as soon as
+// their last use has issued, with counted waits so that a row starts as soon as its own fragment has arrived;
+// one barrier per step, placed as early as the fragment reads allow.  The loop body is inline assembly so
+// that this order is the order issued; the compiler knows neither the LDS reads nor the MFMAs and therefore
+// inserts no wait states of its own: every s_waitcnt below is part of the schedule.
 //
 // The MFMA is issued with the B fragment as the first operand, which produces the
 // transposed 16x16 tile: a lane then holds 4 consecutive N elements of one C row (see store_tile for
@@ -82,18 +79,8 @@ using Ring = GemmRing<2, 4>;
                : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fa[4]), "+v"(fa[5]),     \
                  "+v"(fa[6]), "+v"(fa[7]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]))
 
-// acc(transposed tile) += B_frag . A_frag^T
-#define MI355_MFMA_BF16(acc, fb, fa) \
-  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(fb), "v"(fa))
-#define MI355_MFMA_F16(acc, fb, fa) \
-  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(fb), "v"(fa))
-// int8: 16 bytes per lane are K=16 of the 64, the accumulator registers hold int32
-#define MI355_MFMA_I8(acc, fb, fa) \
-  asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc) : "v"(fb), "v"(fa))
-
-// Operand types of the kernel that walks a slab as two K halves (16 bytes per lane and half):
-// bf16 and f16 (K=32 per instruction, fp32 accumulate) and int8 (K=64, int32 accumulate).
-enum { kBf16 = 0, kF16 = 1, kI8 = 2, kScaledBf16 = 3 };   // kScaledBf16: output type of the fp8 kernels only
+// Output types of store_tile: bf16, f16, int32 (bits as they are), bf16 after a scale (the fp8 kinds).
+enum { kBf16 = 0, kF16 = 1, kI8 = 2, kScaledBf16 = 3 };
 
 // The barrier of a step: every wave holds all fragments of the step's slab (its two slots are free)
 // and, loads returning in order, with its 4 youngest loads (the A rows three slabs ahead) still
@@ -110,105 +97,6 @@ enum { kBf16 = 0, kF16 = 1, kI8 = 2, kScaledBf16 = 3 };   // kScaledBf16: output
 #define MI355_END_OF_TILE(acc)                                                                     \
   asm volatile("s_nop 15\n s_nop 15\n s_waitcnt vmcnt(4)"                                          \
                : "+v"(acc[7][0]), "+v"(acc[7][1]), "+v"(acc[7][2]), "+v"(acc[7][3]), "+v"(acc[6][3]) :: "memory")
-
-// One step of K: 64 MFMAs per wave, 32 on fragment set F0 (first K half of the slab) then 32 on
-// F1, each set walked row by row in alternating directions ((0,0)..(0,3),(1,3)..(1,0),(2,0)..) so that
-// every instruction shares one source register set with the one before it: re-reading the registers the
-// last instruction read costs less power than reading others, and power is what bounds this kernel.  The order written here is the order issued; never more than one memory instruction between
-// two MFMAs, because a ds_read_b128 (about 11 cycles of issue) slips into the 16-cycle shadow of
-// the MFMA before it, while two in a row would stall the matrix pipe.
-// `first` (wave-uniform): the first step of a tile, whose barrier needs no wait for loads (the end of
-// the tile before did it, ahead of the stores that are now in the queue).  A step always prefetches:
-// the last step of a tile reads the first fragments of the next tile, which the ring already holds.
-template <int KIND>
-__device__ __forceinline__ void gemm_step(f32x4v (&acc)[8][4], bf16x8v (&fa0)[8], bf16x8v (&fb0)[4],
-                                          bf16x8v (&fa1)[8], bf16x8v (&fb1)[4], const GemmWalk &w, uint32_t first) {
-  constexpr bool READS = true;
-  const uint32_t a1 = w.a_cur ^ 64u, b1 = w.b_cur ^ 64u;   // second K half of this step
-#define MM(F, i, j)                                                                                \
-  do {                                                                                             \
-    if (KIND == kBf16) MI355_MFMA_BF16(acc[i][j], F##b##_[j], F##a##_[i]);                         \
-    else if (KIND == kF16) MI355_MFMA_F16(acc[i][j], F##b##_[j], F##a##_[i]);                      \
-    else MI355_MFMA_I8(acc[i][j], F##b##_[j], F##a##_[i]);                                         \
-  } while (0)
-#define LDA(q) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
-#define LDB(q) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
-  bf16x8v(&x0a_)[8] = fa0; bf16x8v(&x0b_)[4] = fb0; bf16x8v(&x1a_)[8] = fa1; bf16x8v(&x1b_)[4] = fb1;
-  // ---- MFMAs 0..12 (on F0); the 12 reads of F1 in the first 6 gaps ------------------------------
-  MM(x0, 0, 0); MI355_DS_READ(fb1[0], b1, 0); MI355_DS_READ(fb1[1], b1, 2048);
-  MM(x0, 0, 1); MI355_DS_READ(fb1[2], b1, 4096); MI355_DS_READ(fb1[3], b1, 6144);
-  MM(x0, 0, 2); MI355_DS_READ(fa1[0], a1, 0); MI355_DS_READ(fa1[1], a1, 2048);
-  MM(x0, 0, 3); MI355_DS_READ(fa1[2], a1, 4096); MI355_DS_READ(fa1[3], a1, 6144);
-  MM(x0, 1, 3); MI355_DS_READ(fa1[4], a1, 8192); MI355_DS_READ(fa1[5], a1, 10240);
-  MM(x0, 1, 2); MI355_DS_READ(fa1[6], a1, 12288); MI355_DS_READ(fa1[7], a1, 14336);
-  MM(x0, 1, 1); MM(x0, 1, 0);
-  MM(x0, 2, 0); MM(x0, 2, 1); MM(x0, 2, 2); MM(x0, 2, 3);
-  MM(x0, 3, 3);
-  MI355_WAIT_FRAGS(fa1, fb1);
-  // Every wave holds all fragments of this step's slab: its two slots are free.  Loads return in
-  // order, so with the 4 A loads of the last step (for the slab three steps ahead) still allowed in
-  // flight, this wave's B rows of the next slab and its A rows of the next slab (older still) have
-  // landed.
-  MI355_STEP_BARRIER(first, "");
-  // ---- MFMAs 13..63: B rows of the slab two steps ahead into the freed A slot, then A rows of the slab
-  //      three steps ahead into the freed B slot, one load every sixth MFMA so that the fill path sees a
-  //      steady stream; from MFMA 40 on (F0 is dead since MFMA 31) the next step's F0 reads ------------
-  MM(x0, 3, 2);
-  MM(x0, 3, 1); LDB(0);
-  MM(x0, 3, 0);
-  MM(x0, 4, 0);
-  MM(x0, 4, 1);
-  MM(x0, 4, 2);
-  MM(x0, 4, 3);
-  MM(x0, 5, 3); LDB(1);
-  MM(x0, 5, 2);
-  MM(x0, 5, 1);
-  MM(x0, 5, 0);
-  MM(x0, 6, 0);
-  MM(x0, 6, 1);
-  MM(x0, 6, 2); LDB(2);
-  MM(x0, 6, 3);
-  MM(x0, 7, 3);
-  MM(x0, 7, 2);
-  MM(x0, 7, 1);
-  MM(x0, 7, 0);
-  MM(x1, 0, 0); LDB(3);
-  MM(x1, 0, 1);
-  MM(x1, 0, 2);
-  MM(x1, 0, 3);
-  MM(x1, 1, 3);
-  MM(x1, 1, 2);
-  MM(x1, 1, 1); LDA(0);
-  MM(x1, 1, 0);
-  MM(x1, 2, 0); if (READS) MI355_DS_READ(fb0[0], w.b_nxt, 0);
-  MM(x1, 2, 1); if (READS) MI355_DS_READ(fb0[1], w.b_nxt, 2048);
-  MM(x1, 2, 2); if (READS) MI355_DS_READ(fb0[2], w.b_nxt, 4096);
-  MM(x1, 2, 3); if (READS) MI355_DS_READ(fb0[3], w.b_nxt, 6144);
-  MM(x1, 3, 3); LDA(1);
-  MM(x1, 3, 2); if (READS) MI355_DS_READ(fa0[0], w.a_nxt, 0);
-  MM(x1, 3, 1); if (READS) MI355_DS_READ(fa0[1], w.a_nxt, 2048);
-  MM(x1, 3, 0); if (READS) MI355_DS_READ(fa0[2], w.a_nxt, 4096);
-  MM(x1, 4, 0); if (READS) MI355_DS_READ(fa0[3], w.a_nxt, 6144);
-  MM(x1, 4, 1); if (READS) MI355_DS_READ(fa0[4], w.a_nxt, 8192);
-  MM(x1, 4, 2); LDA(2);
-  MM(x1, 4, 3); if (READS) MI355_DS_READ(fa0[5], w.a_nxt, 10240);
-  MM(x1, 5, 3); if (READS) MI355_DS_READ(fa0[6], w.a_nxt, 12288);
-  MM(x1, 5, 2); if (READS) MI355_DS_READ(fa0[7], w.a_nxt, 14336);
-  MM(x1, 5, 1);
-  MM(x1, 5, 0);
-  MM(x1, 6, 0); LDA(3);
-  MM(x1, 6, 1);
-  MM(x1, 6, 2);
-  MM(x1, 6, 3);
-  MM(x1, 7, 3);
-  MM(x1, 7, 2);
-  MM(x1, 7, 1);
-  MM(x1, 7, 0);
-  MI355_WAIT_FRAGS(fa0, fb0);
-#undef LDA
-#undef LDB
-#undef MM
-}
 
 // Store a wave's 128x64 accumulators.  A lane holds 4 consecutive N elements of one row per 16x16 tile
 // (8 bytes of bf16 / f16, 16 bytes of int32), lane group g = lane/16 the 4 elements 4g..4g+3.  Stored as
@@ -257,13 +145,120 @@ __device__ __forceinline__ void store_tile(const f32x4v (&acc)[8][4], void *__re
     }
 }
 
-template <int KIND>
+// ---- the step of the 8-bit and 16-bit kinds ------------------------------------------------------------
+// A slab of 128 bytes per row is one K=128 fp8 instruction per 16x16 tile, or two instructions of the
+// 16-bit / int8 kinds.  A lane's operand bytes are the two 16-byte chunks g and g+4 of its row (g = lane/16),
+// which in the swizzled layout are the addresses x and x^64: two ds_read_b128 fill the low and the high half
+// (the 8-register fp8 operand, or the operands of the first and of the second instruction of a pair).
+//
+// Fragments are reloaded in place as soon as their last use has issued.  The 32 slots run as two sweeps over
+// the 8 A fragments, first against B fragments 0,1 and then against 2,3:
+//     MFMA  0..9    (i,0),(i,1): this step's A fragment 7 and B fragments 2,3 are read in gaps 0..2;
+//                   counted waits let row i start as soon as its own fragment has arrived
+//     wait all reads; wait own loads but the 4 youngest; barrier   <- slab s+1 complete, slab s free
+//     MFMA 10..15   the wave's 4 loads of B rows (slab s+2)
+//     MFMA 16..31   (i,2),(i,3): next step's B fragments 0,1 in gaps 16,17, next step's A fragment
+//                   i-1 after row i (a fragment is overwritten no sooner than one instruction after
+//                   its last use); the wave's 4 loads of A rows (slab s+3) in the even gaps 18..24
+// What one (i, j) slot of the step issues on a lane's two 16-byte halves (first and second K half of the slab):
+//   fp8: one K=128 instruction on the 32-byte operands (e5m2 A: format field blgp, the A fragment being the
+//        second source of the transposed product);
+//   bf16 / f16 / int8: two instructions, first half then second, BACK TO BACK ON THE SAME ACCUMULATOR.  The
+//        matrix pipe forwards the accumulator to the next instruction that names it, so the pair issues like
+//        two independent instructions, and an instruction that names its predecessor's accumulator costs less
+//        power than one that switches (see mfma_dense.hip), which is what bounds these kernels.
+enum { kOpE4m3 = 0, kOpE5m2 = 1, kOpBf16 = 2, kOpF16 = 3, kOpI8 = 4 };
+#define MI355_MFMA_SLOT(OP, acc, blo, bhi, alo, ahi)                                               \
+  do {                                                                                             \
+    if (OP == kOpE4m3 || OP == kOpE5m2) {                                                          \
+      const i32x8v b8_ = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7);                \
+      const i32x8v a8_ = __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);                \
+      if (OP == kOpE5m2)                                                                           \
+        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 blgp:1" : "+v"(acc) : "v"(b8_), "v"(a8_));       \
+      else                                                                                         \
+        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(acc) : "v"(b8_), "v"(a8_)); \
+    } else if (OP == kOpBf16) {                                                                    \
+      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n v_mfma_f32_16x16x32_bf16 %0, %3, %4, %0" \
+                   : "+v"(acc) : "v"(blo), "v"(alo), "v"(bhi), "v"(ahi));                          \
+    } else if (OP == kOpF16) {                                                                     \
+      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n v_mfma_f32_16x16x32_f16 %0, %3, %4, %0" \
+                   : "+v"(acc) : "v"(blo), "v"(alo), "v"(bhi), "v"(ahi));                          \
+    } else {                                                                                       \
+      asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0\n v_mfma_i32_16x16x64_i8 %0, %3, %4, %0"   \
+                   : "+v"(acc) : "v"(blo), "v"(alo), "v"(bhi), "v"(ahi));                          \
+    }                                                                                              \
+  } while (0)
+
+// At most `n` LDS reads still outstanding (they return in order).
+#define MI355_WAIT_LGKM(n) asm volatile("s_waitcnt lgkmcnt(" #n ")" ::: "memory")
+
+struct RingFrags {
+  i32x4v a_lo[8], a_hi[8], b_lo[4], b_hi[4];
+};
+
+template <int OP>
+__device__ __forceinline__ void gemm_ring_step(f32x4v (&acc)[8][4], RingFrags &f, const GemmWalk &w, uint32_t first) {
+  constexpr bool READS = true;
+  const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u, an_hi = w.a_nxt ^ 64u, bn_hi = w.b_nxt ^ 64u;
+#define MM(i, j) MI355_MFMA_SLOT(OP, acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i])
+#define LDA(q) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
+#define LDB(q) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
+#define RD_A_NEXT(i, off)                                                                          \
+  if (READS) { MI355_DS_READ(f.a_lo[i], w.a_nxt, off); MI355_DS_READ(f.a_hi[i], an_hi, off); }
+#define RD_B_NEXT(j, off)                                                                          \
+  if (READS) { MI355_DS_READ(f.b_lo[j], w.b_nxt, off); MI355_DS_READ(f.b_hi[j], bn_hi, off); }
+  // On entry the reads of B fragments 0,1 and A fragments 0..6 of this step are in flight, in that order.
+  MI355_WAIT_LGKM(12);                                   // B0, B1, A0 have arrived
+  MM(0, 0); MI355_DS_READ(f.a_lo[7], w.a_cur, 14336); MI355_DS_READ(f.a_hi[7], a_hi, 14336);
+  MM(0, 1); MI355_DS_READ(f.b_lo[2], w.b_cur, 4096); MI355_DS_READ(f.b_hi[2], b_hi, 4096);
+  MI355_WAIT_LGKM(14);                                   // A1
+  MM(1, 0); MI355_DS_READ(f.b_lo[3], w.b_cur, 6144); MI355_DS_READ(f.b_hi[3], b_hi, 6144);
+  MM(1, 1);
+  MI355_WAIT_LGKM(14);                                   // A2
+  MM(2, 0); MM(2, 1);
+  MI355_WAIT_LGKM(12);                                   // A3
+  MM(3, 0); MM(3, 1);
+  MI355_WAIT_LGKM(10);                                   // A4
+  MM(4, 0); MM(4, 1);
+  // every read of this step's slab has returned (its two slots are free); with the 4 A loads of the
+  // last step still allowed in flight, this wave's share of the next slab has landed
+  MI355_STEP_BARRIER(first, "s_waitcnt lgkmcnt(0)\n");
+  MM(5, 0); LDB(0);
+  MM(5, 1);
+  MM(6, 0); LDB(1);
+  MM(6, 1);
+  MM(7, 0); LDB(2);
+  MM(7, 1); LDB(3);
+  MM(0, 2); RD_B_NEXT(0, 0);
+  MM(0, 3); RD_B_NEXT(1, 2048);
+  MM(1, 2); LDA(0);
+  MM(1, 3); RD_A_NEXT(0, 0);
+  MM(2, 2); LDA(1);
+  MM(2, 3); RD_A_NEXT(1, 2048);
+  MM(3, 2); LDA(2);
+  MM(3, 3); RD_A_NEXT(2, 4096);
+  MM(4, 2); LDA(3);
+  MM(4, 3); RD_A_NEXT(3, 6144);
+  MM(5, 2);
+  MM(5, 3); RD_A_NEXT(4, 8192);
+  MM(6, 2);
+  MM(6, 3); RD_A_NEXT(5, 10240);
+  MM(7, 2);
+  MM(7, 3); RD_A_NEXT(6, 12288);
+#undef RD_A_NEXT
+#undef RD_B_NEXT
+#undef LDA
+#undef LDB
+#undef MM
+}
+
+template <int OP>
 __global__ void __launch_bounds__(kThreads)
-gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, void *__restrict__ Cout,
-                 uint32_t N, uint32_t k_bytes, uint32_t tiles_m, uint32_t tiles_n) {
+gemm_ring_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, void *__restrict__ C,
+                uint32_t N, uint32_t k_bytes, float scale, uint32_t tiles_m, uint32_t tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const uint32_t tid = threadIdx.x, lane = tid % 64;
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);   // wave-uniform, and known to be
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const uint32_t wm = wave / 4, wn = wave % 4;
   const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
 
@@ -276,21 +271,34 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
   for (int i = 0; i < 8; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
-  bf16x8v fa0[8], fb0[4], fa1[8], fb1[4];
-  MI355_READ_FRAGS(fa0, fb0, ring.w.a_cur, ring.w.b_cur);
-  MI355_WAIT_FRAGS(fa0, fb0);
+  RingFrags f;
+  // what a step expects in flight on entry: B fragments 0,1 then A fragments 0..6
+  {
+    const GemmWalk &w = ring.w;
+    const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u;
+    MI355_DS_READ(f.b_lo[0], w.b_cur, 0); MI355_DS_READ(f.b_hi[0], b_hi, 0);
+    MI355_DS_READ(f.b_lo[1], w.b_cur, 2048); MI355_DS_READ(f.b_hi[1], b_hi, 2048);
+    MI355_DS_READ(f.a_lo[0], w.a_cur, 0); MI355_DS_READ(f.a_hi[0], a_hi, 0);
+    MI355_DS_READ(f.a_lo[1], w.a_cur, 2048); MI355_DS_READ(f.a_hi[1], a_hi, 2048);
+    MI355_DS_READ(f.a_lo[2], w.a_cur, 4096); MI355_DS_READ(f.a_hi[2], a_hi, 4096);
+    MI355_DS_READ(f.a_lo[3], w.a_cur, 6144); MI355_DS_READ(f.a_hi[3], a_hi, 6144);
+    MI355_DS_READ(f.a_lo[4], w.a_cur, 8192); MI355_DS_READ(f.a_hi[4], a_hi, 8192);
+    MI355_DS_READ(f.a_lo[5], w.a_cur, 10240); MI355_DS_READ(f.a_hi[5], a_hi, 10240);
+    MI355_DS_READ(f.a_lo[6], w.a_cur, 12288); MI355_DS_READ(f.a_hi[6], a_hi, 12288);
+  }
 
   // one loop over the steps of all tiles of the workgroup
   uint32_t round = 0, left = steps, first = 1;
   for (uint32_t g = grid.mine * steps; g > 0; g--) {
-    gemm_step<KIND>(acc, fa0, fb0, fa1, fb1, ring.w, first);
+    gemm_ring_step<OP>(acc, f, ring.w, first);
     ring.advance();
     first = 0;
     if (--left == 0) {
       MI355_END_OF_TILE(acc);
       uint32_t tm, tn;
       tile_at(grid, round, tm, tn);
-      store_tile<KIND>(acc, Cout, N, tm * kTile + wm * 128u + lane % 16u, tn * kTile + wn * 64u, lane, 1.0f);
+      store_tile<(OP == kOpBf16 ? kBf16 : OP == kOpF16 ? kF16 : OP == kOpI8 ? kI8 : kScaledBf16)>(
+          acc, C, N, tm * kTile + wm * 128u + lane % 16u, tn * kTile + wn * 64u, lane, scale);
 #pragma unroll
       for (int i = 0; i < 8; i++)
 #pragma unroll
@@ -304,7 +312,8 @@ gemm_bf16_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
 }
 
 // ---- fp32 ----------------------------------------------------------------------------------------
-// Same tiling, ring, loads and LDS layout; a 128-byte row segment is 32 floats.  The fp32 matrix
+// Same tiling, ring, loads and LDS layout, but two fragment sets (one per K half); a 128-byte row segment is
+// 32 floats.  The fp32 matrix
 // instruction is 16x16x4 with ONE float per lane and operand (row lane%16, k = lane/16).  A lane's
 // 16-byte fragment read is chunk lane/16 of its row, i.e. floats 4*(lane/16) .. +3; register t of it,
 // used as the operand of the t-th of four instructions, makes lane group g supply k = 4g + t: the four
@@ -399,158 +408,6 @@ gemm_f32_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, fl
   MI355_DRAIN_RING();
 }
 
-// ---- fp8 e4m3 ------------------------------------------------------------------------------------
-// Same tiling, LDS layout, loads and barrier discipline as above; a slab of 128 bytes per row is
-// exactly one K=128 matrix instruction per 16x16 tile, 32 instructions of 32 cycles per wave and step.
-// A lane's 32-byte operand is the two 16-byte chunks g and g+4 of its row (g = lane/16), which in
-// the swizzled layout are the addresses x and x^64: two ds_read_b128 fill the low and the high half
-// of the 8-register operand.
-//
-// There are no spare registers for a second set of fragments (128 accumulators + 96 fragment
-// registers), so fragments are reloaded in place as soon as their last use has issued.  The 32
-// instructions run as two sweeps over the 8 A fragments, first against B fragments 0,1 and then
-// against 2,3:
-//     MFMA  0..9    (i,0),(i,1): this step's A fragment 7 and B fragments 2,3 are read in gaps 0..2;
-//                   counted waits let row i start as soon as its own fragment has arrived
-//     wait all reads; wait own loads but the 4 youngest; barrier   <- slab s+1 complete, slab s free
-//     MFMA 10..15   the wave's 4 loads of B rows (slab s+2)
-//     MFMA 16..31   (i,2),(i,3): next step's B fragments 0,1 in gaps 16,17, next step's A fragment
-//                   i-1 after row i (a fragment is overwritten no sooner than one instruction after
-//                   its last use); the wave's 4 loads of A rows (slab s+3) in the even gaps 18..24
-// E5M2: the A matrix holds e5m2 codes, B stays e4m3.  A fragments are the second source operand
-// here (transposed product), whose format field is blgp.
-#define MI355_MFMA_FP8(E5M2, acc, blo, bhi, alo, ahi)                                              \
-  do {                                                                                             \
-    const i32x8v b8_ = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7);                  \
-    const i32x8v a8_ = __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);                  \
-    if (E5M2)                                                                                      \
-      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 blgp:1" : "+v"(acc) : "v"(b8_), "v"(a8_));         \
-    else                                                                                           \
-      asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(acc) : "v"(b8_), "v"(a8_)); \
-  } while (0)
-
-// At most `n` LDS reads still outstanding (they return in order).
-#define MI355_WAIT_LGKM(n) asm volatile("s_waitcnt lgkmcnt(" #n ")" ::: "memory")
-
-struct Fp8Frags {
-  i32x4v a_lo[8], a_hi[8], b_lo[4], b_hi[4];
-};
-
-template <bool E5M2>
-__device__ __forceinline__ void gemm_fp8_step(f32x4v (&acc)[8][4], Fp8Frags &f, const GemmWalk &w, uint32_t first) {
-  constexpr bool READS = true;
-  const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u, an_hi = w.a_nxt ^ 64u, bn_hi = w.b_nxt ^ 64u;
-#define MM(i, j) MI355_MFMA_FP8(E5M2, acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i])
-#define LDA(q) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
-#define LDB(q) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
-#define RD_A_NEXT(i, off)                                                                          \
-  if (READS) { MI355_DS_READ(f.a_lo[i], w.a_nxt, off); MI355_DS_READ(f.a_hi[i], an_hi, off); }
-#define RD_B_NEXT(j, off)                                                                          \
-  if (READS) { MI355_DS_READ(f.b_lo[j], w.b_nxt, off); MI355_DS_READ(f.b_hi[j], bn_hi, off); }
-  // On entry the reads of B fragments 0,1 and A fragments 0..6 of this step are in flight, in that order.
-  MI355_WAIT_LGKM(12);                                   // B0, B1, A0 have arrived
-  MM(0, 0); MI355_DS_READ(f.a_lo[7], w.a_cur, 14336); MI355_DS_READ(f.a_hi[7], a_hi, 14336);
-  MM(0, 1); MI355_DS_READ(f.b_lo[2], w.b_cur, 4096); MI355_DS_READ(f.b_hi[2], b_hi, 4096);
-  MI355_WAIT_LGKM(14);                                   // A1
-  MM(1, 0); MI355_DS_READ(f.b_lo[3], w.b_cur, 6144); MI355_DS_READ(f.b_hi[3], b_hi, 6144);
-  MM(1, 1);
-  MI355_WAIT_LGKM(14);                                   // A2
-  MM(2, 0); MM(2, 1);
-  MI355_WAIT_LGKM(12);                                   // A3
-  MM(3, 0); MM(3, 1);
-  MI355_WAIT_LGKM(10);                                   // A4
-  MM(4, 0); MM(4, 1);
-  // every read of this step's slab has returned (its two slots are free); with the 4 A loads of the
-  // last step still allowed in flight, this wave's share of the next slab has landed
-  MI355_STEP_BARRIER(first, "s_waitcnt lgkmcnt(0)\n");
-  MM(5, 0); LDB(0);
-  MM(5, 1);
-  MM(6, 0); LDB(1);
-  MM(6, 1);
-  MM(7, 0); LDB(2);
-  MM(7, 1); LDB(3);
-  MM(0, 2); RD_B_NEXT(0, 0);
-  MM(0, 3); RD_B_NEXT(1, 2048);
-  MM(1, 2); LDA(0);
-  MM(1, 3); RD_A_NEXT(0, 0);
-  MM(2, 2); LDA(1);
-  MM(2, 3); RD_A_NEXT(1, 2048);
-  MM(3, 2); LDA(2);
-  MM(3, 3); RD_A_NEXT(2, 4096);
-  MM(4, 2); LDA(3);
-  MM(4, 3); RD_A_NEXT(3, 6144);
-  MM(5, 2);
-  MM(5, 3); RD_A_NEXT(4, 8192);
-  MM(6, 2);
-  MM(6, 3); RD_A_NEXT(5, 10240);
-  MM(7, 2);
-  MM(7, 3); RD_A_NEXT(6, 12288);
-#undef RD_A_NEXT
-#undef RD_B_NEXT
-#undef LDA
-#undef LDB
-#undef MM
-}
-
-template <bool E5M2>
-__global__ void __launch_bounds__(kThreads)
-gemm_fp8_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, uint16_t *__restrict__ C,
-                uint32_t N, uint32_t k_bytes, float scale, uint32_t tiles_m, uint32_t tiles_n) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-  const uint32_t tid = threadIdx.x, lane = tid % 64;
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
-  const uint32_t wm = wave / 4, wn = wave % 4;
-  const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
-
-  // ring, loads and fragment addresses exactly as in the bf16 kernel (rows are 128 bytes in both)
-  Ring ring;
-  ring.start(A, B, k_bytes, (uint32_t)(uintptr_t)lds, wave, lane, grid);
-  const uint32_t steps = ring.steps;
-
-  f32x4v acc[8][4];
-#pragma unroll
-  for (int i = 0; i < 8; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
-  Fp8Frags f;
-  // what a step expects in flight on entry: B fragments 0,1 then A fragments 0..6
-  {
-    const GemmWalk &w = ring.w;
-    const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u;
-    MI355_DS_READ(f.b_lo[0], w.b_cur, 0); MI355_DS_READ(f.b_hi[0], b_hi, 0);
-    MI355_DS_READ(f.b_lo[1], w.b_cur, 2048); MI355_DS_READ(f.b_hi[1], b_hi, 2048);
-    MI355_DS_READ(f.a_lo[0], w.a_cur, 0); MI355_DS_READ(f.a_hi[0], a_hi, 0);
-    MI355_DS_READ(f.a_lo[1], w.a_cur, 2048); MI355_DS_READ(f.a_hi[1], a_hi, 2048);
-    MI355_DS_READ(f.a_lo[2], w.a_cur, 4096); MI355_DS_READ(f.a_hi[2], a_hi, 4096);
-    MI355_DS_READ(f.a_lo[3], w.a_cur, 6144); MI355_DS_READ(f.a_hi[3], a_hi, 6144);
-    MI355_DS_READ(f.a_lo[4], w.a_cur, 8192); MI355_DS_READ(f.a_hi[4], a_hi, 8192);
-    MI355_DS_READ(f.a_lo[5], w.a_cur, 10240); MI355_DS_READ(f.a_hi[5], a_hi, 10240);
-    MI355_DS_READ(f.a_lo[6], w.a_cur, 12288); MI355_DS_READ(f.a_hi[6], a_hi, 12288);
-  }
-
-  // one loop over the steps of all tiles of the workgroup
-  uint32_t round = 0, left = steps, first = 1;
-  for (uint32_t g = grid.mine * steps; g > 0; g--) {
-    gemm_fp8_step<E5M2>(acc, f, ring.w, first);
-    ring.advance();
-    first = 0;
-    if (--left == 0) {
-      MI355_END_OF_TILE(acc);
-      uint32_t tm, tn;
-      tile_at(grid, round, tm, tn);
-      store_tile<kScaledBf16>(acc, C, N, tm * kTile + wm * 128u + lane % 16u, tn * kTile + wn * 64u, lane, scale);
-#pragma unroll
-      for (int i = 0; i < 8; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = (f32x4v){0.f, 0.f, 0.f, 0.f};
-      round++;
-      left = steps;
-      first = 1;
-    }
-  }
-  MI355_DRAIN_RING();
-}
-
 int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, uint32_t M, uint32_t N, uint32_t K,
                  uint32_t elem) {
   MI355_REQUIRE(dev, A && B && C, "gemm: null buffer");
@@ -561,25 +418,14 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
   return MI355_OK;
 }
 
-template <int KIND>
-int launch_halves(mi355_dev *dev, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N,
-                  uint32_t K, uint32_t elem) {
+template <int OP>
+int launch_ring(mi355_dev *dev, const char *what, const void *A, const void *B, void *C, uint32_t M,
+               uint32_t N, uint32_t K, uint32_t elem, float scale) {
   if (int rc = check_shapes(dev, A, B, C, M, N, K, elem)) return rc;
-  if (int rc = allow_full_lds(dev, &gemm_bf16_kernel<KIND>, KIND == kBf16 ? kLdsBf16 : KIND == kF16 ? kLdsF16 : kLdsI8)) return rc;
+  if (int rc = allow_full_lds(dev, &gemm_ring_kernel<OP>, kLdsRing0 + OP)) return rc;
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_bf16_kernel<KIND><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
-      (const uint8_t *)A, (const uint8_t *)B, C, N, K * elem, tiles_m, tiles_n);
-  MI355_LAUNCH_CHECK(dev, what);
-  return MI355_OK;
-}
-
-template <bool E5M2>
-int launch_fp8(mi355_dev *dev, const char *what, const uint8_t *A, const uint8_t *B, uint16_t *C, uint32_t M,
-               uint32_t N, uint32_t K, float scale) {
-  if (int rc = check_shapes(dev, A, B, C, M, N, K, 1)) return rc;
-  if (int rc = allow_full_lds(dev, &gemm_fp8_kernel<E5M2>, E5M2 ? kLdsFp8E5m2 : kLdsFp8E4m3)) return rc;
-  const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
-  gemm_fp8_kernel<E5M2><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(A, B, C, N, K, scale, tiles_m, tiles_n);
+  gemm_ring_kernel<OP><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
+      (const uint8_t *)A, (const uint8_t *)B, C, N, K * elem, scale, tiles_m, tiles_n);
   MI355_LAUNCH_CHECK(dev, what);
   return MI355_OK;
 }
@@ -589,13 +435,13 @@ int launch_fp8(mi355_dev *dev, const char *what, const uint8_t *A, const uint8_t
 extern "C" int mi355_gemm_bf16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C, uint32_t M,
                                uint32_t N, uint32_t K) {
   MI355_ENTER(dev);
-  return launch_halves<kBf16>(dev, "gemm_bf16", A, B, C, M, N, K, 2);
+  return launch_ring<kOpBf16>(dev, "gemm_bf16", A, B, C, M, N, K, 2, 1.0f);
 }
 
 extern "C" int mi355_gemm_f16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C, uint32_t M,
                               uint32_t N, uint32_t K) {
   MI355_ENTER(dev);
-  return launch_halves<kF16>(dev, "gemm_f16", A, B, C, M, N, K, 2);
+  return launch_ring<kOpF16>(dev, "gemm_f16", A, B, C, M, N, K, 2, 1.0f);
 }
 
 extern "C" int mi355_gemm_f32(mi355_dev *dev, const float *A, const float *B, float *C, uint32_t M, uint32_t N,
@@ -613,17 +459,17 @@ extern "C" int mi355_gemm_f32(mi355_dev *dev, const float *A, const float *B, fl
 extern "C" int mi355_gemm_i8(mi355_dev *dev, const int8_t *A, const int8_t *B, int32_t *C, uint32_t M, uint32_t N,
                              uint32_t K) {
   MI355_ENTER(dev);
-  return launch_halves<kI8>(dev, "gemm_i8", A, B, C, M, N, K, 1);
+  return launch_ring<kOpI8>(dev, "gemm_i8", A, B, C, M, N, K, 1, 1.0f);
 }
 
 extern "C" int mi355_gemm_fp8_e4m3(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C, uint32_t M,
                                    uint32_t N, uint32_t K, float scale_a, float scale_b) {
   MI355_ENTER(dev);
-  return launch_fp8<false>(dev, "gemm_fp8_e4m3", A, B, C, M, N, K, scale_a * scale_b);
+  return launch_ring<kOpE4m3>(dev, "gemm_fp8_e4m3", A, B, C, M, N, K, 1, scale_a * scale_b);
 }
 
 extern "C" int mi355_gemm_fp8_e5m2(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C, uint32_t M,
                                    uint32_t N, uint32_t K, float scale_a, float scale_b) {
   MI355_ENTER(dev);
-  return launch_fp8<true>(dev, "gemm_fp8_e5m2", A, B, C, M, N, K, scale_a * scale_b);
+  return launch_ring<kOpE5m2>(dev, "gemm_fp8_e5m2", A, B, C, M, N, K, 1, scale_a * scale_b);
 }

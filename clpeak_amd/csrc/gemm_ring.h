@@ -174,7 +174,7 @@ constexpr size_t kRingBytes = 5 * (size_t)kSlabBytes;   // five 32 KiB slots: al
 
 // A kernel that takes the whole LDS must be allowed to, once per device handle (the attribute belongs to
 // the function on the handle's device).  `bit` names the kernel within mi355_dev::full_lds_allowed.
-enum { kLdsBf16 = 0, kLdsF16, kLdsI8, kLdsFp8E4m3, kLdsFp8E5m2, kLdsF32, kLdsMxfp4 };
+enum { kLdsF32 = 0, kLdsMxfp4, kLdsRing0 /* + the operand kind of gemm_ring_kernel, five of them */ };
 template <typename Kernel>
 inline int allow_full_lds(mi355_dev *dev, Kernel kernel, unsigned bit) {
   if (dev->full_lds_allowed & (1u << bit)) return MI355_OK;

@@ -54,12 +54,12 @@ def test_gemm_kernels_fit_the_register_file(tmp_path):
     asm = device_asm(tmp_path, "gemm.hip")
     meta = kernel_metadata(asm)
     # (kernel template, instantiation tag in the mangled name) -> the matrix instruction of its loop and how
-    # many of them the one instance of the step holds (the loop runs through all tiles of a workgroup)
-    expect = {("gemm_bf16_kernel", "ILi0E"): ("v_mfma_f32_16x16x32_bf16", 64),
-              ("gemm_bf16_kernel", "ILi1E"): ("v_mfma_f32_16x16x32_f16", 64),
-              ("gemm_bf16_kernel", "ILi2E"): ("v_mfma_i32_16x16x64_i8", 64),
-              ("gemm_fp8_kernel", "ILb0E"): ("v_mfma_f32_16x16x128_f8f6f4", 32),
-              ("gemm_fp8_kernel", "ILb1E"): ("v_mfma_f32_16x16x128_f8f6f4", 32)}
+    # many of them the one instance of the step holds: 32 slots, one fp8 instruction or a pair per slot
+    expect = {("gemm_ring_kernel", "ILi0E"): ("v_mfma_f32_16x16x128_f8f6f4", 32),
+              ("gemm_ring_kernel", "ILi1E"): ("v_mfma_f32_16x16x128_f8f6f4", 32),
+              ("gemm_ring_kernel", "ILi2E"): ("v_mfma_f32_16x16x32_bf16", 64),
+              ("gemm_ring_kernel", "ILi3E"): ("v_mfma_f32_16x16x32_f16", 64),
+              ("gemm_ring_kernel", "ILi4E"): ("v_mfma_i32_16x16x64_i8", 64)}
     for (kernel, tag), (insn, count) in expect.items():
         name = next(k for k in meta if kernel + tag in k)
         m = meta[name]
@@ -71,15 +71,18 @@ def test_gemm_kernels_fit_the_register_file(tmp_path):
         assert m.get("group_segment_fixed_size", 0) == 0, (name, m)
         body = kernel_body(asm, name)
         assert body.count(insn) == count, (name, body.count(insn))
-        if tag == "ILb1E":
+        if tag == "ILi1E":
             assert body.count("blgp:1") == count      # the e5m2 operand is the second source
+        if count == 64:   # a pair is issued back to back on one accumulator: same destination twice in a row
+            dst = re.findall(insn + r" (v\[\d+:\d+\]),", body)
+            assert len(dst) == 64 and all(dst[2 * k] == dst[2 * k + 1] for k in range(32)), name
         # the direct-to-LDS loads: 20 in the prologue (five ring slots) + 8 per steady-state step
         assert body.count("global_load_lds_dwordx4") >= 20 + 8, name
         # no LDS stores at all on this path
         assert "ds_write" not in body, name
         # the accumulators leave through the packed conversions, two values per instruction
-        if tag != "ILi2E":
-            cvt = "v_cvt_pk_f16_f32" if tag == "ILi1E" else "v_cvt_pk_bf16_f32"
+        if tag != "ILi4E":
+            cvt = "v_cvt_pk_f16_f32" if tag == "ILi3E" else "v_cvt_pk_bf16_f32"
             assert body.count(cvt) == 64, (name, body.count(cvt))   # 32 tiles x 4 values per lane
 
 
