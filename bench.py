@@ -71,6 +71,8 @@ def bench_rows(dev, quick, only):
         _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=False, one_set=False)
     if "matrix_zero" in only:
         _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=True, one_set=True)
+    if "matrix_ref" in only:
+        _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=False, one_set=True, reference=True)
     if "gemm" in only:
         _gemm_rows(dev, capi, wl, add, budget, constant=False)
     if "gemm_const" in only:
@@ -128,7 +130,7 @@ def _mad_rows(dev, capi, add, budget):
     out.free()
 
 
-def _matrix_rows(dev, wl, add, budget, only, zero, one_set):
+def _matrix_rows(dev, wl, add, budget, only, zero, one_set, reference=False):
     # --- dense MFMA / SMFMAC: 2048 waves x 4 chains x 4096 iterations ------------------------
     # one_set: the four accumulator chains of a wave share one A and one B fragment, held in the same
     # registers, as the reference's kernels do (src/rocm/rocm_kernels/mfma_bf16.hip:16-30); that is the
@@ -138,13 +140,15 @@ def _matrix_rows(dev, wl, add, budget, only, zero, one_set):
     # zero: the same launches on all-zero operands.  Nothing toggles in the multipliers, the part holds
     # its boost clock, and the row shows the issue rate of the loop itself (the seeded rows show what the
     # part sustains under the power that random operands draw).
+    # reference: the same launches on the constants the reference's own kernels multiply (1.0, byte 0x38,
+    # byte 0x01, nibble 4 under scales of 0x3f, sparsity index 0): like for like with what it measures.
     waves, iters = 2048, 4096
-    tail = " zero operands" if zero else ("" if one_set else " distinct operands per chain")
+    tail = " zero operands" if zero else " reference operands" if reference else ("" if one_set else " distinct operands per chain")
     clk = dev.alloc(16)
     peaks = {0: "f16", 1: "bf16", 2: "f16", 3: "bf16", 4: "int8", 5: "fp8", 6: "fp8", 7: "fp6", 8: "fp6", 9: "fp4"}
     for kind in sorted(wl.DENSE) if "mfma" in only else []:
         s = wl.DENSE[kind]
-        A, B, sA, sB = wl.dense_inputs(kind, waves, SEED)
+        A, B, sA, sB = wl.reference_dense_inputs(kind, waves) if reference else wl.dense_inputs(kind, waves, SEED)
         if zero:
             A, B = np.zeros_like(A), np.zeros_like(B)
         bufs = [dev.from_host(A), dev.from_host(B), dev.from_host(sA) if sA is not None else None,
@@ -161,7 +165,7 @@ def _matrix_rows(dev, wl, add, budget, only, zero, one_set):
     speaks = {0: "f16", 1: "bf16", 2: "fp8", 3: "fp8", 4: "int8"}
     for kind in sorted(wl.SPARSE) if "smfmac" in only else []:
         s = wl.SPARSE[kind]
-        Ac, meta, B = wl.sparse_inputs(kind, waves, SEED)
+        Ac, meta, B = wl.reference_sparse_inputs(kind, waves) if reference else wl.sparse_inputs(kind, waves, SEED)
         if zero:
             Ac, B = np.zeros_like(Ac), np.zeros_like(B)
         bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
@@ -345,8 +349,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel over 1 GiB (20 launches): under rocprofv3 --pmc this "
                          "gives what FETCH_SIZE / WRITE_SIZE read for a transfer of known size")
-    ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,gemm,gemm_const,lds,transfer",
-                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,gemm,gemm_const,lds,transfer")
+    ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer",
+                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; the hot path has no multi-GPU step "

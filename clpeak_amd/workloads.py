@@ -43,6 +43,15 @@ SPARSE = {
     4: dict(name="smfmac_int8", shape="16x16x128", K=128, fmt=I8, sigma=0.0),
 }
 
+# The operand codes of the reference's own kernels, which run on constants: 1.0 in the 16-bit kinds
+# (src/rocm/rocm_kernels/mfma_fp16.hip:24-25, mfma_bf16.hip:16-17), byte 0x38 in the 8-bit floating kinds
+# (mfma_fp8.hip:17-18: 1.0 as e4m3, 0.5 as e5m2), byte 0x01 for int8 (mfma_int8.hip:17-18), nibble 4 (2.0 as
+# e2m1) under E8M0 scales of 0x3f for the block-scaled kind (mfma_mxfp4.hip:23-29), sparsity index 0
+# (smfmac_fp16.hip:26).  The two fp6 kinds, which the reference does not have, take their code of 1.0.
+REFERENCE_CODE = {F16: 0x3C00, BF16: 0x3F80, E4M3: 0x38, E5M2: 0x38, E2M3: 0x08, E3M2: 0x0C, E2M1: 0x4, I8: 0x01}
+REFERENCE_VALUE = {F16: 1.0, BF16: 1.0, E4M3: 1.0, E5M2: 0.5, E2M3: 1.0, E3M2: 1.0, E2M1: 2.0, I8: 1}
+REFERENCE_SCALE, REFERENCE_META = 0x3F, 0x00
+
 _lib = None
 
 
@@ -68,6 +77,40 @@ def operand(fmt, sigma, seed, stream, n):
     if got != out.size:
         raise RuntimeError(f"host generator wrote {got} of {out.size} bytes")
     return out
+
+
+def constant_operand(fmt, code, n):
+    """n elements, each the bit pattern `code` of `fmt`, packed as `operand` packs them."""
+    bits = _BITS[fmt]
+    if bits == 16:
+        return np.full(n, code, dtype="<u2").view(np.uint8)
+    if bits == 8:
+        return np.full(n, code, dtype=np.uint8)
+    if bits == 4:
+        return np.full(n // 2, code | code << 4, dtype=np.uint8)
+    word = code | code << 6 | code << 12 | code << 18          # four 6-bit elements in three bytes
+    return np.tile(np.array([word & 0xFF, word >> 8 & 0xFF, word >> 16 & 0xFF], dtype=np.uint8), n // 4)
+
+
+def reference_dense_inputs(kind, waves):
+    """The shapes of `dense_inputs`, every element the constant the reference's kernel of the kind holds."""
+    s = DENSE[kind]
+    units = waves * 4
+    A = constant_operand(s["fmt"], REFERENCE_CODE[s["fmt"]], units * s["M"] * s["K"])
+    B = constant_operand(s["fmt"], REFERENCE_CODE[s["fmt"]], units * s["N"] * s["K"])
+    sA = sB = None
+    if s["scaled"]:
+        sA = np.full(units * s["M"] * (s["K"] // 32), REFERENCE_SCALE, dtype=np.uint8)
+        sB = np.full(units * s["N"] * (s["K"] // 32), REFERENCE_SCALE, dtype=np.uint8)
+    return A, B, sA, sB
+
+
+def reference_sparse_inputs(kind, waves):
+    s = SPARSE[kind]
+    units = waves * 4
+    Ac = constant_operand(s["fmt"], REFERENCE_CODE[s["fmt"]], units * 16 * (s["K"] // 2))
+    B = constant_operand(s["fmt"], REFERENCE_CODE[s["fmt"]], units * 16 * s["K"])
+    return Ac, np.full(units * 16 * (s["K"] // 4), REFERENCE_META, dtype=np.uint8), B
 
 
 def e8m0_scales(seed, stream, n):

@@ -17,6 +17,7 @@ import numpy as np
 import pytest
 
 from clpeak_amd import capi
+from clpeak_amd import workloads as product_wl
 from oracle import pyoracle as orc
 from oracle import workloads as wl
 
@@ -138,3 +139,61 @@ def test_smfmac_parity_one_operand_set(dev, kind, iters):
 def test_smfmac_full_launch(dev, kind, one_set):
     got, ref, ab, is_int = _run_sparse(dev, kind, 2048, 4096, one_set=one_set)
     _check(got, ref, ab, is_int, wl.SPARSE[kind]["name"], 4096)
+
+
+def _closed_form(fmt, terms, iters, scaled):
+    """acc after `iters` instructions that each add `terms` products of the reference's constant with itself."""
+    v = float(product_wl.REFERENCE_VALUE[fmt])
+    block = 2.0 ** (2 * (product_wl.REFERENCE_SCALE - 127)) if scaled else 1.0
+    return iters * terms * v * v * block
+
+
+@pytest.mark.parametrize("one_set", [False, True])
+@pytest.mark.parametrize("kind", sorted(product_wl.DENSE))
+def test_mfma_dense_on_the_reference_operands(dev, kind, one_set):
+    """The reference's kernels multiply constants (1.0, byte 0x38, byte 0x01, nibble 4 under scales of 0x3f:
+    src/rocm/rocm_kernels/mfma_bf16.hip:16-17, mfma_fp8.hip:17-18, mfma_int8.hip:17-18, mfma_mxfp4.hip:23-29).
+    On those inputs every element of every accumulator is iterations x K x constant^2 (x both block
+    scales), a power of two times an integer below 2^24: exact in fp32 and int32, so the comparison is."""
+    s = product_wl.DENSE[kind]
+    waves = 8
+    A, B, sA, sB = product_wl.reference_dense_inputs(kind, waves)
+    n_out = waves * 4 * s["M"] * s["N"]
+    for iters in (1, 13, 4096):
+        bufs = [dev.from_host(x) if x is not None else None for x in (A, B, sA, sB)]
+        out = dev.alloc(n_out * 4)
+        dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], out, waves, iters, one_set=one_set)
+        is_int = s["fmt"] == product_wl.I8
+        got = out.download(np.int32 if is_int else np.float32, n_out)
+        want = _closed_form(s["fmt"], s["K"], iters, s["scaled"])
+        assert np.all(got == (np.int32(want) if is_int else np.float32(want))), (s["name"], iters, got[:4], want)
+        ref, _ = orc.mfma_dense(kind, A, B, sA, sB, waves, iters, s["M"] * s["N"], is_int=is_int)
+        assert np.array_equal(got, ref), (s["name"], iters)
+        for b in bufs + [out]:
+            if b is not None:
+                b.free()
+
+
+@pytest.mark.parametrize("one_set", [False, True])
+@pytest.mark.parametrize("kind", sorted(product_wl.SPARSE))
+def test_smfmac_on_the_reference_operands(dev, kind, one_set):
+    """Constants and sparsity index 0 (src/rocm/rocm_kernels/smfmac_fp16.hip:24-27, smfmac_fp8.hip:19-21,
+    smfmac_int8.hip:18-20): K/2 kept values per row, each against a B element of the same constant.  Index 0
+    names position 0 of every group twice, which the oracle refuses as metadata; it is given the first
+    proper pattern (positions 0 and 1) instead, which on a constant B selects the same values."""
+    s = product_wl.SPARSE[kind]
+    waves = 8
+    Ac, meta, B = product_wl.reference_sparse_inputs(kind, waves)
+    n_out = waves * 4 * 256
+    for iters in (1, 13, 4096):
+        bufs = [dev.from_host(x) for x in (Ac, meta, B)]
+        out = dev.alloc(n_out * 4)
+        dev.smfmac(kind, bufs[0], bufs[1], bufs[2], out, waves, iters, one_set=one_set)
+        is_int = s["fmt"] == product_wl.I8
+        got = out.download(np.int32 if is_int else np.float32, n_out)
+        want = _closed_form(s["fmt"], s["K"] // 2, iters, False)
+        assert np.all(got == (np.int32(want) if is_int else np.float32(want))), (s["name"], iters, got[:4], want)
+        ref, _ = orc.smfmac(kind, Ac, np.full_like(meta, 0b0100), B, waves, iters, is_int=is_int)
+        assert np.array_equal(got, ref), (s["name"], iters)
+        for b in bufs + [out]:
+            b.free()

@@ -1,6 +1,8 @@
 """Pins the oracle's kernels (CPU only) against what the mathematics fixes: closed forms
 of the affine recurrence, numpy restatements written from the definitions in
 include/clpeak_mi355.h, exact integer arithmetic in Python, special cases."""
+import os
+
 import numpy as np
 import pytest
 
@@ -381,3 +383,27 @@ def test_gemm_tile2_fp32_and_fp64_against_exact_sums():
     big_a = rng.standard_normal((8, 32)); big_b = rng.standard_normal((6, 32))
     got = orc.gemm_tile2(orc.FMT_F64, orc.FMT_F64, big_a, big_b, 32, 32, 32, 2, 1, 4, 3)
     assert np.allclose(got, big_a[2:6] @ big_b[1:4].T, rtol=1e-13, atol=1e-13)
+
+
+# ---- the reference's own operands ---------------------------------------------------------------
+def test_oracle_on_the_reference_constants_is_the_closed_form():
+    """The reference's kernels run on constants (src/rocm/rocm_kernels/mfma_bf16.hip:16-17, mfma_fp8.hip:17-18,
+    mfma_int8.hip:17-18, mfma_mxfp4.hip:23-29, smfmac_fp16.hip:24-27).  Every accumulator element is then
+    iterations x terms x constant^2 (x both block scales), exactly; the builders live on the product side."""
+    from clpeak_amd import workloads as product_wl
+    if not os.path.exists(product_wl.HOST_LIB_PATH):
+        pytest.skip("host library not built")
+    waves, iters = 4, 257
+    for kind, s in product_wl.DENSE.items():
+        A, B, sA, sB = product_wl.reference_dense_inputs(kind, waves)
+        is_int = s["fmt"] == product_wl.I8
+        out, _ = orc.mfma_dense(kind, A, B, sA, sB, waves, iters, s["M"] * s["N"], is_int=is_int)
+        v = product_wl.REFERENCE_VALUE[s["fmt"]]
+        want = iters * s["K"] * v * v * (2.0 ** (2 * (product_wl.REFERENCE_SCALE - 127)) if s["scaled"] else 1.0)
+        assert np.all(out == want), (s["name"], out[:4], want)
+    for kind, s in product_wl.SPARSE.items():
+        Ac, meta, B = product_wl.reference_sparse_inputs(kind, waves)
+        is_int = s["fmt"] == product_wl.I8
+        out, _ = orc.smfmac(kind, Ac, np.full_like(meta, 0b0100), B, waves, iters, is_int=is_int)
+        v = product_wl.REFERENCE_VALUE[s["fmt"]]
+        assert np.all(out == iters * (s["K"] // 2) * v * v), (s["name"], out[:4])
