@@ -186,12 +186,12 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
     s43, s52 = 448.0, 57344.0
     kinds = [("rocblas-fp", "fp32", 4, 4, "fp32_mat", "tflops", 0x3f),
              ("rocblas-fp", "fp64", 8, 8, "fp64_mat", "tflops", 0x3f),
-             ("rocblas-fp", "fp16", 2, 2, "f16", "tflops", 0x3c),
+             ("rocblas-fp", "fp16", 2, 2, "f16", "tflops", 0x3f),
              ("rocblas-fp", "bf16", 2, 2, "bf16", "tflops", 0x3f),
              ("hipblaslt-fp8", "fp8_e4m3", 1, 2, "fp8", "tflops", 0x38),
              ("hipblaslt-fp8", "fp8_e5m2", 1, 2, "fp8", "tflops", 0x38),
-             ("hipblaslt-fp8", "mxf4_e2m1", 0.5, 2, "fp4", "tflops", 0x22),
-             ("rocblas-int", "int8", 1, 4, "int8", "tops", 0x01)]
+             ("hipblaslt-fp8", "mxf4_e2m1", 0.5, 2, "fp4", "tflops", 0x38),
+             ("rocblas-int", "int8", 1, 4, "int8", "tops", 0x3f)]
     for test, metric, eb, ob, peak, unit, const_byte in kinds:
         dA, dB, dC = dev.alloc(int(M * K * eb)), dev.alloc(int(N * K * eb)), dev.alloc(M * N * ob)
         extra = []
@@ -227,9 +227,10 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
             dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
             fn = lambda: dev.gemm_i8(dA, dB, dC, M, N, K)
         if constant:
-            # the same launch on constant buffers, as the reference fills them (every byte 0x3f / 0x38,
-            # src/rocm/rocblas.cpp:211-212, src/rocm/hipblaslt_gemm.cpp:271-273): constant operands draw less
-            # power and the part holds a higher clock
+            # the same launch on constant buffers, as the reference fills them (every byte 0x3f in its rocBLAS
+            # test, src/rocm/rocblas.cpp:211-212, every byte 0x38 under block scales of 0x7f in its hipBLASLt
+            # test, src/rocm/hipblaslt_gemm.cpp:272-273 and 417-418): constant operands draw less power and the
+            # part holds a higher clock
             dev.memset(dA, const_byte); dev.memset(dB, const_byte)
             metric += " constant operands"
         us, _ = timed(dev, fn, **budget)

@@ -23,6 +23,14 @@ size_t clpeak_host_seeded_operand(int fmt, double sigma, unsigned long long seed
   return v.size();
 }
 
+// The same formats: n elements of the constant the reference's kernel of the format multiplies.
+size_t clpeak_host_reference_operand(int fmt, unsigned long long n, unsigned char *out, size_t cap) {
+  const std::vector<uint8_t> v = reference_operand((OperandFormat)fmt, n);
+  if (v.size() > cap) return 0;
+  memcpy(out, v.data(), v.size());
+  return v.size();
+}
+
 size_t clpeak_host_seeded_bytes(int what, unsigned long long seed, unsigned stream, unsigned long long n, unsigned char *out) {
   const std::vector<uint8_t> v = what == 0 ? seeded_e8m0(seed, stream, n) : seeded_sparse_meta(seed, stream, n);
   memcpy(out, v.data(), v.size());

@@ -322,12 +322,18 @@ void Mi355Peak::runMfma(Category phase) {
   for (size_t r = 0; r < n; r++) {
     const MfmaRow &m = rows[r];
     auto test = device_->beginTest({m.tag, m.display, m.unit, Category::Unknown, m.description});
-    const std::vector<uint8_t> A = seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_A, units * m.M * m.K);
-    const std::vector<uint8_t> B = seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_B, units * m.N * m.K);
+    const bool ref = workload.referenceOperands;
+    const std::vector<uint8_t> A = ref ? reference_operand(m.fmt, units * m.M * m.K)
+                                       : seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_A, units * m.M * m.K);
+    const std::vector<uint8_t> B = ref ? reference_operand(m.fmt, units * m.N * m.K)
+                                       : seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_B, units * m.N * m.K);
     Buffer dA(api_, dev_, A.size()), dB(api_, dev_, B.size()), out(api_, dev_, units * m.M * m.N * 4);
     Buffer sA(api_, dev_, m.scaled ? units * m.M * (m.K / 32) : 16), sB(api_, dev_, m.scaled ? units * m.N * (m.K / 32) : 16);
     bool ok = dA && dB && out && sA && sB && dA.upload(A) && dB.upload(B);
-    if (ok && m.scaled)
+    if (ok && m.scaled && ref)
+      ok = sA.upload(std::vector<uint8_t>(units * m.M * (m.K / 32), kReferenceScale)) &&
+           sB.upload(std::vector<uint8_t>(units * m.N * (m.K / 32), kReferenceScale));
+    else if (ok && m.scaled)
       ok = sA.upload(seeded_e8m0(workload.seed, MI355_STREAM_SCALE_A, units * m.M * (m.K / 32))) &&
            sB.upload(seeded_e8m0(workload.seed, MI355_STREAM_SCALE_B, units * m.N * (m.K / 32)));
     if (!ok) {
@@ -359,9 +365,13 @@ void Mi355Peak::runSparseMfma(Category phase) {
   for (size_t r = 0; r < n; r++) {
     const SparseRow &m = rows[r];
     auto test = device_->beginTest({m.tag, m.display, m.unit, Category::Unknown, m.description});
-    const std::vector<uint8_t> Ac = seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_A, units * 16 * (m.K / 2));
-    const std::vector<uint8_t> B = seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_B, units * 16 * m.K);
-    const std::vector<uint8_t> meta = seeded_sparse_meta(workload.seed, MI355_STREAM_SPARSE, units * 16 * (m.K / 4));
+    const bool ref = workload.referenceOperands;
+    const std::vector<uint8_t> Ac = ref ? reference_operand(m.fmt, units * 16 * (m.K / 2))
+                                        : seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_A, units * 16 * (m.K / 2));
+    const std::vector<uint8_t> B = ref ? reference_operand(m.fmt, units * 16 * m.K)
+                                       : seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_B, units * 16 * m.K);
+    const std::vector<uint8_t> meta = ref ? std::vector<uint8_t>(units * 16 * (m.K / 4), kReferenceSparseMeta)
+                                          : seeded_sparse_meta(workload.seed, MI355_STREAM_SPARSE, units * 16 * (m.K / 4));
     Buffer dA(api_, dev_, Ac.size()), dB(api_, dev_, B.size()), dM(api_, dev_, meta.size()), out(api_, dev_, units * 256 * 4);
     if (!(dA && dB && dM && out && dA.upload(Ac) && dB.upload(B) && dM.upload(meta))) {
       test.skip(m.tag, ResultStatus::Error, "Failed to allocate or upload operand buffers");
@@ -382,11 +392,19 @@ void Mi355Peak::runSparseMfma(Category phase) {
 
 // ---- GEMM (the slots of the vendor-library tests) ------------------------------------------------------------------
 // One GEMM row: fill the operands on the device, time the launch like any kernel, emit 2*D^3 / time.
+// With reference operands every byte of A and B is `referenceByte`, as the reference's tests set them
+// (0x3f: src/rocm/rocblas.cpp:211-212; 0x38: src/rocm/hipblaslt_gemm.cpp:272-273).
 void Mi355Peak::runGemmRow(logger::TestScope &test, const char *metric, const char *note, size_t elemBytes, size_t outBytes,
-                           const std::function<int(void *, void *)> &fill, const std::function<int(void *, void *, void *)> &launch) {
+                           uint8_t referenceByte, const std::function<int(void *, void *)> &fill,
+                           const std::function<int(void *, void *, void *)> &launch) {
   const uint32_t D = workload.gemmDim;
-  Buffer A(api_, dev_, (size_t)D * D * elemBytes), B(api_, dev_, (size_t)D * D * elemBytes), C(api_, dev_, (size_t)D * D * outBytes);
-  if (!(A && B && C) || fill(A.ptr, B.ptr) != MI355_OK) {
+  const size_t abBytes = (size_t)D * D * elemBytes;
+  Buffer A(api_, dev_, abBytes), B(api_, dev_, abBytes), C(api_, dev_, (size_t)D * D * outBytes);
+  auto constantFill = [&](void *a, void *b) {
+    const int rc = api_.fill_bytes(dev_, (uint8_t *)a, abBytes, workload.seed, MI355_STREAM_GEMM_A, referenceByte, 1);
+    return rc != MI355_OK ? rc : api_.fill_bytes(dev_, (uint8_t *)b, abBytes, workload.seed, MI355_STREAM_GEMM_B, referenceByte, 1);
+  };
+  if (!(A && B && C) || (workload.referenceOperands ? constantFill(A.ptr, B.ptr) : fill(A.ptr, B.ptr)) != MI355_OK) {
     test.skip(metric, ResultStatus::Error, "Failed to allocate or fill GEMM buffers", note);
     return;
   }
@@ -401,25 +419,25 @@ void Mi355Peak::runGemmFp() {
                                   "operands), not a vendor library."});
   const uint32_t D = workload.gemmDim;
   const uint64_t n = (uint64_t)D * D;
-  runGemmRow(test, "fp32", "fp32 inputs, accumulation and output, on the fp32 matrix instruction; A row-major, B column-major.", 4, 4,
+  runGemmRow(test, "fp32", "fp32 inputs, accumulation and output, on the fp32 matrix instruction; A row-major, B column-major.", 4, 4, 0x3f,
              [&](void *a, void *b) {
                const int rc = api_.fill_f32(dev_, (float *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
                return rc != MI355_OK ? rc : api_.fill_f32(dev_, (float *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
              },
              [&](void *a, void *b, void *c) { return api_.gemm_f32(dev_, (const float *)a, (const float *)b, (float *)c, D, D, D); });
-  runGemmRow(test, "fp64", "fp64 inputs, accumulation and output, on the fp64 matrix instruction; A row-major, B column-major.", 8, 8,
+  runGemmRow(test, "fp64", "fp64 inputs, accumulation and output, on the fp64 matrix instruction; A row-major, B column-major.", 8, 8, 0x3f,
              [&](void *a, void *b) {
                const int rc = api_.fill_f64(dev_, (double *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
                return rc != MI355_OK ? rc : api_.fill_f64(dev_, (double *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
              },
              [&](void *a, void *b, void *c) { return api_.gemm_f64(dev_, (const double *)a, (const double *)b, (double *)c, D, D, D); });
-  runGemmRow(test, "fp16", "IEEE half inputs, fp32 accumulation, half output; A row-major, B column-major.", 2, 2,
+  runGemmRow(test, "fp16", "IEEE half inputs, fp32 accumulation, half output; A row-major, B column-major.", 2, 2, 0x3f,
              [&](void *a, void *b) {
                const int rc = api_.fill_f16(dev_, (uint16_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
                return rc != MI355_OK ? rc : api_.fill_f16(dev_, (uint16_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
              },
              [&](void *a, void *b, void *c) { return api_.gemm_f16(dev_, (const uint16_t *)a, (const uint16_t *)b, (uint16_t *)c, D, D, D); });
-  runGemmRow(test, "bf16", "bf16 inputs, fp32 accumulation, bf16 output; A row-major, B column-major.", 2, 2,
+  runGemmRow(test, "bf16", "bf16 inputs, fp32 accumulation, bf16 output; A row-major, B column-major.", 2, 2, 0x3f,
              [&](void *a, void *b) {
                const int rc = api_.fill_bf16(dev_, (uint16_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
                return rc != MI355_OK ? rc : api_.fill_bf16(dev_, (uint16_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
@@ -434,7 +452,7 @@ void Mi355Peak::runGemmFp8() {
   const uint32_t D = workload.gemmDim;
   const uint64_t n = (uint64_t)D * D;
   const float s43 = 448.0f, s52 = 57344.0f;   // uniform [-1,1) stretched over the range of the format
-  runGemmRow(test, "fp8_e4m3", "OCP e4m3 inputs, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2,
+  runGemmRow(test, "fp8_e4m3", "OCP e4m3 inputs, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2, 0x38,
              [&](void *a, void *b) {
                const int rc = api_.fill_fp8_e4m3(dev_, (uint8_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1, s43);
                return rc != MI355_OK ? rc : api_.fill_fp8_e4m3(dev_, (uint8_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1, s43);
@@ -442,7 +460,7 @@ void Mi355Peak::runGemmFp8() {
              [&](void *a, void *b, void *c) {
                return api_.gemm_fp8_e4m3(dev_, (const uint8_t *)a, (const uint8_t *)b, (uint16_t *)c, D, D, D, 1.0f / s43, 1.0f / s43);
              });
-  runGemmRow(test, "fp8_e5m2", "An OCP e5m2 A against an e4m3 B, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2,
+  runGemmRow(test, "fp8_e5m2", "An OCP e5m2 A against an e4m3 B, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2, 0x38,
              [&](void *a, void *b) {
                const int rc = api_.fill_fp8_e5m2(dev_, (uint8_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1, s52);
                return rc != MI355_OK ? rc : api_.fill_fp8_e4m3(dev_, (uint8_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1, s43);
@@ -453,13 +471,15 @@ void Mi355Peak::runGemmFp8() {
   // block-scaled FP4: two e2m1 codes per byte, one E8M0 scale per 32 elements (2^-4 .. 2^4)
   const char *mxNote = "OCP MXFP4: e2m1 inputs with one E8M0 scale per 32 elements along K, fp32 accumulation, bf16 output.";
   {
+    // reference operands: bytes of 0x38 under scales of 0x7f (src/rocm/hipblaslt_gemm.cpp:272-273, 417-418)
+    const bool ref = workload.referenceOperands;
     Buffer A(api_, dev_, (size_t)n / 2), B(api_, dev_, (size_t)n / 2), SA(api_, dev_, (size_t)n / 32), SB(api_, dev_, (size_t)n / 32),
         C(api_, dev_, (size_t)n * 2);
     const bool ok = A && B && SA && SB && C && D % 256 == 0 &&
-                    api_.fill_bytes(dev_, (uint8_t *)A.ptr, n / 2, workload.seed, MI355_STREAM_GEMM_A, 0, 256) == MI355_OK &&
-                    api_.fill_bytes(dev_, (uint8_t *)B.ptr, n / 2, workload.seed, MI355_STREAM_GEMM_B, 0, 256) == MI355_OK &&
-                    api_.fill_bytes(dev_, (uint8_t *)SA.ptr, n / 32, workload.seed, MI355_STREAM_SCALE_A, 123, 9) == MI355_OK &&
-                    api_.fill_bytes(dev_, (uint8_t *)SB.ptr, n / 32, workload.seed, MI355_STREAM_SCALE_B, 123, 9) == MI355_OK;
+                    api_.fill_bytes(dev_, (uint8_t *)A.ptr, n / 2, workload.seed, MI355_STREAM_GEMM_A, ref ? 0x38 : 0, ref ? 1 : 256) == MI355_OK &&
+                    api_.fill_bytes(dev_, (uint8_t *)B.ptr, n / 2, workload.seed, MI355_STREAM_GEMM_B, ref ? 0x38 : 0, ref ? 1 : 256) == MI355_OK &&
+                    api_.fill_bytes(dev_, (uint8_t *)SA.ptr, n / 32, workload.seed, MI355_STREAM_SCALE_A, ref ? 0x7f : 123, ref ? 1 : 9) == MI355_OK &&
+                    api_.fill_bytes(dev_, (uint8_t *)SB.ptr, n / 32, workload.seed, MI355_STREAM_SCALE_B, ref ? 0x7f : 123, ref ? 1 : 9) == MI355_OK;
     float us = -1.0f;
     if (ok)
       us = runKernel([&] { return api_.gemm_mxfp4(dev_, (const uint8_t *)A.ptr, (const uint8_t *)B.ptr, (const uint8_t *)SA.ptr,
@@ -477,7 +497,7 @@ void Mi355Peak::runGemmInt() {
                                   "kernel, not a vendor library."});
   const uint32_t D = workload.gemmDim;
   const uint64_t n = (uint64_t)D * D;
-  runGemmRow(test, "int8", "8-bit integers in [-8, 7], 32-bit totals; A row-major, B column-major.", 1, 4,
+  runGemmRow(test, "int8", "8-bit integers in [-8, 7], 32-bit totals; A row-major, B column-major.", 1, 4, 0x3f,
              [&](void *a, void *b) {
                const int rc = api_.fill_i8(dev_, (int8_t *)a, n, workload.seed, MI355_STREAM_GEMM_A);
                return rc != MI355_OK ? rc : api_.fill_i8(dev_, (int8_t *)b, n, workload.seed, MI355_STREAM_GEMM_B);

@@ -38,6 +38,9 @@ class Mi355Peak : public Peak {
     uint32_t latencyLaunches = 10000;
     uint64_t ldsThreads = 0;              // 0: the reference's rule, max(32M, CUs * 2048 * 256)
     uint64_t transferBytes = 1ull << 29;  // pinned staging buffer of the transfer test
+    // The matrix rows on the constants the reference's kernels and GEMM tests run on instead of seeded
+    // operands (--reference-operands): like for like with the reference's readings.
+    bool referenceOperands = false;
   } workload;
 
  private:
@@ -57,7 +60,7 @@ class Mi355Peak : public Peak {
   void runMfma(Category phase);
   void runSparseMfma(Category phase);
   void runGemmRow(logger::TestScope &test, const char *metric, const char *note, size_t elemBytes, size_t outBytes,
-                  const std::function<int(void *, void *)> &fill, const std::function<int(void *, void *, void *)> &launch);
+                  uint8_t referenceByte, const std::function<int(void *, void *)> &fill, const std::function<int(void *, void *, void *)> &launch);
   void runGemmFp();
   void runGemmFp8();
   void runGemmInt();

@@ -57,6 +57,7 @@ void printUsage(std::ostream &os) {
         "  --describe              print what each test and reading means\n"
         "  --list-devices          list devices and exit\n"
         "  --verbose               diagnostics on stderr\n"
+        "  --reference-operands    matrix rows on the constant operands clpeak's own kernels use, not seeded ones\n"
         "  -v, --version | -h, --help\n";
 }
 
@@ -107,6 +108,7 @@ ParseResult parseCliCore(int argc, char **argv, CliOptions &opts, HostExtras &ex
     else if (a == "--list-devices") opts.listDevices = true;
     else if (a == "--verbose") opts.verbose = true;
     else if (a == "--fake-device") extras.fakeDevice = true;
+    else if (a == "--reference-operands") extras.shape.referenceOperands = true;
     else if (a == "--small-shapes") {
       Mi355Peak::Workload &s = extras.shape;
       s.madItems = 1 << 12; s.madSteps = 64; s.bwFloats = 1 << 22; s.mfmaWavesPerCU = 1;

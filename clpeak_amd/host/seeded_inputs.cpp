@@ -82,6 +82,29 @@ std::vector<uint8_t> seeded_operand(OperandFormat f, double sigma, uint64_t seed
   return out;
 }
 
+std::vector<uint8_t> reference_operand(OperandFormat f, uint64_t n) {
+  uint32_t code = 0;
+  switch (f) {
+    case OperandFormat::F16: code = 0x3C00; break;
+    case OperandFormat::BF16: code = 0x3F80; break;
+    case OperandFormat::E4M3: case OperandFormat::E5M2: code = 0x38; break;
+    case OperandFormat::E2M3: code = 0x08; break;
+    case OperandFormat::E3M2: code = 0x0C; break;
+    case OperandFormat::E2M1: code = 0x4; break;
+    case OperandFormat::I8: code = 0x01; break;
+  }
+  const int bits = operand_bits(f);
+  std::vector<uint8_t> out((n * bits + 7) / 8, 0);
+  for (uint64_t i = 0; i < n; i++) {
+    const uint64_t bit = i * bits;
+    const uint32_t shifted = code << (bit & 7);
+    out[bit >> 3] |= (uint8_t)shifted;
+    if ((bit & 7) + bits > 8) out[(bit >> 3) + 1] |= (uint8_t)(shifted >> 8);
+    if ((bit & 7) + bits > 16) out[(bit >> 3) + 2] |= (uint8_t)(shifted >> 16);
+  }
+  return out;
+}
+
 std::vector<uint8_t> seeded_e8m0(uint64_t seed, uint32_t stream, uint64_t n) {
   std::vector<uint8_t> out(n);
   for (uint64_t i = 0; i < n; i++) out[i] = (uint8_t)(123 + mi355_rng_below(mi355_rng_word(seed, stream, i), 9));

@@ -19,6 +19,14 @@ std::vector<uint8_t> seeded_e8m0(uint64_t seed, uint32_t stream, uint64_t n);
 // 2:4 keep patterns: one byte per group of four, first kept position | second << 2, first < second.
 std::vector<uint8_t> seeded_sparse_meta(uint64_t seed, uint32_t stream, uint64_t n);
 
+// The constants of the reference's matrix kernels, in the packing of seeded_operand: 1.0 in the 16-bit
+// formats (src/rocm/rocm_kernels/mfma_fp16.hip:24-25, mfma_bf16.hip:16-17), byte 0x38 in the 8-bit floating
+// formats (mfma_fp8.hip:17-18), byte 0x01 for int8 (mfma_int8.hip:17-18), nibble 4 for e2m1
+// (mfma_mxfp4.hip:23-26); the fp6 formats, which the reference lacks, take their code of 1.0.  Its block
+// scales are bytes of 0x3f (mfma_mxfp4.hip:28-29), its sparsity index register is 0 (smfmac_fp16.hip:26).
+std::vector<uint8_t> reference_operand(OperandFormat f, uint64_t n);
+constexpr uint8_t kReferenceScale = 0x3f, kReferenceSparseMeta = 0x00;
+
 // dst[i] = uniform [0,1) element i of `stream` (the values the device fill of the bandwidth buffer writes).
 void seeded_uniform_f32(float *dst, uint64_t n, uint64_t seed, uint32_t stream);
 

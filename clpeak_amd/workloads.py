@@ -64,6 +64,8 @@ def _host():
         L.clpeak_host_seeded_operand.argtypes = [C.c_int, C.c_double, C.c_ulonglong, C.c_uint, C.c_ulonglong,
                                                  C.c_void_p, C.c_size_t]
         L.clpeak_host_seeded_operand.restype = C.c_size_t
+        L.clpeak_host_reference_operand.argtypes = [C.c_int, C.c_ulonglong, C.c_void_p, C.c_size_t]
+        L.clpeak_host_reference_operand.restype = C.c_size_t
         L.clpeak_host_seeded_bytes.argtypes = [C.c_int, C.c_ulonglong, C.c_uint, C.c_ulonglong, C.c_void_p]
         L.clpeak_host_seeded_bytes.restype = C.c_size_t
         _lib = L
@@ -92,12 +94,22 @@ def constant_operand(fmt, code, n):
     return np.tile(np.array([word & 0xFF, word >> 8 & 0xFF, word >> 16 & 0xFF], dtype=np.uint8), n // 4)
 
 
+def reference_operand(fmt, n):
+    """n elements of the reference's constant for `fmt`, from the host layer's generator (what `Mi355Peak`
+    uploads under --reference-operands)."""
+    out = np.empty(n * _BITS[fmt] // 8, dtype=np.uint8)
+    got = _host().clpeak_host_reference_operand(fmt, n, out.ctypes.data, out.size)
+    if got != out.size:
+        raise RuntimeError(f"host generator wrote {got} of {out.size} bytes")
+    return out
+
+
 def reference_dense_inputs(kind, waves):
     """The shapes of `dense_inputs`, every element the constant the reference's kernel of the kind holds."""
     s = DENSE[kind]
     units = waves * 4
-    A = constant_operand(s["fmt"], REFERENCE_CODE[s["fmt"]], units * s["M"] * s["K"])
-    B = constant_operand(s["fmt"], REFERENCE_CODE[s["fmt"]], units * s["N"] * s["K"])
+    A = reference_operand(s["fmt"], units * s["M"] * s["K"])
+    B = reference_operand(s["fmt"], units * s["N"] * s["K"])
     sA = sB = None
     if s["scaled"]:
         sA = np.full(units * s["M"] * (s["K"] // 32), REFERENCE_SCALE, dtype=np.uint8)
@@ -108,8 +120,8 @@ def reference_dense_inputs(kind, waves):
 def reference_sparse_inputs(kind, waves):
     s = SPARSE[kind]
     units = waves * 4
-    Ac = constant_operand(s["fmt"], REFERENCE_CODE[s["fmt"]], units * 16 * (s["K"] // 2))
-    B = constant_operand(s["fmt"], REFERENCE_CODE[s["fmt"]], units * 16 * s["K"])
+    Ac = reference_operand(s["fmt"], units * 16 * (s["K"] // 2))
+    B = reference_operand(s["fmt"], units * 16 * s["K"])
     return Ac, np.full(units * 16 * (s["K"] // 4), REFERENCE_META, dtype=np.uint8), B
 
 

@@ -36,6 +36,20 @@ def test_cli_small_shapes_all_rows(tmp_path):
     assert skipped[("kernel_launch_latency", "dispatch")] == "unsupported"
 
 
+def test_cli_reference_operands(tmp_path):
+    """The matrix rows on the constants the reference's kernels run on: all measured, none an error."""
+    x = tmp_path / "ref.xml"
+    r = subprocess.run([CLI, "--small-shapes", "--reference-operands", "--max-time", "20", "--no-bandwidth", "--no-latency",
+                        "--xml-file", str(x)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    run = ET.parse(x).getroot().find("run")
+    got = {(t.get("name"), m.get("name")): (m.get("status"), m.text) for t in run.iter("test") for m in t.findall("metric")}
+    assert not [k for k, (status, _) in got.items() if status == "error"], got
+    for key in [("mfma_bf16", "mfma_bf16"), ("mfma_mxfp4", "mfma_mxfp4"), ("smfmac_fp8", "smfmac_fp8"), ("smfmac_int8", "smfmac_int8"),
+                ("rocblas-fp", "fp64"), ("rocblas-fp", "bf16"), ("hipblaslt-fp8", "mxf4_e2m1"), ("rocblas-int", "int8")]:
+        assert got[key][0] is None and float(got[key][1]) > 0, key
+
+
 def test_cli_list_devices():
     r = subprocess.run([CLI, "--list-devices"], capture_output=True, text=True, timeout=60)
     assert r.returncode == 0 and "=== ROCm backend ===" in r.stdout and "ROCm Device 0:" in r.stdout and "[GPU]" in r.stdout

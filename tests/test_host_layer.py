@@ -275,6 +275,26 @@ def test_backend_workloads_equal_oracle_workloads():
     assert [getattr(pw, n) for n in dir(pw) if n.startswith("STREAM_")] == [getattr(wl, n) for n in dir(pw) if n.startswith("STREAM_")]
 
 
+def test_reference_operands(host, tmp_path):
+    """--reference-operands: the host generator's constants are the codes listed for the reference's kernels,
+    in the packing of the seeded operands, and the flag leaves the row set as it is."""
+    from clpeak_amd import workloads as pw
+    for fmt, code in pw.REFERENCE_CODE.items():
+        n = 256
+        assert np.array_equal(pw.reference_operand(fmt, n), pw.constant_operand(fmt, code, n)), fmt
+    # decoded through the oracle's format tables: the values the closed forms of the GPU tests use
+    for fmt, ofmt in ((pw.F16, orc.FMT_F16), (pw.BF16, orc.FMT_BF16), (pw.E4M3, orc.FMT_E4M3), (pw.E5M2, orc.FMT_E5M2),
+                      (pw.E2M3, orc.FMT_E2M3), (pw.E3M2, orc.FMT_E3M2), (pw.E2M1, orc.FMT_E2M1)):
+        dt = np.uint16 if ofmt in (orc.FMT_F16, orc.FMT_BF16) else np.uint8
+        assert orc.decode(ofmt, np.array([pw.REFERENCE_CODE[fmt]], dtype=dt))[0] == pw.REFERENCE_VALUE[fmt], fmt
+    a, b = tmp_path / "seeded.xml", tmp_path / "reference.xml"
+    assert run_cli("--xml-file", str(a)).returncode == 0
+    assert run_cli("--reference-operands", "--xml-file", str(b)).returncode == 0
+    rows = lambda p: [(c, t, u, [(m, s) for m, s, _ in ms]) for c, t, u, ms in parse_xml(p)[1]]
+    assert rows(a) == rows(b)
+    assert "--reference-operands" in subprocess.run([CLI, "--help"], capture_output=True, text=True).stdout
+
+
 # ---- the reference's own result files (tests/golden/reference_results_*.xml, copied as data from its results/) ----
 GOLDEN = os.path.join(ROOT, "tests", "golden")
 
