@@ -1,7 +1,7 @@
 // Hand-written MFMA GEMM:  C[M][N] = scale * A[M][K] . B[N][K]^T.  Both operands are K-contiguous
-// ("row-major A, column-major B").  Operand types: bf16, f16, fp8 (e4m3, or an e5m2 A against an e4m3 B)
-// with fp32 accumulation and a 16-bit C; int8 with an int32 C; fp32.  The tile walk, the LDS ring and the
-// persistent workgroups live in gemm_ring.h and are shared with gemm_mxfp4.hip.
+// ("row-major A, column-major B").  Operand types: bf16, f16, fp8 (e4m3, or an e5m2 A against an e4m3 B) and
+// block-scaled e2m1 (entry point and scale pre-pass in gemm_mxfp4.hip) with fp32 accumulation and a 16-bit C;
+// int8 with an int32 C; fp32.  The tile walk, the LDS ring and the persistent workgroups live in gemm_ring.h.
 //
 // Tiling.  One workgroup of 512 threads (8 waves, 2 per SIMD) owns a 256x256 tile
 // of C and walks K in steps of one 128-byte row segment (64 bf16 or 128 fp8
@@ -86,8 +86,8 @@ enum { kBf16 = 0, kF16 = 1, kI8 = 2, kScaledBf16 = 3 };
 // and, loads returning in order, with its 4 youngest loads (the A rows three slabs ahead) still
 // allowed in flight, its share of the next slab has landed.  In the first step of a tile that
 // wait was done at the end of the tile before, and the stores issued since must not count.
-#define MI355_STEP_BARRIER(first, lds_wait)                                                        \
-  asm volatile(lds_wait "s_cmp_lg_u32 %0, 0\n s_cbranch_scc1 1f\n s_waitcnt vmcnt(4)\n1:\n s_barrier"  \
+#define MI355_STEP_BARRIER(first, lds_wait, youngest)                                              \
+  asm volatile(lds_wait "s_cmp_lg_u32 %0, 0\n s_cbranch_scc1 1f\n s_waitcnt vmcnt(" youngest ")\n1:\n s_barrier"  \
                :: "s"(first) : "memory", "scc")
 
 // Between the last matrix instruction of a tile and the first read of its accumulators: the wait
@@ -167,7 +167,7 @@ __device__ __forceinline__ void store_tile(const f32x4v (&acc)[8][4], void *__re
 //        matrix pipe forwards the accumulator to the next instruction that names it, so the pair issues like
 //        two independent instructions, and an instruction that names its predecessor's accumulator costs less
 //        power than one that switches (see mfma_dense.hip), which is what bounds these kernels.
-enum { kOpE4m3 = 0, kOpE5m2 = 1, kOpBf16 = 2, kOpF16 = 3, kOpI8 = 4 };
+enum { kOpE4m3 = 0, kOpE5m2 = 1, kOpBf16 = 2, kOpF16 = 3, kOpI8 = 4, kOpMx = 5 };
 #define MI355_MFMA_SLOT(OP, acc, blo, bhi, alo, ahi)                                               \
   do {                                                                                             \
     if (OP == kOpE4m3 || OP == kOpE5m2) {                                                          \
@@ -189,6 +189,36 @@ enum { kOpE4m3 = 0, kOpE5m2 = 1, kOpBf16 = 2, kOpF16 = 3, kOpI8 = 4 };
     }                                                                                              \
   } while (0)
 
+// Block-scaled e2m1 (OCP MXFP4): the pair of a slot with the scale bytes of its two K halves.  A lane's 16-byte
+// chunk is the 32 codes of one scale block; byte (op_sel + 2 * op_sel_hi) of the scale register is used:
+// op_sel = K half, op_sel_hi = parity of the fragment (JB for B, IB for A), register = fragment / 2.
+#define MI355_MFMA_MX_PAIR(JB, IB, acc, blo, bhi, alo, ahi, sb, sa)                                \
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %5, %6 op_sel:[0,0,0] op_sel_hi:[" #JB "," #IB ",0] cbsz:4 blgp:4\n" \
+               "v_mfma_scale_f32_16x16x128_f8f6f4 %0, %3, %4, %0, %5, %6 op_sel:[1,1,0] op_sel_hi:[" #JB "," #IB ",0] cbsz:4 blgp:4"   \
+               : "+v"(acc) : "v"(blo), "v"(alo), "v"(bhi), "v"(ahi), "v"(sb), "v"(sa))
+#define MI355_PARITY_0 0
+#define MI355_PARITY_1 1
+#define MI355_PARITY_2 0
+#define MI355_PARITY_3 1
+#define MI355_PARITY_4 0
+#define MI355_PARITY_5 1
+#define MI355_PARITY_6 0
+#define MI355_PARITY_7 1
+#define MI355_MX_SLOT2(JB, IB, acc, blo, bhi, alo, ahi, sb, sa) MI355_MFMA_MX_PAIR(JB, IB, acc, blo, bhi, alo, ahi, sb, sa)
+#define MI355_MX_SLOT(i, j, acc, blo, bhi, alo, ahi, sb, sa) \
+  MI355_MX_SLOT2(MI355_PARITY_##j, MI355_PARITY_##i, acc, blo, bhi, alo, ahi, sb, sa)
+
+// The scale bytes of a wave, per lane: byte 2i+h of `sa` belongs to A fragment i, K half h (16 bytes for the
+// 8 fragments), byte 2j+h of `sb` to B fragment j (8 bytes).  They do not pass through LDS (it is full): a
+// pre-pass has written them in this order, and the step loads those of the next step with one instruction per
+// operand, the wave's oldest loads of the step.
+struct MxScales {
+  i32x4v sa, sa_n;
+  i32x2v sb, sb_n;
+  uint64_t sa_next, sb_next;   // uniform addresses of the next step's 1 KiB (A) and 512 bytes (B)
+  uint32_t off_a, off_b;       // this lane's offset there
+};
+
 // At most `n` LDS reads still outstanding (they return in order).
 #define MI355_WAIT_LGKM(n) asm volatile("s_waitcnt lgkmcnt(" #n ")" ::: "memory")
 
@@ -197,10 +227,29 @@ struct RingFrags {
 };
 
 template <int OP>
-__device__ __forceinline__ void gemm_ring_step(f32x4v (&acc)[8][4], RingFrags &f, const GemmWalk &w, uint32_t first) {
+__device__ __forceinline__ void gemm_ring_step(f32x4v (&acc)[8][4], RingFrags &f, const GemmWalk &w, uint32_t first,
+                                               MxScales &sc) {
   constexpr bool READS = true;
   const uint32_t a_hi = w.a_cur ^ 64u, b_hi = w.b_cur ^ 64u, an_hi = w.a_nxt ^ 64u, bn_hi = w.b_nxt ^ 64u;
-#define MM(i, j) MI355_MFMA_SLOT(OP, acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i])
+  if constexpr (OP == kOpMx) {
+    // this step's scale bytes were requested a step ago, ahead of that step's 8 loads into LDS (in the first
+    // step of a tile they were waited for at the end of the tile before, and the stores since must not count)
+    asm volatile("s_cmp_lg_u32 %2, 0\n s_cbranch_scc1 1f\n s_waitcnt vmcnt(8)\n1:" : "+v"(sc.sa_n), "+v"(sc.sb_n) : "s"(first) : "scc");
+    sc.sa = sc.sa_n;
+    sc.sb = sc.sb_n;
+    // ordinary vector moves; the matrix instruction that reads one as a scale must not issue right behind it
+    asm volatile("s_nop 7" : "+v"(sc.sa), "+v"(sc.sb));
+    // the next step's scale bytes: the wave's oldest loads of this step, a whole step to land
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(sc.sa_n) : "v"(sc.off_a), "s"(sc.sa_next) : "memory");
+    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(sc.sb_n) : "v"(sc.off_b), "s"(sc.sb_next) : "memory");
+  }
+#define MM(i, j)                                                                                   \
+  do {                                                                                             \
+    if constexpr (OP == kOpMx)                                                                     \
+      MI355_MX_SLOT(i, j, acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i], sc.sb[(j) / 2], sc.sa[(i) / 2]); \
+    else                                                                                           \
+      MI355_MFMA_SLOT(OP, acc[i][j], f.b_lo[j], f.b_hi[j], f.a_lo[i], f.a_hi[i]);                  \
+  } while (0)
 #define LDA(q) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)(q) * w.row8, w.dst_a + (q) * 1024u)
 #define LDB(q) MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(q) * w.row8, w.dst_b + (q) * 1024u)
 #define RD_A_NEXT(i, off)                                                                          \
@@ -222,7 +271,9 @@ __device__ __forceinline__ void gemm_ring_step(f32x4v (&acc)[8][4], RingFrags &f
   MM(4, 0); MM(4, 1);
   // every read of this step's slab has returned (its two slots are free); with the 4 A loads of the
   // last step still allowed in flight, this wave's share of the next slab has landed
-  MI355_STEP_BARRIER(first, "s_waitcnt lgkmcnt(0)\n");
+  // (block-scaled kind: the two scale loads of this step are younger still)
+  if constexpr (OP == kOpMx) MI355_STEP_BARRIER(first, "s_waitcnt lgkmcnt(0)\n", "6");
+  else MI355_STEP_BARRIER(first, "s_waitcnt lgkmcnt(0)\n", "4");
   MM(5, 0); LDB(0);
   MM(5, 1);
   MM(6, 0); LDB(1);
@@ -255,12 +306,43 @@ __device__ __forceinline__ void gemm_ring_step(f32x4v (&acc)[8][4], RingFrags &f
 template <int OP>
 __global__ void __launch_bounds__(kThreads)
 gemm_ring_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, void *__restrict__ C,
-                uint32_t N, uint32_t k_bytes, float scale, uint32_t tiles_m, uint32_t tiles_n) {
+                uint32_t N, uint32_t k_bytes, float scale, uint32_t tiles_m, uint32_t tiles_n,
+                const uint8_t *__restrict__ scales_a, const uint8_t *__restrict__ scales_b) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const uint32_t tid = threadIdx.x, lane = tid % 64;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const uint32_t wm = wave / 4, wn = wave % 4;
   const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
+
+  // block-scaled kind: the stream of lane-ordered scale bytes, one step ahead of the slab being multiplied
+  // (per block of 128 A rows / 64 B rows and step 1 KiB / 512 bytes, the steps of a block consecutive)
+  MxScales sc{};
+  const uint32_t steps_of_tile = k_bytes / kRowBytes;
+  uint32_t s_round = 0, s_left = steps_of_tile;
+  auto scales_of = [&](uint32_t rnd) {
+    uint32_t tm, tn;
+    tile_at(grid, rnd, tm, tn);
+    sc.sa_next = (uint64_t)(uintptr_t)(scales_a + (size_t)(tm * 2u + wm) * steps_of_tile * 1024u);
+    sc.sb_next = (uint64_t)(uintptr_t)(scales_b + (size_t)(tn * 4u + wn) * steps_of_tile * 512u);
+  };
+  auto next_scales = [&]() {
+    if (--s_left == 0u) {
+      s_round = s_round + 1u == grid.mine ? 0u : s_round + 1u;
+      scales_of(s_round);
+      s_left = steps_of_tile;
+    } else {
+      sc.sa_next += 1024;
+      sc.sb_next += 512;
+    }
+  };
+  if constexpr (OP == kOpMx) {   // the first step's scales go out first; the start of the ring waits for every load
+    sc.off_a = lane * 16u;
+    sc.off_b = lane * 8u;
+    scales_of(0);
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(sc.sa_n) : "v"(sc.off_a), "s"(sc.sa_next) : "memory");
+    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(sc.sb_n) : "v"(sc.off_b), "s"(sc.sb_next) : "memory");
+    next_scales();
+  }
 
   Ring ring;
   ring.start(A, B, k_bytes, (uint32_t)(uintptr_t)lds, wave, lane, grid);
@@ -290,14 +372,15 @@ gemm_ring_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
   // one loop over the steps of all tiles of the workgroup
   uint32_t round = 0, left = steps, first = 1;
   for (uint32_t g = grid.mine * steps; g > 0; g--) {
-    gemm_ring_step<OP>(acc, f, ring.w, first);
+    gemm_ring_step<OP>(acc, f, ring.w, first, sc);
     ring.advance();
+    if constexpr (OP == kOpMx) next_scales();
     first = 0;
     if (--left == 0) {
       MI355_END_OF_TILE(acc);
       uint32_t tm, tn;
       tile_at(grid, round, tm, tn);
-      store_tile<(OP == kOpBf16 ? kBf16 : OP == kOpF16 ? kF16 : OP == kOpI8 ? kI8 : kScaledBf16)>(
+      store_tile<(OP == kOpBf16 || OP == kOpMx ? kBf16 : OP == kOpF16 ? kF16 : OP == kOpI8 ? kI8 : kScaledBf16)>(
           acc, C, N, tm * kTile + wm * 128u + lane % 16u, tn * kTile + wn * 64u, lane, scale);
 #pragma unroll
       for (int i = 0; i < 8; i++)
@@ -342,7 +425,7 @@ __device__ __forceinline__ void f32_slot(f32x4v (&acc)[8][4], f32x4v (&fa0)[8], 
   }
   if constexpr (M == 7) {
     MI355_WAIT_FRAGS(fa1, fb1);
-    MI355_STEP_BARRIER(first, "");
+    MI355_STEP_BARRIER(first, "", "4");
   }
   if constexpr (M >= 16 && M < 80 && M % 16 == 0)
     MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)((M - 16) / 16) * w.row8, w.dst_b + ((M - 16) / 16) * 1024u);
@@ -425,12 +508,24 @@ int launch_ring(mi355_dev *dev, const char *what, const void *A, const void *B, 
   if (int rc = allow_full_lds(dev, &gemm_ring_kernel<OP>, kLdsRing0 + OP)) return rc;
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
   gemm_ring_kernel<OP><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
-      (const uint8_t *)A, (const uint8_t *)B, C, N, K * elem, scale, tiles_m, tiles_n);
+      (const uint8_t *)A, (const uint8_t *)B, C, N, K * elem, scale, tiles_m, tiles_n, nullptr, nullptr);
   MI355_LAUNCH_CHECK(dev, what);
   return MI355_OK;
 }
 
 }  // namespace
+
+// The block-scaled FP4 product on the ring kernel; the caller (gemm_mxfp4.hip) has checked the shapes and laid
+// the scale bytes out per lane: A in blocks of 128 rows (16 bytes per lane and step), B in blocks of 64 rows (8).
+int mi355_launch_gemm_mx_ring(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scales_a,
+                              const uint8_t *scales_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
+  if (int rc = allow_full_lds(dev, &gemm_ring_kernel<kOpMx>, kLdsRing0 + kOpMx)) return rc;
+  const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
+  gemm_ring_kernel<kOpMx><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
+      A, B, C, N, K / 2u, 1.0f, tiles_m, tiles_n, scales_a, scales_b);
+  MI355_LAUNCH_CHECK(dev, "gemm_mxfp4");
+  return MI355_OK;
+}
 
 extern "C" int mi355_gemm_bf16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C, uint32_t M,
                                uint32_t N, uint32_t K) {

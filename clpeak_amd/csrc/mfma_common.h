@@ -41,6 +41,7 @@ typedef __bf16   bf16x8v  __attribute__((ext_vector_type(8)));
 typedef __bf16   bf16x16v __attribute__((ext_vector_type(16)));
 typedef float    f32x4v  __attribute__((ext_vector_type(4)));
 typedef float    f32x16v __attribute__((ext_vector_type(16)));
+typedef int      i32x2v  __attribute__((ext_vector_type(2)));
 typedef int      i32x4v  __attribute__((ext_vector_type(4)));
 typedef int      i32x8v  __attribute__((ext_vector_type(8)));
 typedef int      i32x16v __attribute__((ext_vector_type(16)));

@@ -97,42 +97,27 @@ def test_peak_loops_do_not_spill(tmp_path, source):
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
-def test_gemm_mxfp4_keeps_asynchronous_results_out_of_scratch(tmp_path):
-    """One wave per SIMD: 256 accumulation registers for the 64 tiles and the vector registers for fragments
-    and scales.  Nothing may spill, least of all inside the loop: the fragment and scale registers are written
-    asynchronously by the loads."""
-    asm = device_asm(tmp_path, "gemm_mxfp4.hip")
+def test_gemm_mxfp4_instantiation_of_the_ring_kernel(tmp_path):
+    """The block-scaled kind adds 12 scale registers (this step's and the next step's, written asynchronously by
+    loads) to the 128 accumulators and 96 fragment registers: it must still fit 256 without a spill."""
+    asm = device_asm(tmp_path, "gemm.hip")
     meta = kernel_metadata(asm)
-    name = next(k for k in meta if "gemm_mxfp4_kernel" in k)
+    name = next(k for k in meta if "gemm_ring_kernelILi5E" in k)
     m = meta[name]
-    assert m["agpr_count"] == 256 and m["vgpr_count"] <= 512, m
+    assert m["vgpr_spill_count"] == 0 and m["private_segment_fixed_size"] == 0 and m["vgpr_count"] <= 256, m
     body = kernel_body(asm, name)
-    # two instances of the 128-instruction step: the first step of a tile (its first K half starts the
-    # accumulators from zero) and every other step
-    assert body.count("v_mfma_scale_f32_16x16x128_f8f6f4") == 256
-    assert len(re.findall(r"v_mfma_scale_f32_16x16x128_f8f6f4 a\[\d+:\d+\], v\[\d+:\d+\], v\[\d+:\d+\], 0,", body)) == 64
-    assert body.count("v_cvt_pk_bf16_f32") == 128 and body.count("v_permlane16_swap_b32") == 64
-    # a lane-index value or two may spill around the loops; no scratch traffic inside a step (between two
-    # matrix instructions that are close together), where fragment and scale registers are still being written
-    assert m["vgpr_spill_count"] <= 4, m
-    lines = body.split("\n")
-    mfma = [n for n, l in enumerate(lines) if "v_mfma_scale" in l]
-    for n, l in enumerate(lines):
-        if "scratch_" in l:
-            before = max([x for x in mfma if x < n], default=None)
-            after = min([x for x in mfma if x > n], default=None)
-            assert before is None or after is None or after - before > 60, (n, l)
-    # and none in the innermost loop (the steps of a tile after the first)
-    labels = {l.split(":")[0]: n for n, l in enumerate(lines) if l.startswith(".LBB")}
-    loops = []
-    for n, l in enumerate(lines):
-        mt = re.search(r"s_cbranch_\w+ (\.LBB\w+)", l)
-        if mt and mt.group(1) in labels and labels[mt.group(1)] < n:
-            loops.append((labels[mt.group(1)], n))
-    inner = [(a, b) for a, b in loops if not any(a < c and d < b for c, d in loops)]
-    assert inner and any(sum("v_mfma_scale" in x for x in lines[a:b]) == 128 for a, b in inner)
-    for a, b in inner:
-        assert not any("scratch_" in x for x in lines[a:b]), (a, b)
+    insn = "v_mfma_scale_f32_16x16x128_f8f6f4"
+    assert body.count(insn) == 64 and body.count("cbsz:4 blgp:4") == 64
+    # a slot is its two K halves back to back on one accumulator, scale byte picked by op_sel
+    ops = re.findall(insn + r" (v\[\d+:\d+\]), .* op_sel:\[(\d),(\d),0\]", body)
+    assert len(ops) == 64
+    assert all(ops[2 * k][0] == ops[2 * k + 1][0] and ops[2 * k][1:] == ("0", "0") and ops[2 * k + 1][1:] == ("1", "1") for k in range(32))
+    # per step: one 16-byte load of A scales and one 8-byte load of B scales (+ the same two before the loop)
+    assert len(re.findall(r"global_load_dwordx4 v\[", body)) == 2 and len(re.findall(r"global_load_dwordx2 v\[", body)) == 2
+    assert body.count("v_cvt_pk_bf16_f32") == 64 and "ds_write" not in body
+    # the pre-pass and the entry point live in gemm_mxfp4.hip
+    meta = kernel_metadata(device_asm(tmp_path, "gemm_mxfp4.hip"))
+    assert any("mx_scale_layout_kernel" in k for k in meta)
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
