@@ -20,32 +20,49 @@
 
 namespace {
 
-// Pre-pass: scales from row-major [rows][k32] to the per-lane order the main loop loads, both operands
-// in one launch.  One wave per (block of rows, K step): blocks of 128 rows of A (8 fragments of 16 rows, 16
-// bytes per lane), blocks of 64 rows of B (4 fragments, 8 bytes per lane); lane (r,g) gathers its bytes and
-// stores them as one word.
+// Pre-pass: scales from row-major [rows][k32] to the per-lane order the main loop loads, both operands in one
+// launch.  One workgroup per (block of rows, 16 K steps): blocks of 128 rows of A (8 fragments of 16 rows, 16
+// bytes per lane and step), blocks of 64 rows of B (4 fragments, 8 bytes).  16 steps are 128 scale bytes of a
+// row, one cache line: the rows are read once, 8 bytes per thread and fully coalesced, into LDS (row stride 136
+// bytes, so that the 16 rows of a fragment fall into 16 different banks), and each wave then builds the words
+// of every fourth step from byte reads of LDS.  (Gathering the bytes straight from global memory, two per row
+// and lane, took 9.5 us per call at 8192^3, 4 % of the product.)
+constexpr uint32_t kLayoutSteps = 16, kLayoutStride = 136;
+
 __global__ void __launch_bounds__(256)
 mx_scale_layout_kernel(const uint8_t *__restrict__ SA, const uint8_t *__restrict__ SB, uint8_t *__restrict__ out_a,
-                       uint8_t *__restrict__ out_b, uint32_t k32, uint32_t steps, uint32_t units_a, uint32_t units_b) {
-  uint32_t unit = blockIdx.x * (blockDim.x / 64u) + threadIdx.x / 64u;
-  const uint32_t lane = threadIdx.x % 64u;
-  if (unit >= units_a + units_b) return;
+                       uint8_t *__restrict__ out_b, uint32_t k32, uint32_t steps, uint32_t groups_a, uint32_t groups_b) {
+  __shared__ __attribute__((aligned(16))) uint8_t rows[128 * kLayoutStride];
+  const uint32_t chunks = (steps + kLayoutSteps - 1) / kLayoutSteps;   // groups of 16 steps per block of rows
+  uint32_t grp = blockIdx.x;
+  if (grp >= groups_a + groups_b) return;
   const uint8_t *S = SA;
   uint8_t *out = out_a;
   uint32_t frags = 8;
-  if (unit >= units_a) { unit -= units_a; S = SB; out = out_b; frags = 4; }
-  const uint32_t rb = unit / steps, s = unit % steps, r = lane % 16u, g = lane / 16u;
-  uint32_t word[4] = {0, 0, 0, 0};
-#pragma unroll
-  for (uint32_t i = 0; i < 8; i++) {
-    if (i >= frags) break;
-    const uint8_t *row = S + (size_t)(rb * 16u * frags + 16u * i + r) * k32 + 8u * s + g;
-    const uint32_t pair = (uint32_t)row[0] | ((uint32_t)row[4] << 8);
-    if (i % 2 == 0) word[i / 2] = pair;
-    else word[i / 2] |= pair << 16;
+  if (grp >= groups_a) { grp -= groups_a; S = SB; out = out_b; frags = 4; }
+  const uint32_t rb = grp / chunks, s0 = (grp % chunks) * kLayoutSteps;
+  const uint32_t ns = steps - s0 < kLayoutSteps ? steps - s0 : kLayoutSteps, nrows = 16u * frags;
+  for (uint32_t u = threadIdx.x; u < nrows * ns; u += blockDim.x) {
+    const uint32_t row = u / ns, st = u % ns;
+    *reinterpret_cast<uint2 *>(rows + row * kLayoutStride + st * 8u) =
+        *reinterpret_cast<const uint2 *>(S + (size_t)(rb * nrows + row) * k32 + (size_t)(s0 + st) * 8u);
   }
-  if (frags == 8) *reinterpret_cast<uint4 *>(out + ((size_t)unit * 64u + lane) * 16u) = make_uint4(word[0], word[1], word[2], word[3]);
-  else *reinterpret_cast<uint2 *>(out + ((size_t)unit * 64u + lane) * 8u) = make_uint2(word[0], word[1]);
+  __syncthreads();
+  const uint32_t wave = threadIdx.x / 64u, lane = threadIdx.x % 64u, r = lane % 16u, g = lane / 16u;
+  for (uint32_t st = wave; st < ns; st += blockDim.x / 64u) {
+    uint32_t word[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (uint32_t i = 0; i < 8; i++) {
+      if (i >= frags) break;
+      const uint8_t *p = rows + (16u * i + r) * kLayoutStride + st * 8u + g;
+      const uint32_t pair = (uint32_t)p[0] | ((uint32_t)p[4] << 8);   // K halves 0 and 1 of fragment i
+      if (i % 2 == 0) word[i / 2] = pair;
+      else word[i / 2] |= pair << 16;
+    }
+    const size_t unit = (size_t)rb * steps + s0 + st;
+    if (frags == 8) *reinterpret_cast<uint4 *>(out + (unit * 64u + lane) * 16u) = make_uint4(word[0], word[1], word[2], word[3]);
+    else *reinterpret_cast<uint2 *>(out + (unit * 64u + lane) * 8u) = make_uint2(word[0], word[1]);
+  }
 }
 
 }  // namespace
@@ -58,6 +75,7 @@ extern "C" int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t 
   MI355_REQUIRE(dev, M % kTile == 0 && N % kTile == 0, "gemm_mxfp4: M (%u) and N (%u) must be multiples of 256", M, N);
   MI355_REQUIRE(dev, K % 256 == 0, "gemm_mxfp4: K (%u) must be a multiple of 256", K);
   MI355_REQUIRE(dev, (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) == 0, "gemm_mxfp4: buffers must be 16-byte aligned");
+  MI355_REQUIRE(dev, (((uintptr_t)scale_a | (uintptr_t)scale_b) & 7u) == 0, "gemm_mxfp4: scale arrays must be 8-byte aligned");
   // lane-ordered copies of the scales live in a scratch buffer the handle keeps (same size as the scales)
   const uint32_t k32 = K / 32u, steps = K / 256u;
   const size_t sa_bytes = (size_t)M * k32, sb_bytes = (size_t)N * k32;
@@ -72,8 +90,9 @@ extern "C" int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t 
     dev->mx_scratch_bytes = sa_bytes + sb_bytes;
   }
   uint8_t *sal = static_cast<uint8_t *>(dev->mx_scratch), *sbl = sal + sa_bytes;
-  const uint32_t units_a = M / 128u * steps, units_b = N / 64u * steps;
-  mx_scale_layout_kernel<<<(units_a + units_b + 3) / 4, 256, 0, dev->stream>>>(scale_a, scale_b, sal, sbl, k32, steps, units_a, units_b);
+  const uint32_t chunks = (steps + kLayoutSteps - 1) / kLayoutSteps;
+  const uint32_t groups_a = M / 128u * chunks, groups_b = N / 64u * chunks;
+  mx_scale_layout_kernel<<<groups_a + groups_b, 256, 0, dev->stream>>>(scale_a, scale_b, sal, sbl, k32, steps, groups_a, groups_b);
   MI355_LAUNCH_CHECK(dev, "mx_scale_layout");
   return mi355_launch_gemm_mx_ring(dev, A, B, sal, sbl, C, M, N, K);
 }

@@ -275,6 +275,7 @@ int mi355_gemm_f64(mi355_dev *dev, const double *A, const double *B, double *C,
  *          B[N][K/2] hold e2m1 codes two per byte (low nibble = even k), K contiguous;
  *          scale_a[M][K/32], scale_b[N][K/32] hold E8M0 bytes (value 2^(byte-127)).
  *          C[m][n] = sum_k A[m][k]*2^sa[m][k/32] * B[n][k]*2^sb[n][k/32].  K a multiple of 256.
+ *          A, B, C 16-byte aligned, the scale arrays 8-byte aligned.
  *          Each call first rewrites the scales into the order the kernel loads them (one small
  *          launch, part of the timed work); the copy lives in a scratch buffer of the same size
  *          that the handle allocates on the first call and on growth, and frees in mi355_close. */
