@@ -22,6 +22,10 @@
  * tests/test_oracle_*.py (known-answer vectors of SplitMix64, numpy/torch
  * conversions of every narrow format, closed forms of the affine recurrence, brute
  * force on small matrices).
+ * Parity unpinned against the reference's own numbers: orc_gemm_tile / orc_gemm_tile2 stand in for the
+ * rocBLAS / hipBLASLt calls of src/rocm/rocblas.cpp:246-263 and src/rocm/hipblaslt_gemm.cpp:330-400, libraries
+ * that are not part of the reference tree and whose results it never reads back; these two functions are
+ * pinned only by numpy float64 products and exact special cases (tests/test_oracle_kernels.py).
  *
  * Everything is plain C, no fast-math, no contraction: build with oracle/Makefile.
  */
