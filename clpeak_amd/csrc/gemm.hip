@@ -145,7 +145,7 @@ __device__ __forceinline__ void store_tile(const f32x4v (&acc)[8][4], void *__re
     }
 }
 
-// ---- the step of the 8-bit and 16-bit kinds ------------------------------------------------------------
+// ---- the step of the 4-, 8- and 16-bit kinds -----------------------------------------------------------
 // A slab of 128 bytes per row is one K=128 fp8 instruction per 16x16 tile, or two instructions of the
 // 16-bit / int8 kinds.  A lane's operand bytes are the two 16-byte chunks g and g+4 of its row (g = lane/16),
 // which in the swizzled layout are the addresses x and x^64: two ds_read_b128 fill the low and the high half
@@ -167,6 +167,9 @@ __device__ __forceinline__ void store_tile(const f32x4v (&acc)[8][4], void *__re
 //        matrix pipe forwards the accumulator to the next instruction that names it, so the pair issues like
 //        two independent instructions, and an instruction that names its predecessor's accumulator costs less
 //        power than one that switches (see mfma_dense.hip), which is what bounds these kernels.
+//   block-scaled e2m1: likewise two K=128 instructions (a 16-byte chunk is 32 codes, one scale block), each
+//        with the scale bytes of its blocks; the wave's scale bytes of the next step are requested at the top
+//        of the step, ahead of its 8 loads into LDS, and waited for at the top of the next.
 enum { kOpE4m3 = 0, kOpE5m2 = 1, kOpBf16 = 2, kOpF16 = 3, kOpI8 = 4, kOpMx = 5 };
 #define MI355_MFMA_SLOT(OP, acc, blo, bhi, alo, ahi)                                               \
   do {                                                                                             \
