@@ -94,6 +94,19 @@ def test_mfma_dense_full_launch_sampled(dev, kind, one_set):
     _check(got, ref, ab, is_int, wl.DENSE[kind]["name"], 4096)
 
 
+@pytest.mark.parametrize("seed,waves,iters", [(1, 4, 33), (0xDEADBEEF, 12, 95)])
+@pytest.mark.parametrize("one_set", [False, True])
+def test_other_seeds_launch_sizes_and_mixed_loop_trips(dev, seed, waves, iters, one_set):
+    """Iteration counts that take both loops of a kernel (runs of 32, then single instructions), wave counts
+    that are not a power of two, seeds other than the configured one: every dense and sparse kind."""
+    for kind in sorted(wl.DENSE):
+        got, ref, ab, is_int = _run_dense(dev, kind, waves, iters, seed=seed, one_set=one_set)
+        _check(got, ref, ab, is_int, (wl.DENSE[kind]["name"], seed, waves, iters), iters)
+    for kind in sorted(wl.SPARSE):
+        got, ref, ab, is_int = _run_sparse(dev, kind, waves, iters, seed=seed, one_set=one_set)
+        _check(got, ref, ab, is_int, (wl.SPARSE[kind]["name"], seed, waves, iters), iters)
+
+
 def test_mfma_int8_linearity(dev):
     """Size-independent property: n iterations = n x one iteration (exact in int32)."""
     g1, _, _, _ = _run_dense(dev, capi.MFMA_I8_16x16x64, 64, 1)
