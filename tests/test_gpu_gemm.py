@@ -289,8 +289,10 @@ def test_fill_bytes_bit_exact(dev):
     buf.free()
 
 
-@pytest.mark.parametrize("steps", [1, 2, 3, 4, 5, 9])
+@pytest.mark.parametrize("steps", [1, 2, 3, 4, 5, 9, 16, 17, 31])
 def test_gemm_mxfp4_short_walks(dev, steps):
+    """16, 17 and 31 steps: the scale pre-pass works on groups of 16 steps (one full group, a full group and a
+    single step, a full group and one that lacks a step)."""
     _check_mx(dev, 256, 256, steps * 256, [(0, 0), (0, 128), (128, 0), (128, 128)])
 
 
