@@ -4,8 +4,9 @@
 // CU: a 128x128 tile needs 4096 cycles of the matrix pipe per 16 doubles of K and 32 KiB of operands,
 // a sixteenth of the memory rate of the 16-bit GEMM.  So this kernel is the small sibling of gemm.hip:
 // 128x128 tiles, 4 waves of 64x64 (16 accumulator tiles of 4 doubles per lane = 128 registers), two LDS
-// buffers of 32 KiB per workgroup, two workgroups per CU, one barrier per step, and the loads of the
-// next slab in flight under the whole step.  It shares the LDS layout with its siblings (rows of 128
+// buffers of 32 KiB per workgroup, two workgroups per CU, one barrier per step (in its middle, between the
+// two K halves, so that every LDS read lands under 32 matrix instructions), and the loads of the next slab
+// in flight for a whole step.  It shares the LDS layout with its siblings (rows of 128
 // bytes, chunk c of row r at position c ^ (r & 7), global memory straight into LDS).
 //
 // A lane's 16-byte fragment read is chunk lane/16 (+4 for the second K half) of its row, two doubles;
@@ -33,6 +34,9 @@ typedef double f64x4v __attribute__((ext_vector_type(4)));
   asm volatile("ds_read_b128 %0, %1 offset:" #off : "=v"(dst) : "v"(addr))
 #define MI355_WAIT_FRAGS64(fa, fb)                                                                 \
   asm volatile("s_waitcnt lgkmcnt(0)"                                                              \
+               : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]))
+#define MI355_WAIT_FRAGS64_BUT8(fa, fb)                                                            \
+  asm volatile("s_waitcnt lgkmcnt(8)"                                                              \
                : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]))
 #define MI355_READ_FRAGS64(fa, fb, a_addr, b_addr)                                                 \
   MI355_DS_READ64(fb[0], b_addr, 0); MI355_DS_READ64(fb[1], b_addr, 2048);                         \
@@ -90,27 +94,37 @@ gemm_f64_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, do
     for (int j = 0; j < 4; j++) acc[i][j] = (f64x4v){0.0, 0.0, 0.0, 0.0};
   f64x2v fa0[4], fb0[4], fa1[4], fb1[4];
 
+  // Two fragment sets, one per K half of a slab, refilled while the other is being multiplied: the reads of
+  // the second half go out at the top of a step and land under the 32 instructions of the first half; in the
+  // middle of the step this wave's loads of the next slab have landed and, after the barrier, everybody's, and
+  // everybody has read all of this slab: its buffer takes the slab after the next, and the first half of the
+  // next slab is read under the 32 instructions of the second half.
   const uint32_t steps = k_bytes / kRowBytes;
   fetch(0);
   asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
+  if (steps > 1) fetch(1);
+  MI355_READ_FRAGS64(fa0, fb0, lane_a, lane_b);
   for (uint32_t s = 0; s < steps; s++) {
-    const uint32_t cur = (s & 1u) * 2u * kSlab64;
-    if (s + 1 < steps) fetch((s + 1) & 1u);   // lands in the buffer every wave left at the last barrier
-    const uint32_t a0 = lane_a + cur, b0 = lane_b + cur;
-    MI355_READ_FRAGS64(fa0, fb0, a0, b0);
-    MI355_READ_FRAGS64(fa1, fb1, a0 ^ 64u, b0 ^ 64u);
-    MI355_WAIT_FRAGS64(fa0, fb0);   // all 16 reads (they return in order; the second set rides along)
-    MI355_WAIT_FRAGS64(fa1, fb1);
+    const uint32_t cur = (s & 1u) * 2u * kSlab64, nxt = cur ^ (2u * kSlab64);
+    const uint32_t a1 = (lane_a + cur) ^ 64u, b1 = (lane_b + cur) ^ 64u;
+    MI355_READ_FRAGS64(fa1, fb1, a1, b1);
+    MI355_WAIT_FRAGS64_BUT8(fa0, fb0);   // reads return in order: the 8 just issued may still be in flight
     mfma_sweep(acc, fa0, fb0);
-    mfma_sweep(acc, fa1, fb1);
-    // the next slab has landed (own loads), and after the barrier everybody's; this slab's buffer is free.
-    // The accumulators ride along as operands so that the step's matrix instructions stay ahead of the wait:
-    // the loads are meant to fly under them.
-    asm volatile("s_waitcnt vmcnt(0)\n s_barrier"
+    // The accumulators ride along as operands so that the first half's matrix instructions stay ahead of the
+    // waits (the reads and the loads are meant to fly under them), the second fragment set so that none of
+    // the second half's can be placed before them.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier"
                  : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]), "+v"(acc[1][1]),
                    "+v"(acc[1][2]), "+v"(acc[1][3]), "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[2][2]), "+v"(acc[2][3]),
-                   "+v"(acc[3][0]), "+v"(acc[3][1]), "+v"(acc[3][2]), "+v"(acc[3][3])
+                   "+v"(acc[3][0]), "+v"(acc[3][1]), "+v"(acc[3][2]), "+v"(acc[3][3]),
+                   "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fa1[2]), "+v"(fa1[3]), "+v"(fb1[0]), "+v"(fb1[1]), "+v"(fb1[2]), "+v"(fb1[3])
                  :: "memory");
+    if (s + 2 < steps) fetch(s & 1u);
+    if (s + 1 < steps) {
+      const uint32_t a0 = lane_a + nxt, b0 = lane_b + nxt;
+      MI355_READ_FRAGS64(fa0, fb0, a0, b0);
+    }
+    mfma_sweep(acc, fa1, fb1);
   }
 
   const uint32_t row0 = tm * kTile64 + wm * 64u + lane % 16u, col0 = tn * kTile64 + wn * 64u + 4u * (lane / 16u);

@@ -123,7 +123,8 @@ def test_gemm_mxfp4_instantiation_of_the_ring_kernel(tmp_path):
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
 def test_gemm_fp32_and_fp64_kernels(tmp_path):
     """fp32: the ring kernel with four 16x16x4 instructions per 16-byte fragment read, 256 per step.
-    fp64: 64 instructions per step, two 32 KiB buffers (64 KiB static LDS, two workgroups per CU)."""
+    fp64: 64 instructions per step in two halves around the barrier, two 32 KiB buffers (64 KiB static LDS, two
+    workgroups per CU)."""
     asm = device_asm(tmp_path, "gemm.hip")
     meta = kernel_metadata(asm)
     name = next(k for k in meta if "gemm_f32_kernel" in k)
@@ -137,6 +138,14 @@ def test_gemm_fp32_and_fp64_kernels(tmp_path):
     assert meta[name]["group_segment_fixed_size"] == 65536
     body = kernel_body(asm, name)
     assert body.count("v_mfma_f64_16x16x4_f64") == 64 and "ds_write" not in body
-    # the step's matrix instructions stay ahead of the wait for the next slab's loads
-    loop = body[body.index("v_mfma_f64_16x16x4_f64"):]
-    assert loop.rindex("v_mfma_f64_16x16x4_f64") < loop.index("s_barrier")
+    # the order of a step: the 8 reads of the second K half, a counted wait, the 32 instructions of the first
+    # half ahead of the wait for everything and the barrier; then the next slab's loads and first-half reads
+    # under the 32 instructions of the second half
+    marks = []
+    for line in body.split("\n"):
+        t = line.strip()
+        marks.append("M" if t.startswith("v_mfma_f64") else "B" if t.startswith("s_barrier") else "r" if t.startswith("ds_read_b128")
+                     else "w" if t.startswith("s_waitcnt") else "L" if t.startswith("global_load_lds") else "")
+    order = "".join(marks)
+    assert "r" * 8 + "w" + "M" * 32 + "wB" in order, order
+    assert order.count("M" * 32) == 2 and order.count("B") == 2
