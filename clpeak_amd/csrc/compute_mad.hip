@@ -25,20 +25,10 @@ __device__ inline _Float16 bits_to_half(uint16_t h) {
   return r;
 }
 
-// The multiplier is the same for every lane, so the compiler keeps it in a scalar register; a vector
-// instruction with a scalar source runs at half the rate of one whose sources are all vector registers
-// (measured: 75.7 against 123 TFLOP/s for the same v_fmac_f32 stream; the packed half and the 64-bit integer
-// multiply-adds run at one rate either way).  This makes the value opaque and thereby a vector register.
-template <typename T>
-__device__ __forceinline__ T in_vector_register(T v) {
-  asm volatile("" : "+v"(v));
-  return v;
-}
-
 // ---- fp32 / fp64 -----------------------------------------------------------
 template <typename T, int W>
 __global__ void __launch_bounds__(256)
-mad_fp_kernel(uint64_t seed, T a, uint32_t steps, uint64_t n_items, T *__restrict__ out) {
+mad_fp_kernel(uint64_t seed, uint32_t steps, uint64_t n_items, T *__restrict__ out) {
   const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (item >= n_items) return;
   // W accumulators form one vector of the reference's source (float2, double4, ...).  A lane of this machine
@@ -46,14 +36,19 @@ mad_fp_kernel(uint64_t seed, T a, uint32_t steps, uint64_t n_items, T *__restric
   // is accumulator v*W + l.  (As ext_vector_type values the double2 / double4 chains picked up two register
   // copies per 32 multiply-adds from the allocator and ran 6 % below the scalar ones.)
   constexpr int NV = kAcc / W;
-  if constexpr (sizeof(T) == 4) a = in_vector_register(a);   // fp64 is faster with the scalar source: 72.9 against 66.9 TFLOP/s
+  // The multiplier of the workload is a compile-time constant because what a 32-bit vector instruction reads
+  // decides its rate.  As a kernel argument it sat in a scalar register (uniform over the lanes) and v_fma_f32
+  // ran at the 4-cycle rate, 75.7 TFLOP/s; from a vector register (three vector reads) 119; as the literal of
+  // v_fmamk_f32 (two vector reads) 127-130.  fp64 is the other way round: the constant lands in a scalar
+  // register pair, 72.9 TFLOP/s, against 66.9 from vector registers.
+  constexpr T a = (T)1.0001;
   T x0[kAcc], x[kAcc];
 #pragma unroll
   for (int i = 0; i < kAcc; i++) {
     x0[i] = (T)mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + i));
     x[i] = x0[i];
   }
-#pragma unroll 2
+#pragma unroll 8   // at one instruction per two cycles the counter and branch of a short trip show: +4 % over 2
   for (uint32_t s = 0; s < steps; s++) {
 #pragma unroll
     for (int v = 0; v < NV; v++)
@@ -119,33 +114,35 @@ mad_f16_kernel(uint64_t seed, uint16_t a_bits, uint32_t steps, uint64_t n_items,
 // kHalf: operands are IEEE half (maps to the mixed-precision FMA); otherwise bf16.
 template <bool kHalf>
 __global__ void __launch_bounds__(256)
-mad_mixed_kernel(uint64_t seed, uint16_t a_bits, uint32_t steps, uint64_t n_items, float *__restrict__ out) {
+mad_mixed_kernel(uint64_t seed, uint32_t steps, uint64_t n_items, float *__restrict__ out) {
   const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (item >= n_items) return;
   float acc[kAcc];
   float sum = 0.0f;
   if constexpr (kHalf) {
-    const _Float16 a = bits_to_half(a_bits);
+    // the multiplier is a compile-time constant so that it can be the literal of v_fmac_f32 (see mad_fp_kernel):
+    // 1 - 2^-10, the half below one (code 0x3bfe)
+    constexpr float a = 1.0f - 0.0009765625f;
     _Float16 xn[kAcc];
 #pragma unroll
     for (int j = 0; j < kAcc; j++) {
       xn[j] = bits_to_half(mi355_f32_to_f16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j))));
       acc[j] = (float)xn[j];
     }
-#pragma unroll 2
+#pragma unroll 8
     for (uint32_t s = 0; s < steps; s++) {
 #pragma unroll
-      for (int j = 0; j < kAcc; j++) acc[j] = __builtin_fmaf((float)xn[j], (float)a, acc[j]);
+      for (int j = 0; j < kAcc; j++) acc[j] = __builtin_fmaf((float)xn[j], a, acc[j]);
     }
   } else {
-    const float a = in_vector_register(mi355_bf16_to_f32(a_bits));
+    constexpr float a = 1.0f - 0.00390625f;   // 1 - 2^-8, the bf16 below one (code 0x3f7f)
     float xn[kAcc];
 #pragma unroll
     for (int j = 0; j < kAcc; j++) {
       xn[j] = mi355_bf16_to_f32(mi355_f32_to_bf16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j))));
       acc[j] = xn[j];
     }
-#pragma unroll 2
+#pragma unroll 8
     for (uint32_t s = 0; s < steps; s++) {
 #pragma unroll
       for (int j = 0; j < kAcc; j++) acc[j] = __builtin_fmaf(xn[j], a, acc[j]);
@@ -222,15 +219,15 @@ extern "C" int mi355_compute_mad(mi355_dev *dev, int kind, int width, uint64_t s
 #define BAD_WIDTH() return mi355_fail(dev, MI355_ERR_ARG, "compute_mad: width %d not valid for kind %d", width, kind)
   switch (kind) {
     case MI355_MAD_F32:
-      if (width == 1) mad_fp_kernel<float, 1><<<grid, block, 0, st>>>(seed, 1.0001f, steps, n_items, (float *)out);
-      else if (width == 2) mad_fp_kernel<float, 2><<<grid, block, 0, st>>>(seed, 1.0001f, steps, n_items, (float *)out);
-      else if (width == 4) mad_fp_kernel<float, 4><<<grid, block, 0, st>>>(seed, 1.0001f, steps, n_items, (float *)out);
+      if (width == 1) mad_fp_kernel<float, 1><<<grid, block, 0, st>>>(seed, steps, n_items, (float *)out);
+      else if (width == 2) mad_fp_kernel<float, 2><<<grid, block, 0, st>>>(seed, steps, n_items, (float *)out);
+      else if (width == 4) mad_fp_kernel<float, 4><<<grid, block, 0, st>>>(seed, steps, n_items, (float *)out);
       else BAD_WIDTH();
       break;
     case MI355_MAD_F64:
-      if (width == 1) mad_fp_kernel<double, 1><<<grid, block, 0, st>>>(seed, 1.0001, steps, n_items, (double *)out);
-      else if (width == 2) mad_fp_kernel<double, 2><<<grid, block, 0, st>>>(seed, 1.0001, steps, n_items, (double *)out);
-      else if (width == 4) mad_fp_kernel<double, 4><<<grid, block, 0, st>>>(seed, 1.0001, steps, n_items, (double *)out);
+      if (width == 1) mad_fp_kernel<double, 1><<<grid, block, 0, st>>>(seed, steps, n_items, (double *)out);
+      else if (width == 2) mad_fp_kernel<double, 2><<<grid, block, 0, st>>>(seed, steps, n_items, (double *)out);
+      else if (width == 4) mad_fp_kernel<double, 4><<<grid, block, 0, st>>>(seed, steps, n_items, (double *)out);
       else BAD_WIDTH();
       break;
     case MI355_MAD_F16:  // a = 1 - 2^-10 (0x3bfe): 1.0001 itself rounds to 1.0 in half
@@ -240,11 +237,11 @@ extern "C" int mi355_compute_mad(mi355_dev *dev, int kind, int width, uint64_t s
       break;
     case MI355_MAD_MP:
       if (width != 1) BAD_WIDTH();
-      mad_mixed_kernel<true><<<grid, block, 0, st>>>(seed, 0x3bfe, steps, n_items, (float *)out);
+      mad_mixed_kernel<true><<<grid, block, 0, st>>>(seed, steps, n_items, (float *)out);
       break;
     case MI355_MAD_BF16:  // a = 1 - 2^-8 (0x3f7f)
       if (width != 1) BAD_WIDTH();
-      mad_mixed_kernel<false><<<grid, block, 0, st>>>(seed, 0x3f7f, steps, n_items, (float *)out);
+      mad_mixed_kernel<false><<<grid, block, 0, st>>>(seed, steps, n_items, (float *)out);
       break;
     case MI355_MAD_I32:
       if (width == 1) mad_i32_kernel<1><<<grid, block, 0, st>>>(seed, 3u, steps, n_items, (uint32_t *)out);
