@@ -17,7 +17,7 @@
 // that into "register r of group g is column 4g + r of C": 4 consecutive N elements per lane, 32 bytes,
 // 128 contiguous bytes per row and store instruction.  (SQ_LDS_BANK_CONFLICT reads 32 cycles per wave and
 // step in this kernel, 3 % of its cycles, with this row order and equally with a B-slab swizzle built for
-// it; the matrix pipe is 94 % busy either way, so the layout stays the one of the sibling kernels.)
+// it; the matrix pipe, 96 % busy, does not notice, so the layout stays the one of the sibling kernels.)
 #include "internal.h"
 #include "mfma_common.h"
 #include "gemm_ring.h"
