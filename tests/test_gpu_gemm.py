@@ -311,3 +311,67 @@ def test_gemm_mxfp4_workgroups_walk_several_tiles(dev, steps):
     assert (M // 256) * (N // 256) > dev.props.num_cus
     tiles = [(m + 128 * ((m // 256 + n // 256) % 2), n + 128 * ((m // 256) % 2)) for m in range(0, M, 256) for n in range(0, N, 256)]
     _check_mx(dev, M, N, K, tiles, whole_output_finite=True)
+
+
+# --- the reference's own GEMM inputs ---------------------------------------------------------------------
+def _bf16_bits_of(x):
+    """Nearest-even bf16 code of a float32 value that is finite (numpy only)."""
+    u = np.float32(x).view(np.uint32).astype(np.uint64)
+    return int(((u + 0x7fff + ((u >> 16) & 1)) >> 16) & 0xffff)
+
+
+@pytest.mark.parametrize("kind", ["fp32", "fp64", "fp16", "bf16", "int8", "fp8_e4m3", "fp8_e5m2", "mxf4_e2m1"])
+def test_gemm_on_the_reference_fills(dev, kind):
+    """The reference's GEMM tests run on buffers set to one byte: 0x3f for every type of its rocBLAS test
+    (src/rocm/rocblas.cpp:211-212), 0x38 under block scales of 0x7f in its hipBLASLt test
+    (src/rocm/hipblaslt_gemm.cpp:272-273, 417-418).  On those inputs every element of C is K x a x b rounded to
+    the output type, with a and b the value that byte pattern has in the operand type; for the narrow types the
+    fp32 accumulation is exact at this K, so the whole of C is compared bit for bit with that one number."""
+    M, N, K = 512, 768, 1024
+    ebytes = {"fp32": 4, "fp64": 8, "fp16": 2, "bf16": 2, "int8": 1, "fp8_e4m3": 1, "fp8_e5m2": 1, "mxf4_e2m1": 0.5}[kind]
+    obytes = {"fp32": 4, "fp64": 8, "int8": 4}.get(kind, 2)
+    byte = 0x3f if kind in ("fp32", "fp64", "fp16", "bf16", "int8") else 0x38
+    dA, dB, dC = dev.alloc(int(M * K * ebytes)), dev.alloc(int(N * K * ebytes)), dev.alloc(M * N * obytes)
+    dev.memset(dA, byte); dev.memset(dB, byte); dev.memset(dC, 0xff)
+    pattern = np.full(8, byte, dtype=np.uint8)
+    if kind == "fp32":
+        a = float(pattern.view(np.float32)[0])
+        dev.gemm_f32(dA, dB, dC, M, N, K)
+        got = dC.download(np.float32, M * N)
+        assert np.all(got == got[0]) and abs(float(got[0]) - K * a * a) <= 1e-5 * K * a * a, (got[0], K * a * a)
+    elif kind == "fp64":
+        a = float(pattern.view(np.float64)[0])
+        dev.gemm_f64(dA, dB, dC, M, N, K)
+        got = dC.download(np.float64, M * N)
+        assert np.all(got == got[0]) and abs(float(got[0]) - K * a * a) <= 1e-12 * K * a * a, (got[0], K * a * a)
+    elif kind == "int8":
+        dev.gemm_i8(dA, dB, dC, M, N, K)
+        assert np.all(dC.download(np.int32, M * N) == K * 63 * 63)
+    elif kind == "fp16":
+        a = float(pattern.view(np.float16)[0])                      # 1855/1024: K*a*a needs 22 bits, exact in fp32
+        dev.gemm_f16(dA, dB, dC, M, N, K)
+        want = np.float16(np.float32(K * a * a))
+        assert np.float32(K * a * a) == K * a * a
+        assert np.all(dC.download(np.uint16, M * N) == want.view(np.uint16)), want
+    else:
+        if kind == "bf16":
+            a = b = float((pattern.view(np.uint16)[:1].astype(np.uint32) << 16).view(np.float32)[0])   # 191/256
+            dev.gemm_bf16(dA, dB, dC, M, N, K)
+            total = K * a * b
+        elif kind == "fp8_e4m3":
+            dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1.0, 1.0)        # 0x38 is 1.0 as e4m3
+            total = K * 1.0
+        elif kind == "fp8_e5m2":
+            dev.gemm_fp8_e5m2(dA, dB, dC, M, N, K, 1.0, 1.0)        # ... and 0.5 as e5m2 (the A operand of this row)
+            total = K * 0.5
+        else:
+            dSA, dSB = dev.alloc(M * K // 32), dev.alloc(N * K // 32)
+            dev.memset(dSA, 0x7f); dev.memset(dSB, 0x7f)
+            dev.gemm_mxfp4(dA, dB, dSA, dSB, dC, M, N, K)
+            # byte 0x38: even k holds code 8 (-0), odd k code 3 (1.5); scales 2^0
+            total = (K // 2) * 1.5 * 1.5
+            dSA.free(); dSB.free()
+        assert np.float32(total) == total
+        assert np.all(dC.download(np.uint16, M * N) == _bf16_bits_of(total)), (kind, total)
+    for b in (dA, dB, dC):
+        b.free()
