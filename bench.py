@@ -3,7 +3,8 @@
 
     python bench.py --gpus 1 --steps K --warmup W
 
-Prints ONE JSON line.  A "step" is one launch of the headline kernel: the float4
+The LAST line of stdout is one compact JSON record (under 2000 bytes); the full record with every row
+goes to the rows file (--rows-file) and the rows are listed on stderr.  A "step" is one launch of the headline kernel: the float4
 streaming read-reduce over a 4 GiB fp32 buffer resident in HBM (the HBM configuration
 of the workload list).  `value` is its throughput in GB/s.  The same line carries
 
@@ -11,7 +12,8 @@ of the workload list).  `value` is its throughput in GB/s.  The same line carrie
                 the stream the kernel runs on;
   cpu_baseline  the reference's own DRAM read kernel (where its build exists) and the CPU oracle's kernels,
                 timed on this host with the reference's CPU discipline (bounded samples);
-  rows          every other kernel of the backend (float/float2 reads, MAD chains, launch
+  fracs         one fraction of datasheet peak per target kernel (taken from the rows below);
+  rows (file)   every other kernel of the backend (float/float2 reads, MAD chains, launch
                 latency, dense MFMA, 2:4 SMFMAC, GEMM, LDS, PCIe transfers) with its absolute figure, the
                 MI355X datasheet peak it is compared with and the fraction reached.
 
@@ -347,6 +349,8 @@ def main():
     ap.add_argument("--no-rows", action="store_true", help="headline kernel only")
     ap.add_argument("--quick", action="store_true", help="shorter time budget per extra row")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--rows-file", default=os.path.join(ROOT, "gpurun_out", "bench_rows.json"),
+                    help="where the full record (every row, every CPU figure) is written; '' to skip")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel over 1 GiB (20 launches): under rocprofv3 --pmc this "
                          "gives what FETCH_SIZE / WRITE_SIZE read for a transfer of known size")
@@ -403,7 +407,7 @@ def main():
     dev.close()
 
     achieved = n * 4 / kernel_us / 1e3
-    line = {
+    full = {
         "metric": "MFMA TFLOPS/TOPS per dtype (dense, 2:4) + HBM GB/s, as % of MI355X peak",
         "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -416,8 +420,79 @@ def main():
                      "kernel_us": round(kernel_us, 2), "algorithmic_bytes": n * 4},
         "cpu_baseline": None if args.no_cpu else cpu_baseline(),
         "rows": rows,
+        "rows_file": os.path.relpath(args.rows_file, ROOT) if args.rows_file else None,
     }
-    print(json.dumps(line))
+    emit(full, args.rows_file)
+
+
+def emit(full, rows_file):
+    """Write the whole record (every row, every CPU figure) to `rows_file`, list the rows on stderr, and
+    print the compact record as the LAST line of stdout."""
+    if rows_file:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(rows_file)), exist_ok=True)
+            with open(rows_file, "w") as f:
+                json.dump(full, f, indent=1)
+        except OSError as e:
+            sys.stderr.write(f"bench.py: could not write {rows_file}: {e}\n")
+    for r in full["rows"]:
+        frac = f"  {100 * r['frac']:5.1f} % of {r['peak']:g}" if "frac" in r else ""
+        clk = f"  {r['sclk_mhz']:.0f} MHz" if "sclk_mhz" in r else ""
+        sys.stderr.write(f"{r['test']:28s} {r['metric']:44s} {r['value']:12.2f} {r['unit']:6s} {r['us_per_launch']:10.2f} us{frac}{clk}\n")
+    sys.stderr.flush()
+    print(json.dumps(compact_line(full), separators=(",", ":")), flush=True)
+
+
+# One number per target of the workload list: (key in "fracs", test, metric).
+FRAC_KEYS = [("hbm_float", "global_memory_bandwidth", "float"), ("hbm_float2", "global_memory_bandwidth", "float2"),
+             ("mad_fp32", "single_precision_compute", "float4"), ("mad_fp64", "double_precision_compute", "double"),
+             ("mfma_fp16", "mfma_fp16", "mfma_fp16"), ("mfma_bf16", "mfma_bf16", "mfma_bf16"),
+             ("mfma_fp16_32x32x16", "mfma_fp16_32x32x16", "mfma_fp16_32x32x16"),
+             ("mfma_bf16_32x32x16", "mfma_bf16_32x32x16", "mfma_bf16_32x32x16"),
+             ("mfma_int8", "mfma_int8", "mfma_int8"), ("mfma_fp8", "mfma_fp8", "mfma_fp8"), ("mfma_bf8", "mfma_bf8", "mfma_bf8"),
+             ("mfma_mxfp6_e2m3", "mfma_mxfp6_e2m3", "mfma_mxfp6_e2m3"), ("mfma_mxfp6_e3m2", "mfma_mxfp6_e3m2", "mfma_mxfp6_e3m2"),
+             ("mfma_mxfp4", "mfma_mxfp4", "mfma_mxfp4"),
+             ("smfmac_fp16", "smfmac_fp16", "smfmac_fp16"), ("smfmac_bf16", "smfmac_bf16", "smfmac_bf16"),
+             ("smfmac_fp8", "smfmac_fp8", "smfmac_fp8"), ("smfmac_bf8", "smfmac_bf8", "smfmac_bf8"),
+             ("smfmac_int8", "smfmac_int8", "smfmac_int8"),
+             ("gemm_bf16_seeded", "rocblas-fp", "bf16"), ("gemm_fp16_seeded", "rocblas-fp", "fp16"),
+             ("gemm_fp32", "rocblas-fp", "fp32"), ("gemm_fp64", "rocblas-fp", "fp64"),
+             ("gemm_fp8_e4m3_seeded", "hipblaslt-fp8", "fp8_e4m3"), ("gemm_fp8_e5m2_seeded", "hipblaslt-fp8", "fp8_e5m2"),
+             ("gemm_mxfp4_seeded", "hipblaslt-fp8", "mxf4_e2m1"), ("gemm_int8_seeded", "rocblas-int", "int8"),
+             ("gemm_bf16_const", "rocblas-fp", "bf16 constant operands"),
+             ("lds_float4", "local_memory_bandwidth", "float4")]
+
+
+def compact_line(full):
+    """The record the driver reads: the contract's keys, the roofline of the headline kernel, the CPU
+    baseline's headline figures and one fraction of peak per target; kept under 2000 bytes (the full
+    record with every row is in the rows file)."""
+    line = {k: full[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better",
+                                 "scaling", "vs_baseline", "dtype", "data")}
+    line["config"] = {"workload": "HBM streaming read: float4 grid-stride read-reduce over a 4 GiB seeded fp32 buffer",
+                      "buffer_bytes": full["config"]["buffer_bytes"], "threads": full["config"]["threads"]}
+    line["roofline"] = full["roofline"]
+    cb = full.get("cpu_baseline")
+    if cb is not None:
+        c = {k: cb[k] for k in ("value", "unit", "cores", "kind")}
+        head = (cb.get("reference") or {}).get("global_memory_bandwidth read") or cb["port"]["global_memory_bandwidth float4"]
+        c["ST"], c["MT"] = head.get("ST"), head.get("MT")
+        c["sample"] = cb["sample"][:200]
+        line["cpu_baseline"] = c
+    else:
+        line["cpu_baseline"] = None
+    by_key = {(r["test"], r["metric"]): r for r in full["rows"]}
+    fracs = {}
+    for key, test, metric in FRAC_KEYS:
+        r = by_key.get((test, metric))
+        if r is not None and "frac" in r:
+            fracs[key] = round(r["frac"], 3)
+    line["fracs"] = fracs
+    lat = by_key.get(("kernel_launch_latency", "roundtrip"))
+    if lat is not None:
+        line["launch_roundtrip_us"] = lat["value"]
+    line["rows_file"] = full.get("rows_file")
+    return line
 
 
 # Workgroups per CU of the headline launch (256 threads each); one per CU measured best (a

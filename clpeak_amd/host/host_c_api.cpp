@@ -1,6 +1,7 @@
-// A few C entry points into the host layer so that tests can reach it with ctypes: the seeded
-// operand generator, pickIters, and a whole run against the stand-in device.
+// The auxiliary C entry points of libclpeak_host.so (include/clpeak_host.h): the seeded operand
+// generator, the calibration helpers, the result-file converter and the cancel flag.
 #include <cstring>
+#include "../../include/clpeak_host.h"
 #include <sstream>
 #include "mi355_peak.h"
 #include "results.h"

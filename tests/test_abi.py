@@ -27,6 +27,25 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
+def test_host_library_exports_every_declared_symbol():
+    """libclpeak_host.so: the embedding ABI (clpeak_ffi.h) and the auxiliary one (clpeak_host.h)."""
+    import ctypes as C
+    lib = C.CDLL(os.path.join(ROOT, "clpeak_amd", "libclpeak_host.so"))
+    exported = set()
+    for header, prefix, count in (("clpeak_ffi.h", "clpeak_", 6), ("clpeak_host.h", "clpeak_host_", 10)):
+        text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", header)).read(), flags=re.S)
+        names = sorted(set(re.findall(r"\b(%s[a-z0-9_]+)\s*\(" % prefix, text)))
+        assert len(names) == count, (header, names)
+        for name in names:
+            assert hasattr(lib, name), name
+        exported |= set(names)
+    # and nothing with the library's prefix is exported without being declared
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", lib._name], capture_output=True, text=True).stdout
+    for sym in re.findall(r" T (clpeak_[a-z0-9_]+)", out):
+        assert sym in exported, sym
+
+
 def test_every_entry_point_cites_the_reference():
     """Each declaration is preceded by a comment naming the reference code it replaces
     (or saying that it has no counterpart)."""

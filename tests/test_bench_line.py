@@ -1,0 +1,71 @@
+"""The record bench.py prints last must stay small enough for a reader that keeps only a short tail
+of stdout, and must carry the contract's keys.  No GPU: the formatter runs on a synthetic record of the
+size a full run produces."""
+import io
+import json
+import os
+import sys
+from contextlib import redirect_stderr, redirect_stdout
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+import bench  # noqa: E402
+
+
+def _synthetic_full(with_cpu=True):
+    rows = []
+    for _, test, metric in bench.FRAC_KEYS:
+        rows.append({"test": test, "metric": metric, "value": 123456.78, "unit": "tflops", "us_per_launch": 12345.67,
+                     "peak": 10100.0, "frac": 0.98765, "shape": "8192x8192x8192", "sclk_mhz": 2399.0})
+    # rows without a peak and rows the compact record leaves out
+    rows.append({"test": "kernel_launch_latency", "metric": "roundtrip", "value": 9.47, "unit": "us", "us_per_launch": 9.47})
+    for i in range(80):
+        rows.append({"test": f"mfma_kind{i}", "metric": f"mfma_kind{i} distinct operands per chain", "value": 1.0,
+                     "unit": "tflops", "us_per_launch": 1.0, "peak": 2500.0, "frac": 0.5})
+    cpu = None
+    if with_cpu:
+        fig = {"ST": 12345.67, "MT": 123456.78, "unit": "GB/s", "iters_ST": 10, "iters_MT": 100}
+        cpu = {"value": 516.12, "unit": "GB/s", "cores": 16, "kind": "reference", "pinned_workers": 16,
+               "sample": "x" * 600, "reference": {"isa": "avx512", "global_memory_bandwidth read": fig,
+                                                  "single_precision_compute float": fig},
+               "port": {"global_memory_bandwidth float4": fig, **{f"family {i}": fig for i in range(20)}}}
+    return {"metric": "MFMA TFLOPS/TOPS per dtype (dense, 2:4) + HBM GB/s, as % of MI355X peak",
+            "value": 7457.12, "unit": "GB/s", "n_gpus": 1, "steps": 300, "warmup": 100, "ms_per_step": 0.57612,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "w" * 200, "buffer_bytes": 1 << 32, "threads": 65536, "pct_of_peak": 93.21},
+            "roofline": {"bound": "hbm", "achieved": 7444.11, "peak": 8000.0, "unit": "GB/s", "frac": 0.9305,
+                         "traffic": 4295176192, "kernel_us": 576.95, "algorithmic_bytes": 1 << 32},
+            "cpu_baseline": cpu, "rows": rows, "rows_file": "some/dir/bench_rows.json"}
+
+
+def test_compact_line_is_small_and_complete():
+    full = _synthetic_full()
+    text = json.dumps(bench.compact_line(full), separators=(",", ":"))
+    assert len(text.encode()) < 2000, len(text)
+    line = json.loads(text)
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline", "fracs"):
+        assert key in line, key
+    assert line["config"]["workload"] and "model" not in line["config"]
+    for key in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel_us", "algorithmic_bytes"):
+        assert key in line["roofline"], key
+    for key in ("value", "unit", "cores", "kind", "sample", "ST", "MT"):
+        assert key in line["cpu_baseline"], key
+    for key in ("mfma_fp16", "mfma_bf16", "mfma_fp8", "mfma_mxfp4", "mfma_int8", "smfmac_fp16", "smfmac_int8",
+                "gemm_bf16_seeded"):
+        assert key in line["fracs"], key
+    assert line["launch_roundtrip_us"] == 9.47
+
+
+def test_emit_prints_the_compact_record_last(tmp_path):
+    full = _synthetic_full(with_cpu=False)
+    out, err = io.StringIO(), io.StringIO()
+    rows_file = tmp_path / "rows.json"
+    with redirect_stdout(out), redirect_stderr(err):
+        bench.emit(full, str(rows_file))
+    lines = out.getvalue().splitlines()
+    assert len(lines) == 1 and len(lines[-1].encode()) < 2000
+    assert json.loads(lines[-1])["cpu_baseline"] is None
+    # the full record, every row of it, is in the file; the rows are listed for a human on stderr
+    assert len(json.loads(rows_file.read_text())["rows"]) == len(full["rows"])
+    assert err.getvalue().count("\n") == len(full["rows"])
