@@ -407,3 +407,77 @@ def test_oracle_on_the_reference_constants_is_the_closed_form():
         out, _ = orc.smfmac(kind, Ac, np.full_like(meta, 0b0100), B, waves, iters, is_int=is_int)
         v = product_wl.REFERENCE_VALUE[s["fmt"]]
         assert np.all(out == iters * (s["K"] // 2) * v * v), (s["name"], out[:4])
+
+
+# ---- block-scaled FP4 GEMM tile and the float64 buffer total -----------------------
+# e2m1 values by code, written from the OCP Microscaling specification's table (sign bit 3).
+_E2M1 = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0])
+
+
+def _mx_dense(codes_packed, scales, rows, K):
+    """Decoded, scaled operand [rows][K] from packed nibbles (low nibble = even k) and E8M0 bytes."""
+    by = codes_packed.reshape(rows, K // 2)
+    codes = np.empty((rows, K), dtype=np.uint8)
+    codes[:, 0::2] = by & 15
+    codes[:, 1::2] = by >> 4
+    sc = np.exp2(scales.reshape(rows, K // 32).astype(np.float64) - 127.0)
+    return _E2M1[codes] * np.repeat(sc, 32, axis=1)
+
+
+def test_gemm_mx_tile_against_numpy_product():
+    """Non-square tile with offsets, asymmetric scales: every product and every scaled sum is exact in float64
+    (4-bit values, power-of-two scales within 2^-4..2^4, K = 96), so the comparison is for equality."""
+    rng = np.random.default_rng(11)
+    M, N, K = 48, 40, 96
+    A = rng.integers(0, 256, size=M * K // 2, dtype=np.uint8)
+    B = rng.integers(0, 256, size=N * K // 2, dtype=np.uint8)
+    SA = rng.integers(123, 132, size=M * K // 32, dtype=np.uint8)
+    SB = rng.integers(123, 128, size=N * K // 32, dtype=np.uint8)      # a different range from SA's
+    a, b = _mx_dense(A, SA, M, K), _mx_dense(B, SB, N, K)
+    m0, n0, tm, tn = 16, 8, 24, 32
+    got = orc.gemm_mx_tile(A, B, SA, SB, K, m0, n0, tm, tn)
+    assert np.array_equal(got, a[m0:m0 + tm] @ b[n0:n0 + tn].T)
+    # the whole matrix as one tile too
+    assert np.array_equal(orc.gemm_mx_tile(A, B, SA, SB, K, 0, 0, M, N), a @ b.T)
+
+
+def test_gemm_mx_tile_nibble_order_and_scale_index():
+    """Cases a swapped nibble order or a swapped scale index (row/block, or A's scales used for B) would fail."""
+    M = N = 2
+    K = 64
+    A = np.zeros(M * K // 2, dtype=np.uint8)
+    B = np.zeros(N * K // 2, dtype=np.uint8)
+    SA = np.full(M * K // 32, 127, dtype=np.uint8)
+    SB = np.full(N * K // 32, 127, dtype=np.uint8)
+    # A[0][k=0] = 1.0 (code 2, LOW nibble of byte 0), A[0][k=1] = 6.0 (code 7, HIGH nibble)
+    A[0] = 2 | (7 << 4)
+    # B[1][k=0] = 0.5 (code 1), B[1][k=1] = 0: with the nibbles swapped the product would pair 6.0 with 0.5
+    B[1 * K // 2] = 1
+    C = orc.gemm_mx_tile(A, B, SA, SB, K, 0, 0, M, N)
+    assert C[0, 1] == 0.5 and C[0, 0] == 0 and C[1, 0] == 0 and C[1, 1] == 0
+    # scale of A row 0, block 1 (k = 32..63) only: put a value there and scale that block alone by 2^3
+    A[:] = 0; B[:] = 0
+    A[0 * K // 2 + 32 // 2] = 2          # A[0][32] = 1.0
+    B[1 * K // 2 + 32 // 2] = 4          # B[1][32] = 2.0
+    SA[0 * 2 + 1] = 130                  # A row 0, block 1: 2^3
+    assert orc.gemm_mx_tile(A, B, SA, SB, K, 0, 0, M, N)[0, 1] == 16.0
+    SA[:] = 127
+    SA[1 * 2 + 0] = 130                  # row 1 block 0 instead (the transposed index): must not apply
+    assert orc.gemm_mx_tile(A, B, SA, SB, K, 0, 0, M, N)[0, 1] == 2.0
+    SA[:] = 127
+    SB[1 * 2 + 1] = 125                  # B row 1, block 1: 2^-2
+    assert orc.gemm_mx_tile(A, B, SA, SB, K, 0, 0, M, N)[0, 1] == 0.5
+    # an offset tile sees the same element at its shifted position
+    assert orc.gemm_mx_tile(A, B, SA, SB, K, 0, 1, 1, 1)[0, 0] == 0.5
+
+
+@pytest.mark.parametrize("n", [1, 1000003, (1 << 20) + 7])
+def test_sum_u01_against_numpy_float64(n):
+    """The float64 total of the bandwidth buffer.  Every element is a multiple of 2^-24 below 1, so the sum of
+    up to 2^29 of them is exact in float64 whatever the order: equality with numpy's sum, for lengths that no
+    thread count divides."""
+    seed, stream = 0x1234, wl.STREAM_BW
+    data = orc.fill_f32(n, seed, stream, 0)
+    assert orc.sum_u01(seed, stream, n) == float(data.astype(np.float64).sum())
+    # and it is a sum over elements 0..n-1 of that stream, not of another stream or another seed
+    assert orc.sum_u01(seed, stream + 1, n) != orc.sum_u01(seed, stream, n) or n == 0
