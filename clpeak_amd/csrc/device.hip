@@ -80,6 +80,12 @@ extern "C" int mi355_open(int ordinal, mi355_dev **out) {
     mi355_close(d);
     return code;
   }
+  // the one array of the library that lives in device memory from load to exit: its address on this device
+  if (int code = mi355_mx_resolve_static_scratch(d)) {
+    mi355_global_error() = d->last_error;
+    mi355_close(d);
+    return code;
+  }
   *out = d;
   return MI355_OK;
 }

@@ -65,34 +65,76 @@ mx_scale_layout_kernel(const uint8_t *__restrict__ SA, const uint8_t *__restrict
   }
 }
 
-}  // namespace
-
-extern "C" int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
-                                const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
-  MI355_ENTER(dev);
+// Shape and alignment checks shared by the two entry points.
+int check_mx_shapes(mi355_dev *dev, const void *A, const void *B, const void *scale_a, const void *scale_b, const void *C,
+                    uint32_t M, uint32_t N, uint32_t K) {
   MI355_REQUIRE(dev, A && B && C && scale_a && scale_b, "gemm_mxfp4: null buffer");
   MI355_REQUIRE(dev, M > 0 && N > 0 && K > 0, "gemm_mxfp4: empty problem");
   MI355_REQUIRE(dev, M % kTile == 0 && N % kTile == 0, "gemm_mxfp4: M (%u) and N (%u) must be multiples of 256", M, N);
   MI355_REQUIRE(dev, K % 256 == 0, "gemm_mxfp4: K (%u) must be a multiple of 256", K);
   MI355_REQUIRE(dev, (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) == 0, "gemm_mxfp4: buffers must be 16-byte aligned");
   MI355_REQUIRE(dev, (((uintptr_t)scale_a | (uintptr_t)scale_b) & 7u) == 0, "gemm_mxfp4: scale arrays must be 8-byte aligned");
-  // lane-ordered copies of the scales live in a scratch buffer the handle keeps (same size as the scales)
+  return MI355_OK;
+}
+
+// Pre-pass into `lane_scales` (M*K/32 bytes for A, then N*K/32 for B), then the product.  Both on the handle's stream.
+int run_mx(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a, const uint8_t *scale_b,
+           uint16_t *C, uint32_t M, uint32_t N, uint32_t K, uint8_t *lane_scales) {
   const uint32_t k32 = K / 32u, steps = K / 256u;
-  const size_t sa_bytes = (size_t)M * k32, sb_bytes = (size_t)N * k32;
-  if (dev->mx_scratch_bytes < sa_bytes + sb_bytes) {
-    MI355_HIP(dev, hipStreamSynchronize(dev->stream));
-    if (dev->mx_scratch) MI355_HIP(dev, hipFree(dev->mx_scratch));
-    dev->mx_scratch = nullptr;
-    dev->mx_scratch_bytes = 0;
-    const hipError_t e = hipMalloc(&dev->mx_scratch, sa_bytes + sb_bytes);
-    if (e != hipSuccess) return mi355_fail(dev, e == hipErrorOutOfMemory ? MI355_ERR_OOM : MI355_ERR_HIP,
-                                           "gemm_mxfp4: scratch of %zu bytes: %s", sa_bytes + sb_bytes, hipGetErrorString(e));
-    dev->mx_scratch_bytes = sa_bytes + sb_bytes;
-  }
-  uint8_t *sal = static_cast<uint8_t *>(dev->mx_scratch), *sbl = sal + sa_bytes;
+  uint8_t *sal = lane_scales, *sbl = sal + (size_t)M * k32;
   const uint32_t chunks = (steps + kLayoutSteps - 1) / kLayoutSteps;
   const uint32_t groups_a = M / 128u * chunks, groups_b = N / 64u * chunks;
   mx_scale_layout_kernel<<<groups_a + groups_b, 256, 0, dev->stream>>>(scale_a, scale_b, sal, sbl, k32, steps, groups_a, groups_b);
   MI355_LAUNCH_CHECK(dev, "mx_scale_layout");
   return mi355_launch_gemm_mx_ring(dev, A, B, sal, sbl, C, M, N, K);
+}
+
+}  // namespace
+
+// Scratch of the entry point that allocates nothing: the lane-ordered scales of one call.  4 MiB hold the
+// scales of the 8192^3 product (2 x 8192 x 8192 / 32 bytes).  Every GPU the library runs on holds its own copy
+// of this array, at its own address, until the process ends.
+constexpr size_t kStaticScaleBytes = 4u << 20;
+static __device__ __align__(256) uint8_t scratch[kStaticScaleBytes];
+
+// Called by mi355_open with the handle's device current: the device address of `scratch` on that device.  (In
+// host code the array's name is only a stand-in for the symbol; kernels and copies must be given this address.)
+int mi355_mx_resolve_static_scratch(mi355_dev *dev) {
+  void *ptr = nullptr;
+  MI355_HIP(dev, hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  if (!ptr) return mi355_fail(dev, MI355_ERR_HIP, "gemm_mxfp4: the static scratch array has no device address");
+  dev->mx_static_scratch = ptr;
+  return MI355_OK;
+}
+
+extern "C" int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
+                                const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
+  MI355_ENTER(dev);
+  if (int rc = check_mx_shapes(dev, A, B, scale_a, scale_b, C, M, N, K)) return rc;
+  // lane-ordered copies of the scales live in a scratch buffer the handle keeps (same size as the scales)
+  const size_t need = ((size_t)M + N) * (K / 32u);
+  if (dev->mx_scratch_bytes < need) {
+    MI355_HIP(dev, hipStreamSynchronize(dev->stream));
+    if (dev->mx_scratch) MI355_HIP(dev, hipFree(dev->mx_scratch));
+    dev->mx_scratch = nullptr;
+    dev->mx_scratch_bytes = 0;
+    const hipError_t e = hipMalloc(&dev->mx_scratch, need);
+    if (e != hipSuccess) return mi355_fail(dev, e == hipErrorOutOfMemory ? MI355_ERR_OOM : MI355_ERR_HIP,
+                                           "gemm_mxfp4: scratch of %zu bytes: %s", need, hipGetErrorString(e));
+    dev->mx_scratch_bytes = need;
+  }
+  return run_mx(dev, A, B, scale_a, scale_b, C, M, N, K, static_cast<uint8_t *>(dev->mx_scratch));
+}
+
+extern "C" int mi355_gemm_mxfp4_static(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
+                                       const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
+  MI355_ENTER(dev);
+  if (int rc = check_mx_shapes(dev, A, B, scale_a, scale_b, C, M, N, K)) return rc;
+  const size_t need = ((size_t)M + N) * (K / 32u);
+  MI355_REQUIRE(dev, need <= kStaticScaleBytes,
+                "gemm_mxfp4_static: (M + N) * K / 32 = %zu scale bytes exceed the static scratch of %zu bytes "
+                "(use mi355_gemm_mxfp4 for larger problems)", need, kStaticScaleBytes);
+  MI355_REQUIRE(dev, dev->mx_static_scratch != nullptr, "gemm_mxfp4_static: the static scratch was not resolved when the device was opened");
+  // The pre-pass overwrites every byte the product reads, so nothing of the previous call's contents has to be cleared.
+  return run_mx(dev, A, B, scale_a, scale_b, C, M, N, K, static_cast<uint8_t *>(dev->mx_static_scratch));
 }

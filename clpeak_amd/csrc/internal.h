@@ -16,6 +16,8 @@ struct mi355_dev {
   // scratch owned by the handle: scale bytes of the block-scaled GEMM laid out per lane (grown on demand)
   void        *mx_scratch = nullptr;
   size_t       mx_scratch_bytes = 0;
+  // device address, on this handle's device, of the static array behind mi355_gemm_mxfp4_static (set by mi355_open)
+  void        *mx_static_scratch = nullptr;
   // GEMM kernels that have been allowed the whole LDS of a CU on this device (one bit per kernel)
   uint32_t     full_lds_allowed = 0;
 };
@@ -24,6 +26,9 @@ struct mi355_dev {
 std::string &mi355_global_error();
 
 int mi355_fail(mi355_dev *dev, int code, const char *fmt, ...) __attribute__((format(printf, 3, 4)));
+
+// gemm_mxfp4.hip: look up the device address of its static scratch array (the handle's device is current).
+int mi355_mx_resolve_static_scratch(mi355_dev *dev);
 
 // Wrap a HIP runtime call: on failure record "<call>: <hip error>" and return MI355_ERR_HIP.
 #define MI355_HIP(dev, call)                                                            \

@@ -281,6 +281,17 @@ int mi355_gemm_f64(mi355_dev *dev, const double *A, const double *B, double *C,
  *          that the handle allocates on the first call and on growth, and frees in mi355_close. */
 int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
                      const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K);
+/*   The same product for callers that cannot allocate (code under HIP graph capture, tight serving
+ *          loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Identical
+ *          arguments, checks and result; the lane-ordered scales go into a 4 MiB array that lives in
+ *          the library's device image instead of a buffer of the handle, so the call performs no
+ *          allocation and frees nothing.  Limit: (M + N) * K / 32 <= 4 MiB (8192^3 just fits);
+ *          larger problems are refused with MI355_ERR_ARG and a message.  Every call on a GPU shares
+ *          that GPU's array: calls that overlap on one GPU (two handles, two threads) race; calls on
+ *          one handle are ordered by its stream.  Nothing in it has to start at zero — each call
+ *          overwrites all it reads. */
+int mi355_gemm_mxfp4_static(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
+                            const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K);
 /* Operands for it: dst[i] = lo + floor(span * (z >> 32) / 2^32), a uniform byte in [lo, lo+span)
  * (span 256, lo 0: random code pairs; lo 123, span 9: scales 2^-4 .. 2^4). */
 int mi355_fill_bytes(mi355_dev *dev, uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream,
