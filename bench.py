@@ -241,6 +241,135 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
             b.free()
 
 
+class _Telemetry:
+    """Samples the board's power (hwmon power1_input / power1_average, microwatts) and shader clock (the
+    starred line of pp_dpm_sclk) from sysfs on a thread of its own, every `period` seconds."""
+
+    def __init__(self, period=0.01):
+        import glob
+        self.period = period
+        self.power = next((f for pat in ("power1_input", "power1_average")
+                           for f in sorted(glob.glob(f"/sys/class/drm/card*/device/hwmon/hwmon*/{pat}"))), None)
+        self.sclk = next(iter(sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))), None)
+        cap = next(iter(sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"))), None)
+        self.cap_w = self._read_uw(cap)
+        self.samples = []
+        self._run = False
+
+    @staticmethod
+    def _read_uw(path):
+        try:
+            return int(open(path).read().strip()) / 1e6
+        except (OSError, ValueError, TypeError):
+            return None
+
+    def _read_mhz(self):
+        try:
+            for ln in open(self.sclk).read().splitlines():
+                if ln.rstrip().endswith("*"):
+                    return float(ln.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+        except (OSError, ValueError, TypeError, IndexError):
+            pass
+        return None
+
+    def start(self):
+        import threading
+        self.samples, self._run = [], True
+
+        def loop():
+            while self._run:
+                self.samples.append((time.perf_counter(), self._read_uw(self.power), self._read_mhz()))
+                time.sleep(self.period)
+        self._thread = threading.Thread(target=loop, daemon=True)
+        self._thread.start()
+
+    def stop(self, skip_s=0.5):
+        """Mean and maximum over the samples taken after the first `skip_s` seconds."""
+        self._run = False
+        self._thread.join()
+        t0 = self.samples[0][0] if self.samples else 0.0
+        w = [p for t, p, _ in self.samples if p is not None and t - t0 >= skip_s]
+        m = [c for t, _, c in self.samples if c is not None and t - t0 >= skip_s]
+        return {"samples": len(w), "watts_mean": round(sum(w) / len(w), 1) if w else None, "watts_max": round(max(w), 1) if w else None,
+                "sclk_mhz_mean": round(sum(m) / len(m), 0) if m else None, "sclk_mhz_min": min(m) if m else None}
+
+
+def power_table(dev, seconds):
+    """Board power and shader clock while each matrix workload runs for `seconds`: the seeded launches beside
+    the same launches on constant and on zero operands.  One JSON line per workload."""
+    from clpeak_amd import capi
+    from clpeak_amd import workloads as wl
+    tel = _Telemetry()
+    out = []
+
+    def run(label, fn, work, unit):
+        fn(); dev.sync()
+        tel.start()
+        t0 = time.perf_counter()
+        n = 0
+        while time.perf_counter() - t0 < seconds:
+            us = dev.time_launches(fn, 50)      # HIP events around 50 launches; returns synchronised
+            n += 50
+            last_us = us / 50
+        stats = tel.stop()
+        row = {"workload": label, "us_per_launch": round(last_us, 2), "value": round(work / last_us / 1e6, 1), "unit": unit, **stats}
+        out.append(row)
+        print(json.dumps(row), flush=True)
+
+    t0 = time.perf_counter()
+    tel.start(); time.sleep(min(seconds, 2.0)); idle = tel.stop(skip_s=0.0)
+    print(json.dumps({"workload": "idle", "power_cap_w": tel.cap_w, **idle}), flush=True)
+    M = N = K = 8192
+    dA, dB, dC = dev.alloc(M * K * 2), dev.alloc(N * K * 2), dev.alloc(M * N * 2)
+    flops = 2.0 * M * N * K
+    dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+    run("gemm bf16 8192^3, seeded operands", lambda: dev.gemm_bf16(dA, dB, dC, M, N, K), flops, "tflops")
+    dev.memset(dA, 0x3f); dev.memset(dB, 0x3f)
+    run("gemm bf16 8192^3, constant operands (every byte 0x3f)", lambda: dev.gemm_bf16(dA, dB, dC, M, N, K), flops, "tflops")
+    dev.memset(dA, 0); dev.memset(dB, 0)
+    run("gemm bf16 8192^3, zero operands", lambda: dev.gemm_bf16(dA, dB, dC, M, N, K), flops, "tflops")
+    for b in (dA, dB, dC):
+        b.free()
+    waves, iters = 2048, 4096
+    clk = dev.alloc(16)
+    for kind in (capi.MFMA_BF16_16x16x32, capi.MFMA_F16_32x32x16, capi.MFMA_MXFP6_E3M2):
+        sh = wl.DENSE[kind]
+        for zero in (False, True):
+            A, B, sA, sB = wl.dense_inputs(kind, waves, SEED)
+            if zero:
+                A, B = np.zeros_like(A), np.zeros_like(B)
+            bufs = [dev.from_host(A), dev.from_host(B), dev.from_host(sA) if sA is not None else None, dev.from_host(sB) if sB is not None else None]
+            o = dev.alloc(waves * 4 * sh["M"] * sh["N"] * 4)
+            run(f"{sh['name']} {sh['shape']}, {'zero' if zero else 'seeded'} operands",
+                lambda: dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], o, waves, iters, clk), wl.dense_flops(kind, waves, iters), "tflops")
+            for b in bufs + [o]:
+                if b is not None:
+                    b.free()
+    for kind in (capi.SMFMAC_F16_16x16x64,):
+        sh = wl.SPARSE[kind]
+        for zero in (False, True):
+            Ac, meta, B = wl.sparse_inputs(kind, waves, SEED)
+            if zero:
+                Ac, B = np.zeros_like(Ac), np.zeros_like(B)
+            bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
+            o = dev.alloc(waves * 4 * 256 * 4)
+            run(f"{sh['name']} {sh['shape']}, {'zero' if zero else 'seeded'} operands",
+                lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk), wl.sparse_flops(kind, waves, iters), "tflops")
+            for b in bufs + [o]:
+                b.free()
+    clk.free()
+    n_items, steps = 1 << 20, 4096
+    o = dev.alloc(n_items * 8)
+    run("mad fp32 float4 (vector FMA chains)", lambda: dev.compute_mad(capi.MAD_F32, 4, SEED, n_items, steps, o), n_items * 16 * steps * 2 * 1.0, "tflops")
+    o.free()
+    n = 1 << 30
+    src, o = dev.alloc(n * 4), dev.alloc(dev.props.num_cus * 256 * 4)
+    dev.fill_f32(src, n, SEED, wl.STREAM_BW, capi.DIST_U01)
+    run("hbm float4 read over 4 GiB", lambda: dev.global_bandwidth(4, src, n, o, dev.props.num_cus, 256), n * 4 * 1e3, "gbps")
+    src.free(); o.free()
+    return out
+
+
 def _llc_bytes():
     """Total last-level cache of the machine: the sum of the distinct L3 caches sysfs lists."""
     seen, total = set(), 0
@@ -354,6 +483,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only the plain copy kernel over 1 GiB (20 launches): under rocprofv3 --pmc this "
                          "gives what FETCH_SIZE / WRITE_SIZE read for a transfer of known size")
+    ap.add_argument("--power-table", type=float, default=0.0, metavar="SECONDS",
+                    help="run only the power / clock telemetry: each matrix workload for SECONDS while board power and "
+                         "shader clock are sampled from sysfs every 10 ms; one JSON line per workload")
     ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer",
                     help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer")
     args = ap.parse_args()
@@ -364,6 +496,11 @@ def main():
     from clpeak_amd import capi
     from clpeak_amd import workloads as wl
     dev = capi.Device(0)
+
+    if args.power_table:
+        power_table(dev, args.power_table)
+        dev.close()
+        return
 
     if args.calibrate_copy:
         nbytes = 1 << 30
