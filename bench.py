@@ -120,7 +120,7 @@ def _mad_rows(dev, capi, add, budget):
            ("half_precision_compute", capi.MAD_F16, [(1, "half"), (2, "half2")], 2, "gflops", None),
            ("double_precision_compute", capi.MAD_F64, [(1, "double"), (2, "double2"), (4, "double4")], 2, "gflops", PEAK["fp64_vec"] * 1e3),
            ("mixed_precision_compute", capi.MAD_MP, [(1, "mp")], 2, "gflops", None),
-           ("bfloat16_compute", capi.MAD_BF16, [(1, "bf16")], 2, "gflops", None),
+           ("bfloat16_compute", capi.MAD_BF16, [(1, "bf16")], 4, "gflops", None),   # two products and two additions per step
            ("integer_compute", capi.MAD_I32, [(1, "int"), (2, "int2"), (4, "int4")], 2, "gops", None)]
     for test, kind, variants, ops, unit, peak in mad:
         for width, metric in variants:

@@ -110,44 +110,106 @@ mad_f16_kernel(uint64_t seed, uint16_t a_bits, uint32_t steps, uint64_t n_items,
   out[item] = bits;
 }
 
-// ---- narrow operands, fp32 accumulator: acc = fma(float(xn), float(an), acc) --------
-// kHalf: operands are IEEE half (maps to the mixed-precision FMA); otherwise bf16.
-template <bool kHalf>
+// ---- narrow operands, fp32 accumulator ---------------------------------------------------------------------
+// Both kernels keep the narrow operands live inside the chain and run on the instruction the hardware has for
+// "narrow x narrow + fp32": the reference's kernels are fp32 chains that pass the running value through the
+// narrow type once per block (src/rocm/rocm_kernels/compute_mp.hip:18-23, compute_bf16.hip:26-31), and so are
+// these, with the narrow sources read by the multiply-add itself.
+//
+// mp (half):  x <- fma(x, a, x0), x in fp32, a and x0 IEEE half in registers, widened by v_fma_mix_f32 on every
+//             step (exact), one fused rounding to fp32; after every 16th step x <- float(half(x)) (round to
+//             nearest even) and the next step reads that half directly.  a = 1 - 2^-10 (0x3bfe), x0 = half(u),
+//             x starts at x0.  2 flop per step.
+// bf16:       acc <- acc + xb * ab + x0b * 1, one v_dot2_f32_bf16 per step (packed sources (xb, x0b) and
+//             (ab, 1.0), fp32 accumulator; 4 flop); after every 128th step xb <- bf16(acc) (round to nearest
+//             even).  ab = -2^-8 (0xbb80), x0b = bf16(u), xb and acc start at x0b.
+#define MI355_FMA_MIX_F32(x, a_h, x0_h) \
+  asm volatile("v_fma_mix_f32 %0, %0, %1, %2 op_sel_hi:[0,1,1]" : "+v"(x) : "v"(a_h), "v"(x0_h))
+// first step after a round trip: the chain value itself is the half in the low 16 bits of xh
+#define MI355_FMA_MIX_F32_FROM_HALF(x, xh, a_h, x0_h) \
+  asm volatile("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,1,1]" : "=v"(x) : "v"(xh), "v"(a_h), "v"(x0_h))
+#define MI355_DOT2_F32_BF16(acc, a_pair, b_pair) \
+  asm volatile("v_dot2_f32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a_pair), "v"(b_pair))
+
+constexpr uint32_t kMpBlock = 16, kBf16Block = 128;
+
 __global__ void __launch_bounds__(256)
-mad_mixed_kernel(uint64_t seed, uint32_t steps, uint64_t n_items, float *__restrict__ out) {
+mad_mp_kernel(uint64_t seed, uint32_t steps, uint64_t n_items, float *__restrict__ out) {
   const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (item >= n_items) return;
-  float acc[kAcc];
-  float sum = 0.0f;
-  if constexpr (kHalf) {
-    // the multiplier is a compile-time constant so that it can be the literal of v_fmac_f32 (see mad_fp_kernel):
-    // 1 - 2^-10, the half below one (code 0x3bfe)
-    constexpr float a = 1.0f - 0.0009765625f;
-    _Float16 xn[kAcc];
+  uint32_t x0h[kAcc];   // half bits in the low 16
+  float x[kAcc];
+  uint32_t a_h = 0x3bfeu;
+  asm volatile("" : "+v"(a_h));   // a vector register, not a literal: the mixed form takes no 16-bit literal
 #pragma unroll
-    for (int j = 0; j < kAcc; j++) {
-      xn[j] = bits_to_half(mi355_f32_to_f16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j))));
-      acc[j] = (float)xn[j];
-    }
-#pragma unroll 8
-    for (uint32_t s = 0; s < steps; s++) {
-#pragma unroll
-      for (int j = 0; j < kAcc; j++) acc[j] = __builtin_fmaf((float)xn[j], a, acc[j]);
-    }
-  } else {
-    constexpr float a = 1.0f - 0.00390625f;   // 1 - 2^-8, the bf16 below one (code 0x3f7f)
-    float xn[kAcc];
-#pragma unroll
-    for (int j = 0; j < kAcc; j++) {
-      xn[j] = mi355_bf16_to_f32(mi355_f32_to_bf16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j))));
-      acc[j] = xn[j];
-    }
-#pragma unroll 8
-    for (uint32_t s = 0; s < steps; s++) {
-#pragma unroll
-      for (int j = 0; j < kAcc; j++) acc[j] = __builtin_fmaf(xn[j], a, acc[j]);
-    }
+  for (int j = 0; j < kAcc; j++) {
+    x0h[j] = mi355_f32_to_f16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j)));
+    x[j] = (float)bits_to_half((uint16_t)x0h[j]);
   }
+  const uint32_t blocks = steps / kMpBlock, rem = steps % kMpBlock;
+  uint32_t xh[kAcc];
+  bool from_half = false;
+  for (uint32_t b = 0; b < blocks; b++) {
+    if (from_half) {
+#pragma unroll
+      for (int j = 0; j < kAcc; j++) MI355_FMA_MIX_F32_FROM_HALF(x[j], xh[j], a_h, x0h[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < kAcc; j++) MI355_FMA_MIX_F32(x[j], a_h, x0h[j]);
+    }
+#pragma unroll
+    for (uint32_t t = 1; t < kMpBlock; t++)
+#pragma unroll
+      for (int j = 0; j < kAcc; j++) MI355_FMA_MIX_F32(x[j], a_h, x0h[j]);
+#pragma unroll
+    for (int j = 0; j < kAcc; j++) {
+      const _Float16 h = (_Float16)x[j];   // v_cvt_f16_f32, round to nearest even
+      uint16_t bits;
+      __builtin_memcpy(&bits, &h, 2);
+      xh[j] = bits;
+      x[j] = (float)h;                     // what the chain holds if no further step follows
+    }
+    from_half = true;
+  }
+  for (uint32_t r = 0; r < rem; r++)
+#pragma unroll
+    for (int j = 0; j < kAcc; j++) MI355_FMA_MIX_F32(x[j], a_h, x0h[j]);
+  float sum = 0.0f;
+#pragma unroll
+  for (int j = 0; j < kAcc; j++) sum += x[j];
+  out[item] = sum;
+}
+
+__global__ void __launch_bounds__(256)
+mad_bf16_kernel(uint64_t seed, uint32_t steps, uint64_t n_items, float *__restrict__ out) {
+  const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (item >= n_items) return;
+  uint32_t pair[kAcc];   // low half: xb, high half: x0b
+  float acc[kAcc];
+  uint32_t b_pair = 0x3f80bb80u;   // low half ab = -2^-8, high half 1.0
+  asm volatile("" : "+v"(b_pair));
+#pragma unroll
+  for (int j = 0; j < kAcc; j++) {
+    const uint32_t x0b = mi355_f32_to_bf16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j)));
+    pair[j] = x0b | (x0b << 16);
+    acc[j] = mi355_bf16_to_f32((uint16_t)x0b);
+  }
+  const uint32_t blocks = steps / kBf16Block, rem = steps % kBf16Block;
+  for (uint32_t b = 0; b < blocks; b++) {
+    for (uint32_t t8 = 0; t8 < kBf16Block / 16; t8++) {
+#pragma unroll
+      for (uint32_t t = 0; t < 16; t++)
+#pragma unroll
+        for (int j = 0; j < kAcc; j++) MI355_DOT2_F32_BF16(acc[j], pair[j], b_pair);
+    }
+#pragma unroll
+    for (int j = 0; j < kAcc; j++)   // xb <- bf16(acc), round to nearest even; x0b stays
+      pair[j] = (uint32_t)mi355_f32_to_bf16(acc[j]) | (pair[j] & 0xffff0000u);
+  }
+  for (uint32_t r = 0; r < rem; r++)
+#pragma unroll
+    for (int j = 0; j < kAcc; j++) MI355_DOT2_F32_BF16(acc[j], pair[j], b_pair);
+  float sum = 0.0f;
 #pragma unroll
   for (int j = 0; j < kAcc; j++) sum += acc[j];
   out[item] = sum;
@@ -237,11 +299,11 @@ extern "C" int mi355_compute_mad(mi355_dev *dev, int kind, int width, uint64_t s
       break;
     case MI355_MAD_MP:
       if (width != 1) BAD_WIDTH();
-      mad_mixed_kernel<true><<<grid, block, 0, st>>>(seed, steps, n_items, (float *)out);
+      mad_mp_kernel<<<grid, block, 0, st>>>(seed, steps, n_items, (float *)out);
       break;
-    case MI355_MAD_BF16:  // a = 1 - 2^-8 (0x3f7f)
+    case MI355_MAD_BF16:
       if (width != 1) BAD_WIDTH();
-      mad_mixed_kernel<false><<<grid, block, 0, st>>>(seed, steps, n_items, (float *)out);
+      mad_bf16_kernel<<<grid, block, 0, st>>>(seed, steps, n_items, (float *)out);
       break;
     case MI355_MAD_I32:
       if (width == 1) mad_i32_kernel<1><<<grid, block, 0, st>>>(seed, 3u, steps, n_items, (uint32_t *)out);

@@ -160,10 +160,12 @@ void Mi355Peak::runDevice(int ordinal, logger::BackendScope &backend) {
       "The same chains on 64-bit floats.", MI355_MAD_F64, 8, 2,
       {{"double", 1, widthNote(1)}, {"double2", 2, widthNote(2)}, {"double4", 4, widthNote(4)}, {nullptr, 0, nullptr}}};
   static const MadTest mp = {Benchmark::ComputeMP, "mixed_precision_compute", "Mixed-precision compute fp16xfp16+fp32", "gflops",
-      "Half-precision operands multiplied into a 32-bit running total.", MI355_MAD_MP, 4, 2,
+      "A 32-bit running value times a half-precision factor plus a half-precision addend, widened by the multiply-add "
+      "itself; the running value passes through half precision once every 16 steps.", MI355_MAD_MP, 4, 2,
       {{"mp", 1, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
   static const MadTest bf = {Benchmark::ComputeBF16, "bfloat16_compute", "BF16 compute bf16xbf16+fp32", "gflops",
-      "bfloat16 operands multiplied into a 32-bit running total.", MI355_MAD_BF16, 4, 2,
+      "Two bfloat16 products added to a 32-bit running total per instruction; one factor is refreshed from the total "
+      "once every 128 steps.", MI355_MAD_BF16, 4, 4,
       {{"bf16", 1, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
   static const MadTest i32 = {Benchmark::ComputeInt, "integer_compute", "Integer compute (32-bit IMAD)", "gops",
       "The same chains on 32-bit integers (multiply-add, wrapping).", MI355_MAD_I32, 4, 2,

@@ -154,9 +154,14 @@ int mi355_copy_async(mi355_dev *dev, void *dst, const void *src, size_t bytes, i
 #define MI355_MAD_F16      1  /* same in IEEE half, a = 1-2^-10 (1.0001 is 1.0 in half), x0 = half(u);
                                  width 1: scalar half FMA, 2: packed half2 FMA; out is half bits        */
 #define MI355_MAD_F64      2  /* same in double, a = 1.0001; widths 1,2,4                               */
-#define MI355_MAD_MP       3  /* acc = fma(float(xh), float(ah), acc) in fp32, xh = half(u), acc0 = xh,
-                                 ah = 1-2^-10: half x half + float; width 1                             */
-#define MI355_MAD_BF16     4  /* same with bf16 operands, ab = 1-2^-8; width 1                          */
+#define MI355_MAD_MP       3  /* x = fma(x, ah, x0h): x fp32, ah = 1-2^-10 and x0h = half(u) IEEE half operands
+                                 widened by the instruction (v_fma_mix_f32), one fp32 rounding; x starts
+                                 at x0h; after every 16th step x = float(half(x)), nearest even (the block
+                                 round trip of compute_mp.hip:18-23); width 1                           */
+#define MI355_MAD_BF16     4  /* acc = acc + xb*ab + x0b*1: one two-element bf16 dot product with an fp32
+                                 accumulator per step (v_dot2_f32_bf16, 4 flop); ab = -2^-8, x0b = bf16(u),
+                                 xb and acc start at x0b; after every 128th step xb = bf16(acc), nearest
+                                 even (the block round trip of compute_bf16.hip:26-31); width 1          */
 #define MI355_MAD_I32      5  /* x = x*3 + x0 (wrapping), x0 = high 32 bits of the word; widths 1,2,4   */
 #define MI355_MAD_I8DP     6  /* acc = sdot4(x, y, acc); y ^= acc; `width` in {1,2,4,8} = number of
                                  independent chains (x, y from element item*8+chain of streams

@@ -287,6 +287,23 @@ static int32_t sdot4(uint32_t x, uint32_t y, int32_t acc)
     return (int32_t)r;
 }
 
+/* c + a0*b0 + a1*b1 for bf16-valued a, b (given as floats) and an fp32 c, as v_dot2_f32_bf16 rounds it.
+ * Products of bf16 values are exact in fp32.  orc_dot2_mode selects among the candidate roundings:
+ *   0  the exact three-term sum rounded once (the operands of the MAD workload keep it inside 53 bits);
+ *   1  fma(a1, b1, fma(a0, b0, c));   2  fma(a0, b0, fma(a1, b1, c));   3  round(round(a0*b0 + a1*b1) + c). */
+int orc_dot2_mode = 0;
+void orc_set_dot2_mode(int mode) { orc_dot2_mode = mode; }
+float orc_dot2_bf16(float a0, float b0, float a1, float b1, float c)
+{
+    const double p0 = (double)a0 * (double)b0, p1 = (double)a1 * (double)b1;
+    switch (orc_dot2_mode) {
+    case 1: return __builtin_fmaf(a1, b1, __builtin_fmaf(a0, b0, c));
+    case 2: return __builtin_fmaf(a0, b0, __builtin_fmaf(a1, b1, c));
+    case 3: return (float)((double)(float)(p0 + p1) + (double)c);
+    default: return (float)(p0 + p1 + (double)c);
+    }
+}
+
 /* items [first, first+n): out is n elements of the kind's output type.
  * `width` only matters for MAD_I8DP, where it is the number of chains. */
 int orc_compute_mad(int kind, int width, uint64_t seed, uint64_t first, uint64_t n, uint32_t steps, void *out)
@@ -334,18 +351,41 @@ int orc_compute_mad(int kind, int width, uint64_t seed, uint64_t first, uint64_t
             ((uint16_t *)out)[q] = (uint16_t)fmt_encode(&FMT_F16, sum);
             break;
         }
-        case MAD_MP:
-        case MAD_BF16: {
-            float xn[16], acc[16];
-            const float a = kind == MAD_MP ? (float)(1.0 - 0x1.0p-10) : (float)(1.0 - 0x1.0p-8);
+        case MAD_MP: {
+            /* x <- fma(x, a, x0) in fp32 with a and x0 IEEE half values (exact in fp32), one fused rounding per
+             * step; after every 16th step the chain passes through half, round to nearest even (the block round
+             * trip of src/rocm/rocm_kernels/compute_mp.hip:18-23). */
+            float x0[16], x[16];
+            const float a = (float)(1.0 - 0x1.0p-10);
             for (int j = 0; j < 16; j++) {
                 const double u = (double)upm1_of(orc_rng_word(seed, STREAM_MAD, item * 16 + j));
-                xn[j] = (float)(kind == MAD_MP ? fmt_decode(&FMT_F16, fmt_encode(&FMT_F16, u))
-                                               : fmt_decode(&FMT_BF16, fmt_encode(&FMT_BF16, u)));
-                acc[j] = xn[j];
+                x[j] = x0[j] = (float)fmt_decode(&FMT_F16, fmt_encode(&FMT_F16, u));
             }
             for (uint32_t s = 0; s < steps; s++)
-                for (int j = 0; j < 16; j++) acc[j] = __builtin_fmaf(xn[j], a, acc[j]);
+                for (int j = 0; j < 16; j++) {
+                    x[j] = __builtin_fmaf(x[j], a, x0[j]);
+                    if (s % 16 == 15) x[j] = (float)fmt_decode(&FMT_F16, fmt_encode(&FMT_F16, (double)x[j]));
+                }
+            float sum = 0.0f;
+            for (int j = 0; j < 16; j++) sum = sum + x[j];
+            ((float *)out)[q] = sum;
+            break;
+        }
+        case MAD_BF16: {
+            /* acc <- acc + xb*ab + x0b*1 (the two-element bf16 dot product with an fp32 accumulator), ab = -2^-8;
+             * after every 128th step xb <- bf16(acc), round to nearest even (the block round trip of
+             * src/rocm/rocm_kernels/compute_bf16.hip:26-31).  How the three terms are rounded: orc_dot2_bf16. */
+            float x0[16], xb[16], acc[16];
+            const float ab = -0x1.0p-8f;
+            for (int j = 0; j < 16; j++) {
+                const double u = (double)upm1_of(orc_rng_word(seed, STREAM_MAD, item * 16 + j));
+                acc[j] = xb[j] = x0[j] = (float)fmt_decode(&FMT_BF16, fmt_encode(&FMT_BF16, u));
+            }
+            for (uint32_t s = 0; s < steps; s++)
+                for (int j = 0; j < 16; j++) {
+                    acc[j] = orc_dot2_bf16(xb[j], ab, x0[j], 1.0f, acc[j]);
+                    if (s % 128 == 127) xb[j] = (float)fmt_decode(&FMT_BF16, fmt_encode(&FMT_BF16, (double)acc[j]));
+                }
             float sum = 0.0f;
             for (int j = 0; j < 16; j++) sum = sum + acc[j];
             ((float *)out)[q] = sum;

@@ -149,3 +149,25 @@ def test_gemm_fp32_and_fp64_kernels(tmp_path):
     order = "".join(marks)
     assert "r" * 8 + "w" + "M" * 32 + "wB" in order, order
     assert order.count("M" * 32) == 2 and order.count("B") == 2
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_mixed_precision_mad_loops_run_on_the_mixed_instructions(tmp_path):
+    """The `mp` row's loop is v_fma_mix_f32 (half sources widened by the instruction, fp32 result) and the `bf16`
+    row's loop is v_dot2_f32_bf16; no plain fp32 multiply-add does the work of either, the block round trips are
+    there (one conversion per accumulator per block), and nothing spills."""
+    asm = device_asm(tmp_path, "compute_mad.hip")
+    meta = kernel_metadata(asm)
+    mp = next(n for n in meta if "mad_mp_kernel" in n)
+    bf = next(n for n in meta if "mad_bf16_kernel" in n)
+    for name in (mp, bf):
+        assert meta[name].get("vgpr_spill_count", 0) == 0 and meta[name].get("private_segment_fixed_size", 0) == 0, meta[name]
+    body = kernel_body(asm, mp)
+    # 16 accumulators x (16 steps of a block, entered from fp32 or from the half of the last round trip, + the tail loop)
+    assert body.count("v_fma_mix_f32") == 16 * 16 + 16 + 16, body.count("v_fma_mix_f32")
+    assert body.count("op_sel_hi:[1,1,1]") == 16          # the first step of a block reads the chain value as half
+    assert body.count("v_cvt_f16_f32") >= 16
+    assert not re.search(r"\bv_(fma|fmac|fmamk|fmaak|mad|mac)_f32\b", body)
+    body = kernel_body(asm, bf)
+    assert body.count("v_dot2_f32_bf16") == 16 * 16 + 16, body.count("v_dot2_f32_bf16")
+    assert not re.search(r"\bv_(fma|fmac|fmamk|fmaak|mad|mac)_f32\b", body)

@@ -167,7 +167,10 @@ MAD_CASES = [
     (capi.MAD_F32, 1, 4096, np.float32), (capi.MAD_F32, 2, 100, np.float32), (capi.MAD_F32, 4, 4096, np.float32),
     (capi.MAD_F64, 1, 4096, np.float64), (capi.MAD_F64, 2, 33, np.float64), (capi.MAD_F64, 4, 512, np.float64),
     (capi.MAD_F16, 1, 300, np.uint16), (capi.MAD_F16, 2, 300, np.uint16), (capi.MAD_F16, 2, 7, np.uint16),
-    (capi.MAD_MP, 1, 4096, np.float32), (capi.MAD_BF16, 1, 4096, np.float32),
+    (capi.MAD_MP, 1, 4096, np.float32), (capi.MAD_MP, 1, 15, np.float32), (capi.MAD_MP, 1, 16, np.float32),
+    (capi.MAD_MP, 1, 17, np.float32), (capi.MAD_MP, 1, 100, np.float32),
+    (capi.MAD_BF16, 1, 4096, np.float32), (capi.MAD_BF16, 1, 127, np.float32), (capi.MAD_BF16, 1, 128, np.float32),
+    (capi.MAD_BF16, 1, 129, np.float32), (capi.MAD_BF16, 1, 300, np.float32),
     (capi.MAD_I32, 1, 2048, np.uint32), (capi.MAD_I32, 2, 5, np.uint32), (capi.MAD_I32, 4, 2048, np.uint32),
     (capi.MAD_I8DP, 1, 1024, np.int32), (capi.MAD_I8DP, 2, 1024, np.int32), (capi.MAD_I8DP, 4, 99, np.int32),
     (capi.MAD_I8DP, 8, 1024, np.int32),

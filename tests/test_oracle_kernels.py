@@ -118,19 +118,70 @@ def test_mad_f16_against_numpy_float16():
     assert np.array_equal(got, s.view(np.uint16))
 
 
-def test_mad_mixed_closed_form():
-    """acc_n = xh + n * (xh*a) up to fp32 rounding; operands really are rounded through half / bf16."""
-    n, steps = 8, 1000
-    for kind, a in ((3, 1 - 2.0 ** -10), (4, 1 - 2.0 ** -8)):
-        got = orc.compute_mad(kind, 1, 8, 0, n, steps)
-        u = _seeds(8, 0, n)
-        if kind == 3:
-            xn = u.astype(np.float16).astype(np.float64)
-        else:
-            xn = orc.decode(orc.FMT_BF16, orc.encode(orc.FMT_BF16, u))
-        ref = (xn + steps * xn * a).sum(axis=1)
-        assert np.allclose(got, ref, rtol=1e-4, atol=1e-3)
-        assert not np.allclose(got, (u + steps * u * a).sum(axis=1), rtol=1e-6, atol=0)  # rounding of operands is visible
+def _bf16_round(x):
+    """float32 array -> nearest-even bfloat16, returned as float32 (numpy only)."""
+    u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return (((u + 0x7fff + ((u >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32)
+
+
+def test_mad_mp_against_numpy():
+    """x <- fl32(x*a + x0) with half-valued a and x0, through half every 16th step.  x*a + x0 is exact in float64
+    (x within a factor 2^10 of x0, 24 + 11 bits of product), so one numpy float32 rounding of the float64 value
+    is the fused multiply-add; numpy's float16 is the round trip."""
+    n = 32
+    u = _seeds(8, 0, n)
+    x0 = u.astype(np.float16).astype(np.float32)
+    a = np.float32(np.float16(1 - 2.0 ** -10))
+    for steps in (1, 15, 16, 17, 100, 4096):
+        x = x0.copy()
+        for s in range(steps):
+            x = (x.astype(np.float64) * np.float64(a) + x0.astype(np.float64)).astype(np.float32)
+            if s % 16 == 15:
+                x = x.astype(np.float16).astype(np.float32)
+        ref = np.zeros(n, dtype=np.float32)
+        for j in range(16):
+            ref = (ref + x[:, j]).astype(np.float32)
+        assert np.array_equal(orc.compute_mad(3, 1, 8, 0, n, steps), ref), steps
+    # the recurrence heads for x0 / (1 - a) = 1024 x0: at 4096 steps 1 - a^4097 = 0.982 of it, up to the round trips
+    got = orc.compute_mad(3, 1, 8, 0, n, 4096)
+    terms = 1024.0 * x0.astype(np.float64) * (1 - float(a) ** 4097)
+    assert np.all(np.abs(got - terms.sum(axis=1)) <= 1e-2 * np.abs(terms).sum(axis=1))   # 256 roundings to 11 bits
+    # the half operands are visible: an fp32 x0 gives another result
+    assert not np.allclose(got, (1024.0 * u * (1 - float(a) ** 4097)).sum(axis=1), rtol=1e-7, atol=0)
+
+
+def test_mad_bf16_against_numpy_and_every_rounding_of_the_dot_product():
+    """acc <- acc + xb*ab + x0b in fp32 (ab = -2^-8), xb <- bf16(acc) every 128th step, restated in numpy with the
+    exact three-term sum (float64) rounded once.  The operands keep that sum short enough that the candidate
+    roundings of a two-element dot product (exact sum rounded once; two chained fused multiply-adds in either
+    order; the product pair rounded before the accumulator is added) all agree, so the workload's result does not
+    depend on which one the hardware implements: checked here by running the oracle in each."""
+    n = 64
+    u = _seeds(8, 0, n)
+    x0 = _bf16_round(u.astype(np.float32))
+    ab = np.float64(-2.0 ** -8)
+    L = orc.lib()
+    try:
+        for steps in (1, 127, 128, 129, 300, 4096):
+            acc, xb = x0.copy(), x0.copy()
+            for s in range(steps):
+                acc = (acc.astype(np.float64) + xb.astype(np.float64) * ab + x0.astype(np.float64)).astype(np.float32)
+                if s % 128 == 127:
+                    xb = _bf16_round(acc)
+            ref = np.zeros(n, dtype=np.float32)
+            for j in range(16):
+                ref = (ref + acc[:, j]).astype(np.float32)
+            for mode in range(4):
+                L.orc_set_dot2_mode(mode)
+                assert np.array_equal(orc.compute_mad(4, 1, 8, 0, n, steps), ref), (steps, mode)
+    finally:
+        L.orc_set_dot2_mode(0)
+    # per block the total moves half way to 256 x0b: after 32 blocks it is there
+    got = orc.compute_mad(4, 1, 8, 0, n, 4096)
+    assert np.allclose(got, (256.0 * x0.astype(np.float64)).sum(axis=1), rtol=2e-2, atol=1.0)
+    # 100 steps into the first block: acc = x0b (1 + 100 (1 - 2^-8)) exactly
+    got = orc.compute_mad(4, 1, 8, 0, n, 100)
+    assert np.allclose(got, (x0.astype(np.float64) * (1 + 100 * (1 - 2.0 ** -8))).sum(axis=1), rtol=1e-6, atol=1e-6)
 
 
 def test_mad_i32_exact():
