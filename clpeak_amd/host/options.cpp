@@ -11,12 +11,29 @@ const Named kTests[] = {
     {"half-precision-compute", Benchmark::ComputeHP}, {"mixed-precision-compute", Benchmark::ComputeMP},
     {"single-precision-compute", Benchmark::ComputeSP}, {"double-precision-compute", Benchmark::ComputeDP},
     {"bfloat16-compute", Benchmark::ComputeBF16},     {"integer-compute", Benchmark::ComputeInt},
-    {"integer-compute-int8-dp", Benchmark::ComputeInt8DP}, {"wmma", Benchmark::Wmma},
+    {"int8-dot-product-compute", Benchmark::ComputeInt8DP}, {"wmma", Benchmark::Wmma},
     {"rocwmma", Benchmark::Rocwmma},                  {"mfma", Benchmark::Mfma},
     {"rocblas", Benchmark::Rocblas},                  {"kernel-launch-latency", Benchmark::KernelLatency}};
 struct NamedCat { const char *flag; Category c; };
 const NamedCat kCats[] = {{"fp-compute", Category::FpCompute}, {"int-compute", Category::IntCompute},
-                          {"bandwidth", Category::Bandwidth}, {"latency", Category::Latency}};
+                          {"crypto", Category::Crypto},         {"string", Category::String},
+                          {"bandwidth", Category::Bandwidth},   {"latency", Category::Latency}};
+
+// The rest of clpeak's grammar (src/common/options.cpp:194-264, 469-497, 552-639): flags that select tests, backends
+// and devices this backend does not have.  A front end written against clpeak passes them (the GUI names every
+// selected category and every deselected backend, app/lib/src/model/run_config.dart:98-144), so they parse here
+// with the same effect they have on the ROCm backend there: tests of other backends select nothing of this one but
+// still switch test selection to an allow-list, another backend named alone leaves this one out, device lists of
+// other backends are checked and dropped.
+const char *const kForeignTests[] = {
+    "integer-compute-fast", "integer-compute-char", "integer-compute-short", "int16-dot-product-compute",
+    "fp8-dot-product-compute", "divide-sqrt-compute", "integer-divide-compute", "coopmat", "simdgroup-matrix", "cublas",
+    "mps-gemm", "mps-attention", "texture-sample", "joint-matrix", "onemkl", "amx", "accelerate", "aes", "sha256",
+    "sha512", "crc32c", "string-scan", "utf8-validate", "cache-bandwidth", "memory-latency", "atomics",
+    "branch-penalty", "store-forward", "smt-scaling"};
+const char *const kForeignBackends[] = {"opencl", "vulkan", "cuda", "metal", "oneapi", "cpu"};
+const char *const kForeignDeviceLists[] = {"--cl-platform", "--cl-device", "--vk-device", "--cuda-device", "--mtl-device",
+                                           "--oneapi-device"};
 
 bool parseIntList(const char *s, std::vector<int> &out) {
   std::string tok;
@@ -33,11 +50,13 @@ bool parseIntList(const char *s, std::vector<int> &out) {
   }
 }
 
-bool parseUnsigned(const char *s, unsigned &out) {
+bool parseUnsigned(const char *s, unsigned &out, bool allowZero = true) {
   if (!s || !*s) return false;
+  for (const char *p = s; *p; p++)
+    if (*p < '0' || *p > '9') return false;
   char *end = nullptr;
-  const long v = strtol(s, &end, 10);
-  if (*end || v < 0) return false;
+  const unsigned long long v = strtoull(s, &end, 10);
+  if (*end || v > 0xffffffffull || (!allowZero && v == 0)) return false;
   out = (unsigned)v;
   return true;
 }
@@ -48,7 +67,9 @@ void printUsage(std::ostream &os) {
         "  --rocm-device LIST      comma-separated device ordinals (default: all)\n"
         "  --<test> / --no-<test>  ";
   for (const Named &t : kTests) os << t.flag << " ";
-  os << "\n  --<category> / --no-<category>  fp-compute int-compute bandwidth latency\n"
+  os << "\n  --<category> / --no-<category>  fp-compute int-compute bandwidth latency (crypto, string: none here)\n"
+        "  flags of clpeak's other backends (--opencl, --no-cpu, --cuda-device LIST, --max-time-cpu MS, --aes, ...)\n"
+        "                          are accepted with the meaning they have for the ROCm backend there\n"
         "  -i, --iters N           fixed iteration count per timed batch\n"
         "  -w, --warmup N          warm-up launches (default 2)\n"
         "  --max-time MS           time budget of a timed batch (default 500 ms)\n"
@@ -63,6 +84,7 @@ void printUsage(std::ostream &os) {
 
 ParseResult parseCliCore(int argc, char **argv, CliOptions &opts, HostExtras &extras, std::string &error) {
   bool testsAllowList = false, catsAllowList = false;
+  bool otherBackendNamed = false, rocmNamed = false;
   const char *value = nullptr;
   auto need = [&](int &i) -> bool {
     if (i + 1 >= argc) {
@@ -80,8 +102,31 @@ ParseResult parseCliCore(int argc, char **argv, CliOptions &opts, HostExtras &ex
     const std::string a = argv[i];
     if (a == "-h" || a == "--help") return ParseResult::Help;
     if (a == "-v" || a == "--version") return ParseResult::Version;
-    if (a == "--rocm") continue;                       // the only backend here
+    if (a == "--rocm") { rocmNamed = true; continue; }
     if (a == "--no-rocm") { opts.skipRocm = true; continue; }
+    bool foreign = false;
+    for (const char *b : kForeignBackends) {
+      if (a == std::string("--") + b) { otherBackendNamed = true; foreign = true; }
+      if (a == std::string("--no-") + b) foreign = true;
+    }
+    if (a == "--use-event-timer") foreign = true;   // OpenCL's timer choice
+    for (const char *f : kForeignDeviceLists)
+      if (a == f) {
+        std::vector<int> ignored;
+        if (!need(i)) return ParseResult::Error;
+        if (!parseIntList(value, ignored)) {
+          error = std::string("clpeak: invalid device index list: ") + value + "\n";
+          return ParseResult::Error;
+        }
+        foreign = true;
+      }
+    if (a == "--max-time-cpu") {
+      unsigned ms = 0;
+      if (!need(i)) return ParseResult::Error;
+      if (!parseUnsigned(value, ms, false) || ms > 0xffffffffu / 1000u) return invalid("--max-time-cpu");
+      foreign = true;
+    }
+    if (foreign) continue;
     if (a == "--rocm-device") {
       if (!need(i)) return ParseResult::Error;
       if (!parseIntList(value, opts.rocmDeviceIndices)) {
@@ -90,15 +135,15 @@ ParseResult parseCliCore(int argc, char **argv, CliOptions &opts, HostExtras &ex
       }
     } else if (a == "-i" || a == "--iters") {
       if (!need(i)) return ParseResult::Error;
-      if (!parseUnsigned(value, opts.iters)) return invalid("--iters");
-      opts.forceIters = opts.iters > 0;
+      if (!parseUnsigned(value, opts.iters, false)) return invalid(a.c_str());
+      opts.forceIters = true;
     } else if (a == "-w" || a == "--warmup") {
       if (!need(i)) return ParseResult::Error;
-      if (!parseUnsigned(value, opts.warmupCount)) return invalid("--warmup");
+      if (!parseUnsigned(value, opts.warmupCount)) return invalid(a.c_str());
     } else if (a == "--max-time") {
       unsigned ms = 0;
       if (!need(i)) return ParseResult::Error;
-      if (!parseUnsigned(value, ms)) return invalid("--max-time");
+      if (!parseUnsigned(value, ms, false) || ms > 0xffffffffu / 1000u) return invalid("--max-time");
       opts.targetTimeUs = ms * 1000u;
     } else if (a == "--xml-file") { if (!need(i)) return ParseResult::Error; opts.xmlFile = value; opts.enableXml = true; }
     else if (a == "--json-file") { if (!need(i)) return ParseResult::Error; opts.jsonFile = value; opts.enableJson = true; }
@@ -130,15 +175,27 @@ ParseResult parseCliCore(int argc, char **argv, CliOptions &opts, HostExtras &ex
           opts.enabledCategories.set((size_t)c.c, !neg);
           hit = true;
         }
+      if (name == "integer-compute-int8-dp") {   // this program's earlier spelling of --int8-dot-product-compute
+        if (!neg && !testsAllowList) { opts.enabledTests.reset(); testsAllowList = true; }
+        opts.enabledTests.set((size_t)Benchmark::ComputeInt8DP, !neg);
+        hit = true;
+      }
+      for (const char *t : kForeignTests)
+        if (name == t) {
+          if (!neg && !testsAllowList) { opts.enabledTests.reset(); testsAllowList = true; }
+          hit = true;
+        }
       if (!hit) {
-        error = "clpeak: unknown option " + a + "\n";
+        error = "clpeak: unknown option '" + a + "'\n";
         return ParseResult::Error;
       }
     } else {
-      error = "clpeak: unknown argument " + a + "\n";
+      error = "clpeak: unknown option '" + a + "'\n";
       return ParseResult::Error;
     }
   }
+  // any --<backend> flag means "only the listed backends" (src/common/options.cpp:685-697)
+  if (otherBackendNamed && !rocmNamed) opts.skipRocm = true;
   return ParseResult::Ok;
 }
 

@@ -186,14 +186,42 @@ static std::string statusLabel(ResultStatus s) {
   }
 }
 
+// Word-wrap `text` to 80 columns behind `column` spaces, never narrower than 32 characters; a word longer than
+// that overruns (the --describe layout of src/common/logger_text.cpp:266-299).
+static void writeWrapped(std::ostream &out, size_t column, const std::string &text) {
+  const std::string pad(column, ' ');
+  const size_t width = column + 32 > 80 ? 32 : 80 - column;
+  std::string line;
+  size_t pos = 0;
+  while (pos < text.size()) {
+    const size_t end = text.find(' ', pos);
+    const std::string word = text.substr(pos, end == std::string::npos ? std::string::npos : end - pos);
+    pos = end == std::string::npos ? text.size() : end + 1;
+    if (word.empty()) continue;
+    if (!line.empty() && line.size() + 1 + word.size() > width) {
+      out << pad << line << "\n";
+      line.clear();
+    }
+    if (!line.empty()) line += ' ';
+    line += word;
+  }
+  if (!line.empty()) out << pad << line << "\n";
+}
+
+// Layout (src/common/logger_text.cpp:48-247): the device line sits one step (two spaces) in, or two when a
+// platform line precedes it; properties and test headers one step further, readings one more, sub-readings one
+// more again.  Names are padded to the longest of the test (at least 8), sub-readings two less.
 void LoggerText::flush() {
   size_t width = 8;
   for (const Pending &p : pending_) width = std::max(width, p.entry.metric.size());
+  const size_t readingColumn = (deviceSteps_ + 2) * 2;
   for (const Pending &p : pending_) {
     const ResultEntry &e = p.entry;
+    const size_t column = readingColumn + (p.sub ? 2 : 0);
+    const size_t pad = std::max(p.sub ? width - 2 : width, (size_t)8);
     std::string name = e.metric;
-    name.resize(std::max(width - (p.sub ? 2 : 0), (size_t)8), ' ');
-    out_ << (p.sub ? "      " : "    ") << name << " : ";
+    if (name.size() < pad) name.resize(pad, ' ');
+    out_ << std::string(column, ' ') << name << " : ";
     if (e.status == ResultStatus::Ok) {
       char buf[64];
       snprintf(buf, sizeof buf, "%.2f", e.value);
@@ -210,44 +238,56 @@ void LoggerText::flush() {
       out_ << "[" << statusLabel(e.status) << "] " << e.reason;
     }
     out_ << "\n";
-    if (describe_ && !e.metricDescription.empty()) out_ << "        " << e.metricDescription << "\n";
+    // the reading's note below it, flush with the value column
+    if (describe_ && !e.metricDescription.empty()) writeWrapped(out_, column + pad + 3, e.metricDescription);
   }
   pending_.clear();
   out_.flush();
 }
 
 void LoggerText::onEvent(const LogEvent &e) {
+  const std::string propPad((deviceSteps_ + 1) * 2, ' ');
   switch (e.kind) {
     case LogEvent::Kind::BackendBegin:
-      out_ << "\nBackend: " << e.backend << "\n";
+      out_ << "Backend: " << e.backend << "\n";
       break;
-    case LogEvent::Kind::DeviceBegin:
-      if (e.showPlatformLine) out_ << "Platform: " << e.platform << "\n";
-      out_ << "  Device";
+    case LogEvent::Kind::DeviceBegin: {
+      deviceSteps_ = e.showPlatformLine ? 2 : 1;
+      if (e.showPlatformLine) {
+        out_ << "  Platform";
+        if (e.platformIndex >= 0) out_ << " " << e.platformIndex;
+        out_ << ": " << e.platform << "\n";
+      }
+      out_ << std::string(deviceSteps_ * 2, ' ') << "Device";
       if (e.deviceIndex >= 0) out_ << " " << e.deviceIndex;
       out_ << ": " << e.device << "\n";
-      if (!e.driver.empty()) out_ << "    Driver version  : " << e.driver << "\n";
-      for (const DeviceProp &p : e.props) {
-        std::string k = p.key;
-        k.resize(std::max(k.size(), (size_t)16), ' ');
-        out_ << "    " << k << ": " << p.value << "\n";
-      }
+      const std::string pad((deviceSteps_ + 1) * 2, ' ');
+      auto prop = [&](std::string key, const std::string &value) {
+        if (key.size() < 17) key.resize(17, ' ');
+        out_ << pad << key << ": " << value << "\n";
+      };
+      if (!e.driver.empty()) prop("Driver version", e.driver);
+      for (const DeviceProp &p : e.props) prop(p.key, p.value);
       break;
+    }
     case LogEvent::Kind::TestBegin: {
       flush();
       std::string unit = e.unit;
       for (char &c : unit) c = (char)toupper((unsigned char)c);
-      out_ << "\n    " << e.testDisplay;
+      out_ << "\n" << propPad << e.testDisplay;
       if (!unit.empty()) out_ << " (" << unit << ")";
       out_ << "\n";
-      if (describe_ && !e.testDescription.empty()) out_ << "      " << e.testDescription << "\n\n";
+      if (describe_ && !e.testDescription.empty()) {
+        writeWrapped(out_, (deviceSteps_ + 2) * 2, e.testDescription);
+        out_ << "\n";
+      }
       break;
     }
     case LogEvent::Kind::Metric:
       pending_.push_back({e.entry, e.subMetric});
       break;
     case LogEvent::Kind::TestSkippedAll:
-      out_ << "      [" << statusLabel(e.status) << "] " << e.reason << "\n";
+      out_ << std::string((deviceSteps_ + 2) * 2, ' ') << "[" << statusLabel(e.status) << "] " << e.reason << "\n";
       break;
     case LogEvent::Kind::TestEnd:
       flush();

@@ -141,6 +141,7 @@ class LoggerText : public logger {
   struct Pending { ResultEntry entry; bool sub; };
   std::ostream &out_;
   bool describe_;
+  size_t deviceSteps_ = 1;   // indentation of the device line in steps of two spaces
   std::vector<Pending> pending_;   // rows of the open test, printed together so they align
   void flush();
 };

@@ -197,3 +197,44 @@ def test_loads_a_result_file_the_reference_wrote(ffi):
     assert skipped and all(e["reason"] and "value" not in e for e in skipped)
     assert any(e["reason"].startswith("VK_KHR_shader_bfloat16") for e in skipped)
     assert ffi.clpeak_load_result_file_json(b"/nonexistent/file.xml") is None
+
+
+def test_arguments_the_gui_builds_for_a_partial_selection(ffi):
+    """What RunConfig.toArgs (app/lib/src/model/run_config.dart:96-144) hands to clpeak_launch when the user has
+    deselected one category, two backends and one of two ROCm devices, and changed both time budgets: a
+    --no-<backend> per deselected backend, a device list, a positive flag per remaining category (crypto and
+    string included) and both --max-time flags.  The run must start, and run what those flags select."""
+    args = ["--no-opencl", "--no-vulkan", "--rocm-device", "0", "--no-cpu",
+            "--fp-compute", "--int-compute", "--crypto", "--string", "--bandwidth",
+            "--max-time", "200", "--max-time-cpu", "500"]
+    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "-i", "1"] + args)
+    events = [json.loads(r) for r in raw]
+    assert rc == RUN_OK and events[-1] == {"t": "done", "status": 0, "cancelled": False}
+    tags = {e["test"] for e in events if e["t"] == "test_begin"}
+    assert "single_precision_compute" in tags and "integer_compute" in tags and "global_memory_bandwidth" in tags
+    assert "kernel_launch_latency" not in tags             # latency was the deselected category
+
+
+@pytest.mark.parametrize("args, runs", [
+    (["--cuda"], False),                                   # another backend named alone: this one stays out
+    (["--cuda", "--rocm"], True),
+    (["--no-cuda", "--no-metal", "--no-oneapi"], True),
+    (["--aes"], False),                                    # a test of another backend: allow-list with nothing of ours in it
+    (["--aes", "--mfma"], True),
+    (["--no-aes", "--no-cache-bandwidth", "--use-event-timer"], True),
+    (["--cl-platform", "0", "--cl-device", "0,1", "--vk-device", "1", "--cuda-device", "0", "--mtl-device", "0", "--oneapi-device", "2"], True),
+    (["--crypto"], False),                                 # a category with no test here
+])
+def test_flags_of_the_other_backends_parse_with_their_meaning(ffi, args, runs):
+    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "-i", "1"] + args)
+    events = [json.loads(r) for r in raw]
+    assert rc == RUN_OK, (args, events[:1])
+    began = [e for e in events if e["t"] == "test_begin"]
+    assert bool(began) == runs, (args, [e["test"] for e in began])
+
+
+@pytest.mark.parametrize("args", [["--max-time-cpu"], ["--max-time-cpu", "0"], ["--max-time", "0"], ["--iters", "0"],
+                                  ["--cuda-device", "a"], ["--cl-platform"], ["--integer-compute-wide"]])
+def test_malformed_values_of_those_flags_are_still_refused(ffi, args):
+    rc, raw = launch(ffi, ["--fake-device"] + args)
+    assert rc == RUN_BAD_ARGS and json.loads(raw[0])["message"].startswith("clpeak:")

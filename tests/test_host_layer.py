@@ -101,6 +101,35 @@ def test_text_table_format():
     assert "Single-precision compute (GFLOPS)" in out and "Global memory bandwidth (GBPS)" in out
     assert re.search(r"^\s+float    : \d+\.\d\d$", out, re.M) and re.search(r"^\s+float4   : \d+\.\d\d$", out, re.M)
     assert "MFMA" not in out and "latency" not in out.lower()
+    # the reference's layout (README.md:90-97, src/common/logger_text.cpp:58-100): device one step in, properties and
+    # test headers at two, readings at three; property keys padded to 17 characters
+    lines = out.splitlines()
+    assert lines[0] == "Backend: ROCm" and lines[1] == "  Device 0: Fake MI355X"
+    assert lines[2] == "    Driver version   : 7.2.0" and "    CUs              : 256" in lines
+    assert "    Single-precision compute (GFLOPS)" in lines
+    assert any(re.fullmatch(r"      float    : \d+\.\d\d", ln) for ln in lines)
+
+
+def test_describe_prints_wrapped_notes_under_headers_and_readings():
+    """--describe (src/common/logger_text.cpp:129-135, 238-243, 266-299): the test's description under its header,
+    one step in from it, wrapped to 80 columns and followed by a blank line; each reading's note on the line(s)
+    below the reading, flush with the value column; without the flag none of that text appears."""
+    plain = run_cli("--single-precision-compute", "--kernel-launch-latency").stdout
+    out = run_cli("--describe", "--single-precision-compute", "--kernel-launch-latency").stdout
+    lines = out.splitlines()
+    h = lines.index("    Single-precision compute (GFLOPS)")
+    assert lines[h + 1].startswith("      Vector-ALU rate") and lines[h + 2].startswith("      ") and lines[h + 3] == ""
+    desc = " ".join(ln.strip() for ln in lines[h + 1:h + 3])
+    assert desc.endswith("nothing but registers involved.")
+    assert all(len(ln) <= 80 for ln in lines)
+    f = next(i for i, ln in enumerate(lines) if re.fullmatch(r"      float    : \d+\.\d\d", ln))
+    assert lines[f + 1] == " " * (6 + 8 + 3) + "One value per lane at a time."
+    # a skipped reading carries its note too
+    d = next(i for i, ln in enumerate(lines) if ln.startswith("      dispatch  : [unsupported] "))
+    assert lines[d + 1].startswith(" " * (6 + 9 + 3)) and lines[d + 1].strip()
+    assert "Vector-ALU rate" not in plain and "One value per lane" not in plain
+    reading = re.compile(r"      \S+ +: (\d|\[)")            # the rows themselves are the same with and without
+    assert [ln for ln in plain.splitlines() if reading.match(ln)] == [ln for ln in lines if reading.match(ln)]
 
 
 def test_allow_list_and_subtract_flags(tmp_path):
