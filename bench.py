@@ -411,7 +411,79 @@ def _stream_floats(threads):
     return max(n // threads * threads, threads), llc
 
 
-def cpu_baseline(target_us=2_000_000, extra_target_us=1_000_000):
+def _port_families(orc, pool, target_us):
+    """The CPU oracle's kernel of every GPU row family, timed at one thread and at all of them on a bounded sample
+    of the same seeded workload.  Returns {row: figures}; "_headline" is the raw result of the float4 read."""
+    from oracle import workloads as owl
+    port = {}
+    small = 60_000        # budget of a timed batch of the emulated families, in microseconds
+
+    def entry(q, unit, what):
+        return {"ST": round(q.giga_st, 3), "MT": round(q.giga_mt, 3), "unit": unit, "threads": q.threads_mt,
+                "iters_ST": q.iters_st, "iters_MT": q.iters_mt, "sample": what}
+
+    def ptr(a):
+        return a.ctypes.data if a is not None else None
+
+    # --- read-reduce over the 256 MiB buffer of the CPU configuration, 2^20 partial sums, every width
+    n, T = 1 << 26, 1 << 20
+    buf = orc.fill_f32(n, SEED, owl.STREAM_BW, 0)
+    for width, metric in ((4, "float4"), (2, "float2"), (1, "float")):
+        op = orc.CpuhOp(op=orc.OP_READ, width=width, p0=ptr(buf), n_floats=n, T=T)
+        q = pool.measure_op(op, n * 4.0, n * 4.0 / pool.max_threads, target_us=target_us if width == 4 else small, keep=(buf,))
+        port[f"global_memory_bandwidth {metric}"] = entry(q, "GB/s", f"{metric} read-reduce over a 256 MiB (2^26 float) seeded buffer, "
+                                                          "2^20 partial sums, one pass per iteration")
+        if width == 4:
+            port["_headline"] = q
+    del buf
+    # --- vector multiply-add chains: 8 work-items x 16 accumulators (or `chains`) x 4096 steps per iteration
+    for row, kind, width, chains, ops, unit in (
+            ("single_precision_compute float4", 0, 4, 16, 2, "gflops"), ("half_precision_compute half2", 1, 2, 16, 2, "gflops"),
+            ("double_precision_compute double", 2, 1, 16, 2, "gflops"), ("mixed_precision_compute mp", 3, 1, 16, 2, "gflops"),
+            ("bfloat16_compute bf16", 4, 1, 16, 4, "gflops"), ("integer_compute int", 5, 1, 16, 2, "gops"),
+            ("integer_compute_int8_dp int8_dp8", 6, 8, 8, 8, "gops")):
+        op = orc.CpuhOp(op=orc.OP_MAD, kind=kind, width=width, seed=SEED)
+        q = pool.measure_op(op, orc.OP_MAD_ITEMS * chains * 4096.0 * ops, warmup=1, target_us=target_us if kind == 0 else small)
+        port[row] = entry(q, unit, f"{orc.OP_MAD_ITEMS} work-items x {chains} chains x 4096 steps per iteration")
+    # --- emulated matrix instructions: the 4 chains of one wave, one instruction each, per iteration
+    for kind, sh in sorted(owl.DENSE.items()):
+        A, B, sA, sB = owl.dense_inputs(kind, 1, SEED)
+        op = orc.CpuhOp(op=orc.OP_MFMA, kind=kind, p0=ptr(A), p1=ptr(B), p2=ptr(sA), p3=ptr(sB))
+        q = pool.measure_op(op, 4 * 2.0 * sh["M"] * sh["N"] * sh["K"], warmup=1, target_us=small, keep=(A, B, sA, sB))
+        port[sh["name"]] = entry(q, "gops" if sh["fmt"] is None else "gflops", f"4 emulated {sh['shape']} products per iteration (one wave of 2048)")
+    for kind, sh in sorted(owl.SPARSE.items()):
+        Ac, meta, B = owl.sparse_inputs(kind, 1, SEED)
+        op = orc.CpuhOp(op=orc.OP_SMFMAC, kind=kind, p0=ptr(Ac), p1=ptr(meta), p2=ptr(B))
+        q = pool.measure_op(op, 4 * 2.0 * 16 * 16 * sh["K"], warmup=1, target_us=small, keep=(Ac, meta, B))
+        port[sh["name"]] = entry(q, "gops" if sh["fmt"] is None else "gflops",
+                                 f"4 emulated 2:4 sparse {sh['shape']} products per iteration, dense-equivalent operations")
+    # --- GEMM: one 32x32 tile of the K = 8192 product per iteration (of 65536 such tiles)
+    K, t = 8192, 32
+    for row, fa, fb, unit in (("rocblas-fp bf16", orc.FMT_BF16, orc.FMT_BF16, "gflops"), ("rocblas-fp fp16", orc.FMT_F16, orc.FMT_F16, "gflops"),
+                              ("rocblas-fp fp32", orc.FMT_F32, orc.FMT_F32, "gflops"), ("rocblas-fp fp64", orc.FMT_F64, orc.FMT_F64, "gflops"),
+                              ("hipblaslt-fp8 fp8_e4m3", orc.FMT_E4M3, orc.FMT_E4M3, "gflops"),
+                              ("hipblaslt-fp8 fp8_e5m2", orc.FMT_E5M2, orc.FMT_E4M3, "gflops"), ("rocblas-int int8", orc.FMT_I8, orc.FMT_I8, "gops")):
+        def operand(fmt, stream):
+            if fmt == orc.FMT_I8:
+                return orc.fill_int8(SEED, stream, t * K)
+            if fmt == orc.FMT_F32:
+                return orc.fill_f32(t * K, SEED, stream, 1)
+            if fmt == orc.FMT_F64:
+                return orc.fill_f32(t * K, SEED, stream, 1).astype(np.float64)
+            return orc.fill_fmt(fmt, t * K, SEED, stream, 1, 448.0 if fmt == orc.FMT_E4M3 else 57344.0 if fmt == orc.FMT_E5M2 else 1.0)
+        A, B = operand(fa, owl.STREAM_GEMM_A), operand(fb, owl.STREAM_GEMM_B)
+        op = orc.CpuhOp(op=orc.OP_GEMM, kind=fa, width=fb, p0=ptr(A), p1=ptr(B), K=K, tile=t, scale=1.0)
+        q = pool.measure_op(op, 2.0 * t * t * K, warmup=1, target_us=small, keep=(A, B))
+        port[row] = entry(q, unit, f"one {t}x{t} tile of the K={K} product per iteration")
+    A, B = orc.fill_bytes(t * K // 2, SEED, owl.STREAM_GEMM_A, 0, 256), orc.fill_bytes(t * K // 2, SEED, owl.STREAM_GEMM_B, 0, 256)
+    SA, SB = orc.fill_bytes(t * K // 32, SEED, owl.STREAM_SCALE_A, 123, 9), orc.fill_bytes(t * K // 32, SEED, owl.STREAM_SCALE_B, 123, 9)
+    op = orc.CpuhOp(op=orc.OP_GEMM_MX, p0=ptr(A), p1=ptr(B), p2=ptr(SA), p3=ptr(SB), K=K, tile=t)
+    q = pool.measure_op(op, 2.0 * t * t * K, warmup=1, target_us=small, keep=(A, B, SA, SB))
+    port["hipblaslt-fp8 mxf4_e2m1"] = entry(q, "gflops", f"one {t}x{t} tile of the K={K} block-scaled product per iteration")
+    return port
+
+
+def cpu_baseline(target_us=1_500_000, extra_target_us=600_000):
     """CPU figures beside the GPU ones, all timed with the reference's CPU discipline (pinned persistent
     pool, warm-ups, settle phase before the all-core run, adaptive probe, one timed batch sized to the
     budget), at one thread (ST) and at every logical core (MT).
@@ -425,20 +497,8 @@ def cpu_baseline(target_us=2_000_000, extra_target_us=1_000_000):
     t0 = time.perf_counter()
     ref = orc.reference_kernels()
     with orc.CpuPool(cores) as pool:
-        r = pool.measure(orc.CPUH_READ_FLOAT4, SEED, 2, target_us)
-        port = {"global_memory_bandwidth float4": {
-            "ST": round(r.giga_st, 2), "MT": round(r.giga_mt, 2), "unit": "GB/s", "threads": r.threads_mt,
-            "iters_ST": r.iters_st, "iters_MT": r.iters_mt,
-            "sample": "float4 read-reduce over a 256 MiB (2^26 float) seeded buffer, 2^20 partial sums, one pass per iteration"}}
-        for name, kind, unit, what in (
-                ("single_precision_compute float", orc.CPUH_MAD_F32, "gflops",
-                 "8 work-items x 16 accumulators x 4096 fma per iteration"),
-                ("mfma_bf16", orc.CPUH_MFMA_BF16, "gflops", "4 emulated 16x16x32 bf16 products per iteration"),
-                ("mfma_int8", orc.CPUH_MFMA_I8, "gops", "4 emulated 16x16x64 int8 products per iteration"),
-                ("rocblas-fp bf16", orc.CPUH_GEMM_BF16, "gflops", "one 64x64 tile of the K=8192 bf16 GEMM per iteration")):
-            q = pool.measure(kind, SEED, 2, extra_target_us)
-            port[name] = {"ST": round(q.giga_st, 3), "MT": round(q.giga_mt, 3), "unit": unit, "threads": q.threads_mt,
-                          "iters_ST": q.iters_st, "iters_MT": q.iters_mt, "sample": what}
+        port = _port_families(orc, pool, extra_target_us)
+        r = port.pop("_headline")
         # the other two rows of the reference's DRAM test, restated (all workers only, as it times them)
         n_stream, llc = _stream_floats(cores)
         for name, kind, what in (("global_memory_bandwidth copy", 0, "memcpy of one array into another, 2 x 4 bytes per element"),

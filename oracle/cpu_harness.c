@@ -450,6 +450,115 @@ static void finish(cpuh_pool *p, cpuh_result *r, int n, double units_st, double 
     r->giga_mt = r->us_mt > 0.0 ? units_mt * (double)n / (r->us_mt * 1e3) : -1.0;
 }
 
+/* ------------------------------------------------------------------------- */
+/* Any oracle kernel on operands the caller built: one descriptor, one body.                      */
+/* The caller (the cpu_baseline leg of the benchmark driver) makes the seeded operands with the   */
+/* same generator the GPU rows use and states what one iteration is worth.                         */
+/* ------------------------------------------------------------------------- */
+int orc_smfmac(int kind, const void *Ac, const uint8_t *meta, const void *B, void *out, double *abs_out, uint32_t waves,
+               uint32_t iters);
+int orc_gemm_tile2(int fmt_a, int fmt_b, const void *A, const void *B, uint32_t K, uint32_t lda, uint32_t ldb, uint32_t m0,
+                   uint32_t n0, uint32_t tm, uint32_t tn, double scale, double *C);
+int orc_gemm_mx_tile(const uint8_t *A, const uint8_t *B, const uint8_t *SA, const uint8_t *SB, uint32_t K, uint32_t m0,
+                     uint32_t n0, uint32_t tm, uint32_t tn, double *C);
+
+enum { CPUH_OP_MAD = 0, CPUH_OP_MFMA = 1, CPUH_OP_SMFMAC = 2, CPUH_OP_GEMM = 3, CPUH_OP_GEMM_MX = 4, CPUH_OP_READ = 5 };
+
+typedef struct {
+    int op;
+    int kind;            /* MAD / MFMA / SMFMAC kind (C ABI numbering); GEMM: format of A */
+    int width;           /* MAD: width or chains; READ: vector width; GEMM: format of B */
+    uint64_t seed;       /* MAD */
+    const void *p0, *p1, *p2, *p3;   /* MFMA: A, B, scaleA, scaleB; SMFMAC: Ac, meta, B; GEMM: A, B (MX: + SA, SB); READ: buffer */
+    uint32_t K, tile;    /* GEMM: depth and tile edge */
+    double scale;        /* GEMM */
+    uint64_t n_floats, T;   /* READ: buffer length and number of partial sums */
+} cpuh_op;
+
+typedef struct {
+    cpuh_op op;
+    int n_threads;
+    size_t out_stride;   /* bytes of result space per thread */
+    uint8_t *out;
+    double sink[MAX_T];
+} op_workload;
+
+#define OP_MAD_ITEMS 8
+static void body_op(void *c, int tid, uint64_t iters)
+{
+    op_workload *w = (op_workload *)c;
+    const cpuh_op *o = &w->op;
+    void *out = w->out + (size_t)tid * w->out_stride;
+    for (uint64_t i = 0; i < iters; i++) {
+        switch (o->op) {
+        case CPUH_OP_MAD: {
+            const uint64_t first = (((uint64_t)tid << 14) + i) * OP_MAD_ITEMS % (1ull << 20);
+            orc_compute_mad(o->kind, o->width, o->seed, first, OP_MAD_ITEMS, 4096, out);
+            break;
+        }
+        case CPUH_OP_MFMA:
+            orc_mfma_dense(o->kind, o->p0, o->p1, (const uint8_t *)o->p2, (const uint8_t *)o->p3, out, NULL, 1, 1);
+            break;
+        case CPUH_OP_SMFMAC:
+            orc_smfmac(o->kind, o->p0, (const uint8_t *)o->p1, o->p2, out, NULL, 1, 1);
+            break;
+        case CPUH_OP_GEMM:
+            orc_gemm_tile2(o->kind, o->width, o->p0, o->p1, o->K, o->K, o->K, 0, 0, o->tile, o->tile, o->scale, (double *)out);
+            break;
+        case CPUH_OP_GEMM_MX:
+            orc_gemm_mx_tile((const uint8_t *)o->p0, (const uint8_t *)o->p1, (const uint8_t *)o->p2, (const uint8_t *)o->p3,
+                             o->K, 0, 0, o->tile, o->tile, (double *)out);
+            break;
+        case CPUH_OP_READ: {
+            /* this thread's contiguous share of the T partial sums; the partials are the shared result */
+            const uint64_t t0 = o->T * (uint64_t)tid / (uint64_t)w->n_threads, t1 = o->T * (uint64_t)(tid + 1) / (uint64_t)w->n_threads;
+            orc_global_bandwidth_range(o->width, (const float *)o->p0, o->n_floats, o->T, t0, t1, (float *)w->out);
+            out = (float *)w->out + t0;
+            break;
+        }
+        default:
+            return;
+        }
+        w->sink[tid] += (double)*(const uint32_t *)out;
+    }
+}
+
+/* Times the operation at 1 thread and at every worker.  units_st / units_mt: what one iteration of one thread
+ * is worth (flop, op or byte) in the two runs (they differ only where the threads split one pass: READ). */
+int cpuh_measure_op(cpuh_pool *p, const cpuh_op *op, double units_st, double units_mt, unsigned warmup, unsigned target_us,
+                    cpuh_result *r)
+{
+    if (!op || !r || op->op < CPUH_OP_MAD || op->op > CPUH_OP_READ) return -1;
+    const int n = p->n_max > MAX_T ? MAX_T : p->n_max;
+    op_workload *w = (op_workload *)calloc(1, sizeof(*w));
+    if (!w) return -3;
+    w->op = *op;
+    size_t total;
+    if (op->op == CPUH_OP_READ) {
+        w->out_stride = 0;
+        total = (size_t)op->T * sizeof(float);
+    } else {
+        w->out_stride = op->op == CPUH_OP_GEMM || op->op == CPUH_OP_GEMM_MX ? (size_t)op->tile * op->tile * sizeof(double)
+                        : op->op == CPUH_OP_MAD ? OP_MAD_ITEMS * 8 : 4 * 32 * 32 * sizeof(float);
+        total = w->out_stride * (size_t)n;
+    }
+    w->out = (uint8_t *)aligned_alloc(64, (total + 63) / 64 * 64);
+    if (!w->out) { free(w); return -3; }
+    memset(w->out, 0, total);
+    memset(r, 0, sizeof(*r));
+    w->n_threads = 1;
+    r->us_st = cpuh_run_workload(p, 1, body_op, w, warmup, target_us, 0, &r->iters_st);
+    w->n_threads = n;
+    r->us_mt = cpuh_run_workload(p, n, body_op, w, warmup, target_us, 0, &r->iters_mt);
+    finish(p, r, n, units_st, units_mt);
+    volatile double keep = 0.0;
+    for (int t = 0; t < n; t++) keep += w->sink[t];
+    (void)keep;
+    free(w->out);
+    free(w);
+    return 0;
+}
+
 /* A compute chain at 1 thread and at every worker: value = ops_per_iter * threads / (us * 1e3). */
 int cpuh_measure_chain_fn(cpuh_pool *p, cpuh_chain_fn fn, double ops_per_iter, unsigned warmup, unsigned target_us,
                           cpuh_result *r)

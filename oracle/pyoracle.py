@@ -257,6 +257,16 @@ class CpuhResult(C.Structure):
                 ("units_per_iter_mt", C.c_double), ("giga_st", C.c_double), ("giga_mt", C.c_double)]
 
 
+class CpuhOp(C.Structure):
+    _fields_ = [("op", C.c_int), ("kind", C.c_int), ("width", C.c_int), ("seed", C.c_uint64),
+                ("p0", C.c_void_p), ("p1", C.c_void_p), ("p2", C.c_void_p), ("p3", C.c_void_p),
+                ("K", C.c_uint32), ("tile", C.c_uint32), ("scale", C.c_double), ("n_floats", C.c_uint64), ("T", C.c_uint64)]
+
+
+OP_MAD, OP_MFMA, OP_SMFMAC, OP_GEMM, OP_GEMM_MX, OP_READ = range(6)
+OP_MAD_ITEMS = 8
+
+
 def _bind_harness():
     L = lib()
     if getattr(L, "_harness_bound", False):
@@ -270,6 +280,7 @@ def _bind_harness():
     L.cpuh_pick_iters.argtypes = [dbl, u32, u32, u32]; L.cpuh_pick_iters.restype = u32
     L.cpuh_time_sleep_body.argtypes = [vp, i32, u32, u32, C.POINTER(u32)]; L.cpuh_time_sleep_body.restype = dbl
     L.cpuh_measure.argtypes = [vp, i32, u64, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure.restype = i32
+    L.cpuh_measure_op.argtypes = [vp, C.POINTER(CpuhOp), dbl, dbl, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure_op.restype = i32
     L.cpuh_measure_chain_fn.argtypes = [vp, vp, dbl, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure_chain_fn.restype = i32
     L.cpuh_measure_read_fn.argtypes = [vp, vp, vp, u64, u32, u32, C.POINTER(CpuhResult)]; L.cpuh_measure_read_fn.restype = i32
     L.cpuh_measure_stream.argtypes = [vp, vp, u64, i32, u32, u32, C.POINTER(CpuhResult), vp]; L.cpuh_measure_stream.restype = i32
@@ -318,6 +329,16 @@ class CpuPool:
             raise RuntimeError(f"cpuh_measure({kind}) failed: {rc}")
         return r
 
+
+    def measure_op(self, op, units_st, units_mt=None, warmup=2, target_us=1_000_000, keep=()):
+        """Times one oracle kernel (a CpuhOp descriptor) at 1 thread and at every worker; `keep` holds the numpy
+        operands alive for the duration of the call."""
+        r = CpuhResult()
+        rc = self.L.cpuh_measure_op(self.h, C.byref(op), units_st, units_st if units_mt is None else units_mt, warmup,
+                                    target_us, C.byref(r))
+        if rc != 0:
+            raise RuntimeError(f"cpuh_measure_op({op.op}, {op.kind}) failed: {rc}")
+        return r
 
     def measure_chain_fn(self, fn_ptr, ops_per_iter, warmup=2, target_us=2_000_000):
         """Times a `double fn(uint64_t outer)` chain given as a raw function pointer."""

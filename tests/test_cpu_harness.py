@@ -170,3 +170,44 @@ def test_stream_copy_and_triad_rows(kind):
     assert r.units_per_iter_st == (2 if kind == 0 else 3) * n * 4
     assert abs(r.giga_mt - r.units_per_iter_st / (r.us_mt * 1e3)) <= 1e-6 * r.giga_mt
     assert r.giga_st == -1.0 and r.iters_st == 0          # all workers only, as the reference times these rows
+
+
+def test_measure_op_times_any_oracle_kernel_on_given_operands():
+    """cpuh_measure_op: the harness's discipline around one oracle kernel on operands the caller built.  Unit
+    accounting is the caller's: giga = units x threads / (us x 1e3); and a full-size CPU baseline families
+    table builds without a GPU."""
+    from oracle import workloads as owl
+    with orc.CpuPool(2) as pool:
+        A, B, _, _ = owl.dense_inputs(4, 1, 3)          # int8 16x16x64, the 4 chains of one wave
+        op = orc.CpuhOp(op=orc.OP_MFMA, kind=4, p0=A.ctypes.data, p1=B.ctypes.data)
+        units = 4 * 2.0 * 16 * 16 * 64
+        r = pool.measure_op(op, units, warmup=1, target_us=20_000, keep=(A, B))
+        assert r.iters_st >= 1 and r.iters_mt >= 1 and r.threads_mt == 2
+        assert abs(r.giga_st - units / (r.us_st * 1e3)) <= 1e-9 * r.giga_st
+        assert abs(r.giga_mt - units * 2 / (r.us_mt * 1e3)) <= 1e-9 * r.giga_mt
+        # the read splits one pass over the buffer among the threads
+        n, T = 1 << 20, 1 << 12
+        buf = orc.fill_f32(n, 3, owl.STREAM_BW, 0)
+        op = orc.CpuhOp(op=orc.OP_READ, width=2, p0=buf.ctypes.data, n_floats=n, T=T)
+        r = pool.measure_op(op, n * 4.0, n * 4.0 / 2, warmup=1, target_us=20_000, keep=(buf,))
+        assert r.units_per_iter_st == n * 4.0 and r.units_per_iter_mt == n * 2.0 and r.giga_mt > 0
+        with pytest.raises(RuntimeError):
+            pool.measure_op(orc.CpuhOp(op=99), 1.0)
+
+
+def test_cpu_baseline_covers_every_gpu_row_family():
+    """The families table of the benchmark driver's CPU leg names one oracle kernel per GPU row family."""
+    import bench
+    with orc.CpuPool(2) as pool:
+        port = bench._port_families(orc, pool, 30_000)   # tiny budgets: this checks coverage and plumbing, not speed
+    port.pop("_headline")
+    tests_covered = {k.split(" ")[0] for k in port}
+    for test in ("global_memory_bandwidth", "single_precision_compute", "half_precision_compute", "double_precision_compute",
+                 "mixed_precision_compute", "bfloat16_compute", "integer_compute", "integer_compute_int8_dp",
+                 "mfma_fp16", "mfma_bf16", "mfma_fp16_32x32x16", "mfma_bf16_32x32x16", "mfma_int8", "mfma_fp8", "mfma_bf8",
+                 "mfma_mxfp6_e2m3", "mfma_mxfp6_e3m2", "mfma_mxfp4", "smfmac_fp16", "smfmac_bf16", "smfmac_fp8",
+                 "smfmac_bf8", "smfmac_int8", "rocblas-fp", "rocblas-int", "hipblaslt-fp8"):
+        assert test in tests_covered, test
+    assert {"global_memory_bandwidth float", "global_memory_bandwidth float2", "global_memory_bandwidth float4",
+            "hipblaslt-fp8 fp8_e4m3", "hipblaslt-fp8 mxf4_e2m1"} <= set(port)
+    assert all(v["MT"] > 0 and v["ST"] > 0 for v in port.values())
