@@ -17,8 +17,11 @@ __device__ inline void load_to_lds(const uint8_t *gptr, uint32_t lds_dst) {
 
 // The same as instructions in the hand-scheduled loop: scalar base + per-lane 32-bit offset (no
 // vector ALU work per load), LDS destination through M0 (one wait state after writing it).
+#ifndef MI355_LOAD_LDS_BITS
+#define MI355_LOAD_LDS_BITS ""   // cache-policy bits of the slab loads (none: the default policy measured best)
+#endif
 #define MI355_LOAD_LDS(voff, sbase, m0val)                                                         \
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"                     \
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" MI355_LOAD_LDS_BITS \
                :: "v"(voff), "s"(sbase), "s"(m0val) : "memory", "m0")
 
 #define MI355_DS_READ(dst, addr, off) \
@@ -40,6 +43,22 @@ struct TileGrid {
 
 __device__ __forceinline__ void tile_at(const TileGrid &g, uint32_t round, uint32_t &tm, uint32_t &tn) {
   const uint32_t id = g.first + round * g.stride;
+#ifndef MI355_GEMM_BAND_ORDER
+  // 256 workgroups on a grid whose sides are multiples of 16 tiles: one round of the part is a square of 16x16
+  // tiles, and the squares are visited in serpentine order, so that a round needs 16 tile rows of A and 16 tile
+  // columns of B (128 MiB of bf16 at K = 8192, half of them the round before's) instead of all of A and a few
+  // columns of B: what the part re-reads from round to round stays well inside the 256 MiB last-level cache while
+  // the C tiles stream through it.  Inside a square, XCD x (workgroup id % 8) owns a block of 4 rows x 8 columns
+  // of tiles, walked column-major by its 32 workgroups: 12 slab streams per XCD, as in the general order below.
+  if (g.stride == 256u && g.tiles_m % 16u == 0u && g.tiles_n % 16u == 0u) {
+    const uint32_t xcd = g.first % 8u, i = g.first / 8u;     // i: this workgroup among the 32 of its XCD
+    const uint32_t qcols = g.tiles_n / 16u, qm = round / qcols, qr = round % qcols;
+    const uint32_t qn = (qm & 1u) ? qcols - 1u - qr : qr;
+    tm = qm * 16u + (xcd % 4u) * 4u + (i & 3u);
+    tn = qn * 16u + (xcd / 4u) * 8u + (i >> 2);
+    return;
+  }
+#endif
   uint32_t lin = id;
   if (g.total % 8u == 0u) lin = (id % 8u) * (g.total / 8u) + id / 8u;   // tiles of one XCD are consecutive
   // consecutive tiles walk down a group of 4 tile rows, then move one column right
