@@ -330,6 +330,18 @@ def power_table(dev, seconds):
     run("gemm bf16 8192^3, zero operands", lambda: dev.gemm_bf16(dA, dB, dC, M, N, K), flops, "tflops")
     for b in (dA, dB, dC):
         b.free()
+    # the 8-bit and 4-bit kinds of the same kernel, seeded
+    dA, dB, dC = dev.alloc(M * K), dev.alloc(N * K), dev.alloc(M * N * 4)
+    dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, 448.0); dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, 448.0)
+    run("gemm fp8 e4m3 8192^3, seeded operands", lambda: dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1 / 448.0, 1 / 448.0), flops, "tflops")
+    dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
+    run("gemm int8 8192^3, seeded operands", lambda: dev.gemm_i8(dA, dB, dC, M, N, K), flops, "tops")
+    dSA, dSB = dev.alloc(M * K // 32), dev.alloc(N * K // 32)
+    dev.fill_bytes(dA, M * K // 2, SEED, wl.STREAM_GEMM_A, 0, 256); dev.fill_bytes(dB, N * K // 2, SEED, wl.STREAM_GEMM_B, 0, 256)
+    dev.fill_bytes(dSA, M * K // 32, SEED, wl.STREAM_SCALE_A, 123, 9); dev.fill_bytes(dSB, N * K // 32, SEED, wl.STREAM_SCALE_B, 123, 9)
+    run("gemm block-scaled fp4 8192^3, seeded operands", lambda: dev.gemm_mxfp4(dA, dB, dSA, dSB, dC, M, N, K), flops, "tflops")
+    for b in (dA, dB, dC, dSA, dSB):
+        b.free()
     waves, iters = 2048, 4096
     clk = dev.alloc(16)
     for kind in (capi.MFMA_BF16_16x16x32, capi.MFMA_F16_32x32x16, capi.MFMA_MXFP6_E3M2):
