@@ -49,10 +49,11 @@
 // its last tile a workgroup keeps fetching (the slabs of its first tile again, which nobody
 // reads) so that every step is the same code; those loads are waited for before the wave ends.
 //
-// Tile id -> tile mapping.  Workgroups are dealt round-robin to the 8 XCDs, each
-// with its own L2, and id + k*grid stays on the XCD of id.  The mapping hands every XCD a
-// contiguous band of tile rows, so the A rows a band needs are fetched into one L2 only, and
-// walks each band in column-major order of 4-row groups so that B slabs are reused while hot.
+// Tile id -> tile mapping (tile_at in gemm_ring.h).  Workgroups are dealt round-robin to the 8 XCDs, each
+// with its own L2, and id + k*grid stays on the XCD of id.  With 256 workgroups on a grid whose sides are
+// multiples of 16 tiles, one round of the part is a square of 16x16 tiles (4x8 per XCD), squares in serpentine
+// order, so that what is re-read from round to round fits the last-level cache; other grids hand every XCD a
+// contiguous band of tile rows, walked in column-major order of 4-row groups so that B slabs are reused while hot.
 #include "internal.h"
 #include "mfma_common.h"
 #include "gemm_ring.h"
