@@ -369,6 +369,31 @@ def power_table(dev, seconds):
                 lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk), wl.sparse_flops(kind, waves, iters), "tflops")
             for b in bufs + [o]:
                 b.free()
+    # How fast the limit acts: isolated launches of increasing length (the board idle for 4 ms before each), with the
+    # clock read inside the kernel (shader cycles over a constant-rate counter, by wave 0).  A limit on average power
+    # would let a short launch from an idle board run at the boost clock.
+    for kind in (capi.MFMA_F16_32x32x16,):
+        sh = wl.DENSE[kind]
+        for zero in (False, True):
+            A, B, _, _ = wl.dense_inputs(kind, waves, SEED)
+            if zero:
+                A, B = np.zeros_like(A), np.zeros_like(B)
+            bufs = [dev.from_host(A), dev.from_host(B)]
+            o = dev.alloc(waves * 4 * sh["M"] * sh["N"] * 4)
+            for n_it in (32, 128, 512, 2048, 4096):
+                us, mhz = [], []
+                for _ in range(12):
+                    time.sleep(0.004)
+                    us.append(dev.time_launches(lambda: dev.mfma_dense(kind, bufs[0], bufs[1], None, None, o, waves, n_it, clk), 1))
+                    c = clk.download(np.uint64, 2)
+                    mhz.append(float(c[0]) / max(float(c[1]), 1.0) * 100.0)
+                us.sort(); mhz.sort()
+                row = {"workload": f"{sh['name']} {sh['shape']}, {'zero' if zero else 'seeded'} operands, isolated launch of {n_it} iterations",
+                       "us_per_launch": round(us[len(us) // 2], 1), "clock_in_kernel_mhz": round(mhz[len(mhz) // 2], 0)}
+                out.append(row)
+                print(json.dumps(row), flush=True)
+            for b in bufs + [o]:
+                b.free()
     clk.free()
     n_items, steps = 1 << 20, 4096
     o = dev.alloc(n_items * 8)
