@@ -118,6 +118,29 @@ def test_gemm_workgroups_walk_several_tiles(dev, fp8, steps):
     _check_tiles(dev, fp8, M, N, K, tiles, whole_output_finite=True)
 
 
+@pytest.mark.parametrize("M, N, K", [(4096, 4096, 128), (4096, 8192, 128), (8192, 4096, 384)])
+def test_gemm_rounds_of_16x16_tiles(dev, M, N, K):
+    """Grids whose sides are multiples of 16 tiles on a 256-CU part: a round of the part is a square of 16 x 16
+    tiles, the squares in serpentine order (one, two side by side, two on top of each other).  Every tile is
+    checked on one 128x128 quarter and no element of C keeps the NaN pattern it started with; the int8 product
+    of the same shape is compared whole, bit for bit, with an exact numpy product."""
+    if dev.props.num_cus != 256:
+        pytest.skip("the square rounds are the tile order of a 256-CU part")
+    tiles = [(m + 128 * ((m // 256 + n // 256) % 2), n + 128 * ((m // 256) % 2)) for m in range(0, M, 256) for n in range(0, N, 256)]
+    _check_tiles(dev, False, M, N, K, tiles, whole_output_finite=True)
+    dA, dB, dC = dev.alloc(M * K), dev.alloc(N * K), dev.alloc(M * N * 4)
+    dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
+    dev.memset(dC, 0xff)
+    dev.gemm_i8(dA, dB, dC, M, N, K)
+    a = dA.download(np.int8, M * K).reshape(M, K).astype(np.float64)
+    b = dB.download(np.int8, N * K).reshape(N, K).astype(np.float64)
+    want = (a @ b.T).astype(np.int32)            # |sum| <= 64 K: exact in float64
+    got = dC.download(np.int32, M * N).reshape(M, N)
+    assert np.array_equal(got, want)
+    for buf in (dA, dB, dC):
+        buf.free()
+
+
 # --- the other operand types of the same two kernels -------------------------------------------------
 E5M2_SCALE = 57344.0
 
