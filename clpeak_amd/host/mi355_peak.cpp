@@ -155,7 +155,7 @@ void Mi355Peak::runDevice(int ordinal, logger::BackendScope &backend) {
       {{"float", 1, widthNote(1)}, {"float2", 2, widthNote(2)}, {"float4", 4, widthNote(4)}, {nullptr, 0, nullptr}}};
   static const MadTest hp = {Benchmark::ComputeHP, "half_precision_compute", "Half-precision compute", "gflops",
       "The same chains in IEEE half precision; the packed form does two lanes per instruction.", MI355_MAD_F16, 2, 2,
-      {{"half", 1, "Scalar half FMA."}, {"half2", 2, "Packed half2 FMA."}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
+      {{"half", 1, "Half chains written one value at a time (the compiler issues them as packed pairs)."}, {"half2", 2, "Packed half2 FMA."}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
   static const MadTest dp = {Benchmark::ComputeDP, "double_precision_compute", "Double-precision compute", "gflops",
       "The same chains on 64-bit floats.", MI355_MAD_F64, 8, 2,
       {{"double", 1, widthNote(1)}, {"double2", 2, widthNote(2)}, {"double4", 4, widthNote(4)}, {nullptr, 0, nullptr}}};

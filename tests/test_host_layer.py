@@ -355,3 +355,17 @@ def test_reference_result_files_survive_load_and_save_byte_for_byte(host, tmp_pa
     # CSV keeps every row (it has no device properties)
     assert host.clpeak_host_resave(src.encode(), str(tmp_path / "again.csv").encode(), 2) == rows
     assert host.clpeak_host_resave(str(tmp_path / "again.csv").encode(), str(tmp_path / "c.xml").encode(), 0) == rows
+
+
+def test_shipped_mi355x_result_file_has_the_row_contract():
+    """results/AMD/Instinct_MI355X.xml is a dump of a full run of this backend on an MI355X (the reference keeps
+    such files under results/<vendor>/): same tests, units and metrics, in the same order, as the stand-in run."""
+    path = os.path.join(ROOT, "results", "AMD", "Instinct_MI355X.xml")
+    root, rows = parse_xml(path)
+    assert root.get("format_version") == "2"
+    run = root.find("run")
+    assert run.get("backend") == "ROCm" and [p.get("name") for p in run.findall("prop")] == ["Arch", "HIP", "CUs", "Wave", "VRAM"]
+    assert [(t, u, [m[0] for m in ms]) for _, t, u, ms in rows] == EXPECTED_ROWS
+    measured = {(t, m[0]): float(m[2]) for _, t, _, ms in rows for m in ms if m[1] is None}
+    assert measured[("global_memory_bandwidth", "float4")] > 6800.0          # 85 % of 8 TB/s
+    assert measured[("mfma_bf16", "mfma_bf16")] > 2125.0 and measured[("mfma_int8", "mfma_int8")] > 4250.0
