@@ -57,6 +57,7 @@
 #include "internal.h"
 #include "mfma_common.h"
 #include "gemm_ring.h"
+#include "gemm_quad.h"
 #include <utility>
 
 namespace {
@@ -505,10 +506,12 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
   return MI355_OK;
 }
 
+int g_quad = 1;
 template <int OP>
 int launch_ring(mi355_dev *dev, const char *what, const void *A, const void *B, void *C, uint32_t M,
                uint32_t N, uint32_t K, uint32_t elem, float scale) {
   if (int rc = check_shapes(dev, A, B, C, M, N, K, elem)) return rc;
+  if (g_quad) return mi355_launch_gemm_quad(dev, OP, what, A, B, C, M, N, K * elem, scale);
   if (int rc = allow_full_lds(dev, &gemm_ring_kernel<OP>, kLdsRing0 + OP)) return rc;
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
   gemm_ring_kernel<OP><<<gemm_workgroups(dev, tiles_m * tiles_n), kThreads, kRingBytes, dev->stream>>>(
@@ -530,6 +533,8 @@ int mi355_launch_gemm_mx_ring(mi355_dev *dev, const uint8_t *A, const uint8_t *B
   MI355_LAUNCH_CHECK(dev, "gemm_mxfp4");
   return MI355_OK;
 }
+
+extern "C" void mi355x_use_quad(int v) { g_quad = v; }
 
 extern "C" int mi355_gemm_bf16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C, uint32_t M,
                                uint32_t N, uint32_t K) {

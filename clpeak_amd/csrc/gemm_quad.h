@@ -1,0 +1,10 @@
+// gemm_quad.hip: the four-wave GEMM kernel behind mi355_gemm_bf16 / _f16 / _i8 / _fp8_e4m3 / _fp8_e5m2.
+#pragma once
+#include "internal.h"
+
+enum { kQuadE4m3 = 0, kQuadE5m2 = 1, kQuadBf16 = 2, kQuadF16 = 3, kQuadI8 = 4 };
+enum { kLdsQuad0 = 8 };   // first bit of mi355_dev::full_lds_allowed used by the instantiations of gemm_quad_kernel
+
+// Shapes have been checked by the caller (multiples of 256 x 256, K a multiple of 128 bytes, 16-byte aligned buffers).
+int mi355_launch_gemm_quad(mi355_dev *dev, int op, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N,
+                           uint32_t k_bytes, float scale);

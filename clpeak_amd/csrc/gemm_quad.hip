@@ -1,0 +1,405 @@
+// The 4-, 8- and 16-bit GEMM kernel:  C[M][N] = scale * A[M][K] . B[N][K]^T, both operands K-contiguous, fp32 (int32)
+// accumulation.  One workgroup of FOUR waves, one per SIMD, owns a 256x256 tile of C; a wave owns 128x128 of it,
+// 8x8 tiles of 16x16, its 256 accumulators in the accumulation registers.  K is walked in steps of one 128-byte row
+// segment (a slab: 256 rows x 128 B = 32 KiB per operand).
+//
+// What this arrangement is for.  A workgroup's slab stream (64 KiB per step, 2048 cycles of the matrix pipe) is bound
+// by latency, not by bandwidth: with the real addresses and tile order the part delivers a step's 64 KiB in 0.94 us
+// when a CU keeps 0..64 KiB in flight, in 0.67 us at 32..96 KiB and in 0.65 us from 64..128 KiB on, against 0.85 us for
+// the matrix instructions.  LDS holds 160 KiB, so at most 32 KiB of it may be "being read" at any time:
+//   * the B fragments of a step (8 fragments x 32 bytes per lane) are read in ONE BURST into a second register set
+//     during the last three rows of the step before, and their slot is free again at the next barrier;
+//   * the A fragments are streamed, row by row, two rows ahead of the matrix instructions, through four rotating
+//     register slots; the A slab being streamed is the only resident slab that is not in flight.
+// LDS is three A slots and two B slots of 32 KiB.  Slab s has its A rows in A slot s mod 3, its B rows in B slot
+// s mod 2.  A step has two barriers:
+//   Y (top of step s):    every wave has read B(s) into registers and all of A(s-1): the wave's loads of slab s+2 go
+//                         out, all 16 of them in the first row of the step, into B slot s mod 2 and A slot (s-1) mod 3;
+//   X (row 5 of step s):  every wave's loads of slab s+1 (issued a step and a half before) have landed: the burst of
+//                         B(s+1) and the reads of rows 0,1 of A(s+1) follow.
+// Between Y of one step and X of the next, 128 KiB are in flight; never less than 64 KiB.
+//
+// A step of a wave is 64 slots (row i = 0..7 of A fragments against the 8 B fragments), each slot the pair of
+// instructions on the two K halves of the slab, back to back on one accumulator (one K=128 instruction for fp8).  The
+// loop body is inline assembly; every s_waitcnt in it is part of the schedule.  The step is written once per parity
+// of s (which B register set is current), so no register is ever copied.
+#include "internal.h"
+#include "mfma_common.h"
+#include "gemm_ring.h"
+#include "gemm_quad.h"
+#include <utility>
+
+namespace {
+
+constexpr int kQuadThreads = 256;
+constexpr uint32_t kSlotA0 = 0, kSlotB0 = 3u * kSlabBytes;   // three A slots, then two B slots
+
+struct QuadFrags {
+  i32x4v b_lo[2][8], b_hi[2][8];   // two register sets of B fragments (current step / next step)
+  i32x4v a_lo[4], a_hi[4];         // four rotating A fragment slots: row i lives in slot i mod 4
+};
+
+struct QuadWalk {
+  uint32_t a_cur, a_cur_hi;  // LDS address of this lane's A fragment of row 0, first / second K half, in the slot of slab s
+  uint32_t a_nxt, a_nxt_hi;  // ... in the slot of slab s+1
+  uint32_t lane_a;           // ... within an A slot
+  uint32_t b_base, b_base_hi;   // the same for the B fragment, in B slot 0 (B slot 1 is reached through the offset field)
+  uint32_t off_cur, off_nxt, off_dst;   // byte offsets of the A slots of slabs s, s+1 and s+2 (uniform)
+  uint32_t dst_a;            // LDS destination of this wave's A rows of slab s+2 (uniform)
+  uint32_t dst_wave;         // this wave's rows within a slot (uniform)
+  uint64_t ga, gb;           // global addresses of this wave's first A / B row of slab s+2 (uniform)
+  uint32_t voff[8];          // this lane's byte offset from ga / gb for each of the wave's 8 loads of a slab
+  uint32_t first;            // the step is the first of a tile (uniform)
+};
+
+#ifdef QUAD_NO_READS
+#define Q_DS_READ(dst, addr, off) asm volatile("" : "=v"(dst) : "v"(addr), "n"(off))
+#else
+#define Q_DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#endif
+#ifdef QUAD_NO_LOADS
+#define Q_GLOAD ";"
+#else
+#define Q_GLOAD "global_load_lds_dwordx4"
+#endif
+#define Q_WAIT_LGKM(n) asm volatile("s_waitcnt lgkmcnt(%0)" :: "n"(n) : "memory")
+
+// The accumulators are the accumulation registers a[0:255], named in the instruction text: tile (i, j) of the wave is
+// a[4T : 4T+3], T = 8i + j.  The compiler is told once that they are taken (quad_claim_accumulators) and never sees them
+// as values: with 256 of 256 in use as operands of its own it finds no allocation without spills.
+//
+// One matrix instruction of a pair kind, optionally with one direct-to-LDS load riding along: M0 is set before the
+// matrix instruction (which is the wait state M0 needs before a load reads it) and the load is issued behind it.
+#define Q_INSN_BF16 "v_mfma_f32_16x16x32_bf16"
+#define Q_INSN_F16 "v_mfma_f32_16x16x32_f16"
+#define Q_INSN_I8 "v_mfma_i32_16x16x64_i8"
+#define Q_INSN_F8 "v_mfma_f32_16x16x128_f8f6f4"
+template <int OP, int T>
+__device__ __forceinline__ void q_mfma(const i32x4v &b, const i32x4v &a) {
+#define Q_PLAIN(insn) asm volatile(insn " a[%2:%3], %0, %1, a[%2:%3]" :: "v"(b), "v"(a), "n"(4 * T), "n"(4 * T + 3))
+  if constexpr (OP == kQuadBf16) Q_PLAIN(Q_INSN_BF16);
+  else if constexpr (OP == kQuadF16) Q_PLAIN(Q_INSN_F16);
+  else Q_PLAIN(Q_INSN_I8);
+#undef Q_PLAIN
+}
+template <int OP, int T, int IMM>
+__device__ __forceinline__ void q_mfma_load(const i32x4v &b, const i32x4v &a, uint32_t dst, uint32_t voff, uint64_t base) {
+#define Q_WITH_LOAD(insn)                                                                                              \
+  asm volatile("s_add_u32 m0, %4, %5\n " insn " a[%2:%3], %0, %1, a[%2:%3]\n " Q_GLOAD " %6, %7"           \
+               :: "v"(b), "v"(a), "n"(4 * T), "n"(4 * T + 3), "s"(dst), "n"(IMM), "v"(voff), "s"(base) : "memory", "m0", "scc")
+  if constexpr (OP == kQuadBf16) Q_WITH_LOAD(Q_INSN_BF16);
+  else if constexpr (OP == kQuadF16) Q_WITH_LOAD(Q_INSN_F16);
+  else Q_WITH_LOAD(Q_INSN_I8);
+#undef Q_WITH_LOAD
+}
+// fp8: one K=128 instruction on the 32-byte operands (e5m2 A: format field blgp, the A fragment being the second
+// source of the transposed product).
+template <int OP, int T>
+__device__ __forceinline__ void q_mfma8(const i32x8v &b, const i32x8v &a) {
+  if constexpr (OP == kQuadE5m2) asm volatile(Q_INSN_F8 " a[%2:%3], %0, %1, a[%2:%3] blgp:1" :: "v"(b), "v"(a), "n"(4 * T), "n"(4 * T + 3));
+  else asm volatile(Q_INSN_F8 " a[%2:%3], %0, %1, a[%2:%3]" :: "v"(b), "v"(a), "n"(4 * T), "n"(4 * T + 3));
+}
+template <int OP, int T, int IMM>
+__device__ __forceinline__ void q_mfma8_load(const i32x8v &b, const i32x8v &a, uint32_t dst, uint32_t voff, uint64_t base) {
+#define Q_WITH_LOAD8(fmt)                                                                                              \
+  asm volatile("s_add_u32 m0, %4, %5\n " Q_INSN_F8 " a[%2:%3], %0, %1, a[%2:%3]" fmt "\n " Q_GLOAD " %6, %7"            \
+               :: "v"(b), "v"(a), "n"(4 * T), "n"(4 * T + 3), "s"(dst), "n"(IMM), "v"(voff), "s"(base) : "memory", "m0", "scc")
+  if constexpr (OP == kQuadE5m2) Q_WITH_LOAD8(" blgp:1");
+  else Q_WITH_LOAD8("");
+#undef Q_WITH_LOAD8
+}
+
+constexpr bool quad_is_fp8(int op) { return op == kQuadE4m3 || op == kQuadE5m2; }
+
+// Slot P of a step of parity PAR (the B register set in use): row i = P / 8 of the A fragments, B fragment j = P % 8.
+// Besides its matrix instructions a slot carries its share of everything else a step does, so that nothing is left
+// for the boundary between two steps, where a single wave per SIMD has nothing to hide it behind:
+//   slots 0, 3, .. 45   one load each (8 of B rows, then 8 of A rows, of slab s+2): the texture path takes a load's
+//                       1 KiB in 16 cycles, the four waves' 64 KiB of a step in half of the step
+//   slots 8i            the reads of A row i+2 go out (rows 6, 7: rows 0, 1 of slab s+1), then row i must have arrived
+//   slot 40             barrier X
+//   slots 41..56        the burst of B(s+1)
+//   slots 23, 46, 47    the fetch addresses and the A slots move on; slot 57: the fragment addresses
+//   slot 60             every read has arrived; barrier Y of the NEXT step
+#define Q_PIN() __builtin_amdgcn_sched_barrier(0)
+template <int OP, int PAR, int P>
+__device__ __forceinline__ void quad_slot(QuadFrags &f, QuadWalk &w) {
+  constexpr int i = P / 8, j = P % 8, sl = i % 4, T = P;
+  if constexpr (j == 0) {
+    // (reads return in order: the count is that of the reads issued behind the one waited for)
+    if constexpr (i <= 5) {
+      Q_DS_READ(f.a_lo[(i + 2) % 4], w.a_cur, (i + 2) * 2048);
+      Q_DS_READ(f.a_hi[(i + 2) % 4], w.a_cur_hi, (i + 2) * 2048);
+    } else {
+      Q_DS_READ(f.a_lo[i - 6], w.a_nxt, (i - 6) * 2048);
+      Q_DS_READ(f.a_hi[i - 6], w.a_nxt_hi, (i - 6) * 2048);
+    }
+    if constexpr (i >= 1 && i <= 5) Q_WAIT_LGKM(4);
+    if constexpr (i == 6) Q_WAIT_LGKM(11);   // behind row 6: row 7, 7 reads of the burst, row 0 of the next slab
+    if constexpr (i == 7) Q_WAIT_LGKM(15);   // behind row 7 there are 19; the counter holds 15
+  }
+  constexpr int q = P / 3;
+  constexpr bool with_load = P % 3 == 0 && q < 16;
+  if constexpr (quad_is_fp8(OP)) {
+    const i32x8v b8 = __builtin_shufflevector(f.b_lo[PAR][j], f.b_hi[PAR][j], 0, 1, 2, 3, 4, 5, 6, 7);
+    const i32x8v a8 = __builtin_shufflevector(f.a_lo[sl], f.a_hi[sl], 0, 1, 2, 3, 4, 5, 6, 7);
+    if constexpr (with_load && q < 8) q_mfma8_load<OP, T, kSlotB0 + PAR * kSlabBytes + q * 1024>(b8, a8, w.dst_wave, w.voff[q], w.gb);
+    else if constexpr (with_load) q_mfma8_load<OP, T, (q - 8) * 1024>(b8, a8, w.dst_a, w.voff[q - 8], w.ga);
+    else q_mfma8<OP, T>(b8, a8);
+  } else {
+    if constexpr (with_load && q < 8)
+      q_mfma_load<OP, T, kSlotB0 + PAR * kSlabBytes + q * 1024>(f.b_lo[PAR][j], f.a_lo[sl], w.dst_wave, w.voff[q], w.gb);
+    else if constexpr (with_load)
+      q_mfma_load<OP, T, (q - 8) * 1024>(f.b_lo[PAR][j], f.a_lo[sl], w.dst_a, w.voff[q - 8], w.ga);
+    else
+      q_mfma<OP, T>(f.b_lo[PAR][j], f.a_lo[sl]);
+    q_mfma<OP, T>(f.b_hi[PAR][j], f.a_hi[sl]);
+  }
+  if constexpr (P == 40) {
+    // barrier X: this wave's loads of slab s+1 have landed (the 16 of slab s+2 may be in flight).  In the first step
+    // of a tile that wait was done before the stores of the tile before, which must not be counted here.
+#ifndef QUAD_NO_BARRIER
+    asm volatile("s_cmp_lg_u32 %0, 0\n s_cbranch_scc1 1f\n s_waitcnt vmcnt(16)\n1:\n s_barrier" :: "s"(w.first) : "memory", "scc");
+#endif
+  }
+  if constexpr (P >= 41 && P <= 56) {
+    // the burst: B fragment r/2, K half r%2 of slab s+1 into the other register set
+    constexpr int r = P - 41, jb = r / 2;
+    if constexpr (r % 2 == 0) Q_DS_READ(f.b_lo[PAR ^ 1][jb], w.b_base, (PAR ^ 1) * kSlabBytes + jb * 2048);
+    else Q_DS_READ(f.b_hi[PAR ^ 1][jb], w.b_base_hi, (PAR ^ 1) * kSlabBytes + jb * 2048);
+  }
+  if constexpr (P == 23) { Q_PIN(); w.gb += kRowBytes; w.first = 0; Q_PIN(); }
+  if constexpr (P == 46) { Q_PIN(); w.ga += kRowBytes; Q_PIN(); }
+  if constexpr (P == 47) {
+    Q_PIN();
+    const uint32_t t = w.off_cur;
+    w.off_cur = w.off_nxt; w.off_nxt = w.off_dst; w.off_dst = t;
+    w.dst_a = w.dst_wave + w.off_dst;
+    Q_PIN();
+  }
+  if constexpr (P == 57) {
+    Q_PIN();
+    w.a_cur = w.a_nxt; w.a_cur_hi = w.a_nxt_hi;
+    w.a_nxt = w.lane_a + w.off_nxt; w.a_nxt_hi = w.a_nxt ^ 64u;
+    Q_PIN();
+  }
+  if constexpr (P == 60) {
+    // Everything read in this step has arrived; the registers ride along so that nothing that uses them (a copy the
+    // compiler might place where control flow joins, the next step) can come before the wait.  Then barrier Y of the
+    // next step: every wave has read B(s+1) and all of A(s), whose slots the loads of the next step overwrite.
+#define Q_TIE8(x) "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
+#ifndef QUAD_NO_BARRIER
+    asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier"
+#else
+    asm volatile("s_waitcnt lgkmcnt(0)"
+#endif
+                 : Q_TIE8(f.b_lo[PAR ^ 1]), Q_TIE8(f.b_hi[PAR ^ 1]), "+v"(f.a_lo[0]), "+v"(f.a_hi[0]), "+v"(f.a_lo[1]), "+v"(f.a_hi[1])
+                 :: "memory");
+  }
+}
+
+template <int OP, int PAR, int... Ps>
+__device__ __forceinline__ void quad_step(std::integer_sequence<int, Ps...>, QuadFrags &f, QuadWalk &w) {
+  (quad_slot<OP, PAR, Ps>(f, w), ...);
+}
+
+// The accumulation registers belong to the hand-written code from here on.
+__device__ __forceinline__ void quad_claim_accumulators() {
+#define Q_A8(n) "a" #n "0", "a" #n "1", "a" #n "2", "a" #n "3", "a" #n "4", "a" #n "5", "a" #n "6", "a" #n "7", "a" #n "8", "a" #n "9"
+  asm volatile("" ::: "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", Q_A8(1), Q_A8(2), Q_A8(3), Q_A8(4), Q_A8(5), Q_A8(6),
+               Q_A8(7), Q_A8(8), Q_A8(9), Q_A8(10), Q_A8(11), Q_A8(12), Q_A8(13), Q_A8(14), Q_A8(15), Q_A8(16), Q_A8(17), Q_A8(18),
+               Q_A8(19), Q_A8(20), Q_A8(21), Q_A8(22), Q_A8(23), Q_A8(24), "a250", "a251", "a252", "a253", "a254", "a255");
+#undef Q_A8
+}
+
+// Tile T of the wave out of the accumulation registers (as raw bits), and zero in its place.
+template <int T>
+__device__ __forceinline__ i32x4v quad_take_tile() {
+  int v0, v1, v2, v3;
+  asm volatile("v_accvgpr_read_b32 %0, a[%4]\n v_accvgpr_read_b32 %1, a[%5]\n v_accvgpr_read_b32 %2, a[%6]\n v_accvgpr_read_b32 %3, a[%7]\n"
+               " v_accvgpr_write_b32 a[%4], 0\n v_accvgpr_write_b32 a[%5], 0\n v_accvgpr_write_b32 a[%6], 0\n v_accvgpr_write_b32 a[%7], 0"
+               : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3) : "n"(4 * T), "n"(4 * T + 1), "n"(4 * T + 2), "n"(4 * T + 3));
+  return (i32x4v){v0, v1, v2, v3};
+}
+template <int R>
+__device__ __forceinline__ void quad_zero_register() { asm volatile("v_accvgpr_write_b32 a[%0], 0" :: "n"(R)); }
+template <int... Rs>
+__device__ __forceinline__ void quad_zero_accumulators(std::integer_sequence<int, Rs...>) {
+  (quad_zero_register<Rs>(), ...);
+  asm volatile("s_nop 7");
+}
+
+// Store a wave's 128x128 accumulators and clear them.  A lane holds 4 consecutive N elements of one row per 16x16 tile
+// (the product is issued transposed), lane group g = lane/16 the elements 4g..4g+3.  16-bit kinds: two neighbouring
+// tiles (j, j+1) first trade halves (v_permlane16_swap exchanges the odd lane groups of tile j with the even groups of
+// tile j+1), after which a lane holds 8 consecutive elements: 16 bytes per lane, 64 contiguous bytes per row and
+// instruction.
+template <int OP, int I, int JP>
+__device__ __forceinline__ void quad_store_pair(void *__restrict__ Cout, uint32_t N, uint32_t row0, uint32_t col0, uint32_t lane, float scale) {
+  const i32x4v t0 = quad_take_tile<I * 8 + JP>(), t1 = quad_take_tile<I * 8 + JP + 1>();
+  if constexpr (OP == kQuadI8) {
+    int32_t *dst = static_cast<int32_t *>(Cout) + (size_t)(row0 + I * 16u) * N + col0 + 4u * (lane / 16u) + JP * 16u;
+    *reinterpret_cast<i32x4v *>(dst) = t0;
+    *reinterpret_cast<i32x4v *>(dst + 16) = t1;
+  } else {
+    const uint32_t g = lane / 16u;
+    const uint32_t col = col0 + 16u * (g & 1u) + 8u * (g >> 1);
+    uint32_t p[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      // (through scalar copies: __builtin_bit_cast applied to an element of a vector reads element 0)
+      const int b00 = t0[2 * h], b01 = t0[2 * h + 1], b10 = t1[2 * h], b11 = t1[2 * h + 1];
+      float x[2][2] = {{__builtin_bit_cast(float, b00), __builtin_bit_cast(float, b01)},
+                       {__builtin_bit_cast(float, b10), __builtin_bit_cast(float, b11)}};
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        if constexpr (quad_is_fp8(OP)) { x[t][0] *= scale; x[t][1] *= scale; }
+        p[t][h] = OP == kQuadF16 ? mi355_pack_f16x2(x[t][0], x[t][1]) : mi355_pack_bf16x2(x[t][0], x[t][1]);
+      }
+    }
+    const auto q01 = __builtin_amdgcn_permlane16_swap(p[0][0], p[1][0], false, false);
+    const auto q23 = __builtin_amdgcn_permlane16_swap(p[0][1], p[1][1], false, false);
+    const uint4 packed = make_uint4(q01[0], q23[0], q01[1], q23[1]);
+    *reinterpret_cast<uint4 *>(static_cast<uint16_t *>(Cout) + (size_t)(row0 + I * 16u) * N + col + JP * 16u) = packed;
+  }
+  __builtin_amdgcn_sched_barrier(0);   // one pair of tiles at a time: the fragment registers stay live, few are free
+}
+template <int OP, int... Qs>
+__device__ __forceinline__ void quad_store(std::integer_sequence<int, Qs...>, void *__restrict__ Cout, uint32_t N, uint32_t row0,
+                                           uint32_t col0, uint32_t lane, float scale) {
+  (quad_store_pair<OP, Qs / 4, 2 * (Qs % 4)>(Cout, N, row0, col0, lane, scale), ...);
+  asm volatile("s_nop 7");   // accumulation registers written by the vector unit, read next by the matrix unit
+}
+
+template <int OP>
+__global__ void __launch_bounds__(kQuadThreads)
+gemm_quad_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, void *__restrict__ C, uint32_t N, uint32_t k_bytes,
+                 float scale, uint32_t tiles_m, uint32_t tiles_n) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const uint32_t tid = threadIdx.x, lane = tid % 64;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const uint32_t wm = wave / 2, wn = wave % 2;
+  const TileGrid grid = tiles_of_workgroup(tiles_m, tiles_n);
+  const uint32_t steps = k_bytes / kRowBytes;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  QuadWalk w;
+  // global -> LDS: load q of a wave fills rows [wave*64 + 8q, +8) of a slab; lane i is position i%8 of row i/8,
+  // which holds logical chunk (i%8) ^ (row & 7) = (i%8) ^ (i/8)
+  const uint32_t lchunk = (lane % 8u) ^ (lane / 8u);
+#pragma unroll
+  for (uint32_t q = 0; q < 8; q++) w.voff[q] = (lane / 8u + 8u * q) * k_bytes + lchunk * 16u;
+  w.dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 64u * (uint32_t)kRowBytes);
+  // LDS -> fragments: row lane%16 of the wave's rows, logical chunk lane/16 (+4 for the second K half, the address
+  // with bit 6 flipped), swizzled with row & 7 = lane & 7
+  const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
+  w.lane_a = lds_base + (wm * 128u + lane % 16u) * kRowBytes + swz0;
+  w.b_base = lds_base + kSlotB0 + (wn * 128u + lane % 16u) * kRowBytes + swz0;
+  w.b_base_hi = w.b_base ^ 64u;
+  const uint64_t a_origin = (uint64_t)(uintptr_t)(A + (size_t)wave * 64u * k_bytes);
+  const uint64_t b_origin = (uint64_t)(uintptr_t)(B + (size_t)wave * 64u * k_bytes);
+
+  // the fetch stream: slabs numbered through all tiles of the workgroup (after the last tile it runs on into the
+  // first tile again, two slabs that nobody reads, so that every step is the same code)
+  uint32_t f_round = 0, f_left = steps;
+  auto rows_of = [&](uint32_t rnd) {
+    uint32_t tm, tn;
+    tile_at(grid, rnd, tm, tn);
+    w.ga = a_origin + (uint64_t)tm * kTile * k_bytes;
+    w.gb = b_origin + (uint64_t)tn * kTile * k_bytes;
+  };
+  auto next_fetch_tile = [&]() {
+    f_round = f_round + 1u == grid.mine ? 0u : f_round + 1u;
+    rows_of(f_round);
+    f_left = steps;
+  };
+  auto fetch = [&](uint32_t slot_a, uint32_t slot_b) {
+#pragma unroll
+    for (uint32_t q = 0; q < 8; q++) MI355_LOAD_LDS(w.voff[q], w.gb, w.dst_wave + kSlotB0 + slot_b * kSlabBytes + q * 1024u);
+#pragma unroll
+    for (uint32_t q = 0; q < 8; q++) MI355_LOAD_LDS(w.voff[q], w.ga, w.dst_wave + kSlotA0 + slot_a * kSlabBytes + q * 1024u);
+    w.ga += kRowBytes;
+    w.gb += kRowBytes;
+    if (--f_left == 0u) next_fetch_tile();
+  };
+  rows_of(0);
+  fetch(0, 0);
+  fetch(1, 1);
+  asm volatile("s_waitcnt vmcnt(16)\n s_barrier" ::: "memory");   // slab 0 has landed
+
+  quad_claim_accumulators();
+  quad_zero_accumulators(std::make_integer_sequence<int, 256>{});
+  QuadFrags f;
+  w.off_cur = 0; w.off_nxt = kSlabBytes; w.off_dst = 2u * kSlabBytes;
+  w.dst_a = w.dst_wave + w.off_dst;
+  w.a_cur = w.lane_a; w.a_cur_hi = w.a_cur ^ 64u;
+  w.a_nxt = w.lane_a + w.off_nxt; w.a_nxt_hi = w.a_nxt ^ 64u;
+  w.first = 0;
+  {   // what a step expects on entry: the B fragments of its slab in register set 0, rows 0,1 of its A fragments, and
+      // its barrier Y behind it
+#pragma unroll
+    for (int j = 0; j < 8; j++) { Q_DS_READ(f.b_lo[0][j], w.b_base, j * 2048); Q_DS_READ(f.b_hi[0][j], w.b_base_hi, j * 2048); }
+    Q_DS_READ(f.a_lo[0], w.a_cur, 0); Q_DS_READ(f.a_hi[0], w.a_cur_hi, 0);
+    Q_DS_READ(f.a_lo[1], w.a_cur, 2048); Q_DS_READ(f.a_hi[1], w.a_cur_hi, 2048);
+    asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier"
+                 : Q_TIE8(f.b_lo[0]), Q_TIE8(f.b_hi[0]), "+v"(f.a_lo[0]), "+v"(f.a_hi[0]), "+v"(f.a_lo[1]), "+v"(f.a_hi[1]) :: "memory");
+  }
+
+  // One countdown to the next event: the fetch stream moves on to its next tile (f_left steps from now), or the tile
+  // being multiplied is complete (left steps from now).
+  uint32_t round = 0, left = steps;
+  uint32_t span = left < f_left ? left : f_left, ev = span;
+  auto event = [&]() -> bool {   // true after the last tile
+    left -= span;
+    f_left -= span;
+    if (f_left == 0u) next_fetch_tile();   // (the step has already moved ga / gb on by a slab: overwritten here)
+    bool done = false;
+    if (left == 0u) {
+      // the wait states the compiler cannot know about, then every load of this wave (the next barrier X then needs
+      // no wait of its own, and the stores issued here do not enter its count)
+      asm volatile("s_nop 15\n s_nop 15\n s_waitcnt vmcnt(0)" ::: "memory");
+      uint32_t tm, tn;
+      tile_at(grid, round, tm, tn);
+      quad_store<OP>(std::make_integer_sequence<int, 32>{}, C, N, tm * kTile + wm * 128u + lane % 16u, tn * kTile + wn * 128u, lane, scale);
+      left = steps;
+      w.first = 1;
+      done = ++round == grid.mine;
+    }
+    span = left < f_left ? left : f_left;
+    ev = span;
+    return done;
+  };
+  constexpr auto slots = std::make_integer_sequence<int, 64>{};
+  for (;;) {
+    quad_step<OP, 0>(slots, f, w);
+    if (__builtin_expect(--ev == 0u, 0) && event()) break;
+    quad_step<OP, 1>(slots, f, w);
+    if (__builtin_expect(--ev == 0u, 0) && event()) break;
+  }
+  MI355_DRAIN_RING();
+}
+
+template <int OP>
+int launch_quad(mi355_dev *dev, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N, uint32_t k_bytes,
+                float scale) {
+  if (int rc = allow_full_lds(dev, &gemm_quad_kernel<OP>, kLdsQuad0 + OP)) return rc;
+  const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
+  gemm_quad_kernel<OP><<<gemm_workgroups(dev, tiles_m * tiles_n), kQuadThreads, kRingBytes, dev->stream>>>(
+      (const uint8_t *)A, (const uint8_t *)B, C, N, k_bytes, scale, tiles_m, tiles_n);
+  MI355_LAUNCH_CHECK(dev, what);
+  return MI355_OK;
+}
+
+}  // namespace
+
+int mi355_launch_gemm_quad(mi355_dev *dev, int op, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N,
+                           uint32_t k_bytes, float scale) {
+  switch (op) {
+    case kQuadE4m3: return launch_quad<kQuadE4m3>(dev, what, A, B, C, M, N, k_bytes, scale);
+    case kQuadE5m2: return launch_quad<kQuadE5m2>(dev, what, A, B, C, M, N, k_bytes, scale);
+    case kQuadBf16: return launch_quad<kQuadBf16>(dev, what, A, B, C, M, N, k_bytes, scale);
+    case kQuadF16: return launch_quad<kQuadF16>(dev, what, A, B, C, M, N, k_bytes, scale);
+    case kQuadI8: return launch_quad<kQuadI8>(dev, what, A, B, C, M, N, k_bytes, scale);
+  }
+  return mi355_fail(dev, MI355_ERR_ARG, "gemm: unknown operand kind %d", op);
+}
