@@ -1,33 +1,34 @@
 // Block-scaled FP4 GEMM (OCP MXFP4):  C[M][N] (bf16) = sum_k (A[m][k] * 2^(SA[m][k/32]-127)) * (B[n][k] * 2^(SB[n][k/32]-127)).
 // A and B hold e2m1 codes, two per byte, K contiguous; SA / SB hold one E8M0 byte per 32 elements.
 //
-// The product runs on the ring kernel of gemm.hip (operand kind kOpMx): the same tile walk, LDS ring, swizzle
-// and direct-to-LDS loads as the other kinds, K in steps of 128 bytes per row (256 codes, 8 scale blocks).  A
+// The product runs on the four-wave kernel of gemm_quad.hip (operand kind kQuadMx): the same tile walk, LDS slots,
+// swizzle and direct-to-LDS loads as the other kinds, K in steps of 128 bytes per row (256 codes, 8 scale blocks).  A
 // K=128 instruction takes 16 bytes per lane, one 16-byte chunk of a row, which is exactly one scale block; the
 // two instructions of a slot take chunks g and g+4 (g = lane / 16) like the two bf16 instructions of a slot.
 //
 // Scales do not pass through LDS (it is full).  Lane r+16g of a fragment must hold the scale byte of row r,
 // block g.  The pre-pass below rewrites scale_a / scale_b into that shape once per call: for every block of
-// rows that one wave multiplies (128 rows of A, 64 rows of B) and every K step, 64 lanes x 16 (8) bytes, byte
+// 128 rows (what one wave multiplies, of either operand) and every K step, 64 lanes x 16 bytes, byte
 // 2i+h of lane (r,g) being the scale of row 16i+r, block 8s+4h+g (fragment i, K half h).  The main loop then
 // fetches the scales of a step with ONE load per operand, fully coalesced, a whole step ahead, and the matrix
 // instruction picks byte 2(i%2)+h of register i/2 with its op_sel fields.  (Fetching the bytes from the
 // row-major arrays inside the loop, one gather per fragment and half, more than doubled the run time.)
-// The scale loads are what this kind pays over the fp8 kinds: 12 KiB per workgroup and step on top of the 64 KiB
-// of the slab, through the same fill path that bounds the kernel (waves that share rows load the same bytes).
+// Two waves of a workgroup share each block of rows, so every scale byte is loaded twice per workgroup: 8 KiB per
+// step on top of the 64 KiB of the slab.
 #include "internal.h"
 #include "gemm_ring.h"
+#include "gemm_quad.h"
 
 namespace {
 
 // Pre-pass: scales from row-major [rows][k32] to the per-lane order the main loop loads, both operands in one
-// launch.  One workgroup per (block of rows, 16 K steps): blocks of 128 rows of A (8 fragments of 16 rows, 16
-// bytes per lane and step), blocks of 64 rows of B (4 fragments, 8 bytes).  16 steps are 128 scale bytes of a
+// launch.  One workgroup per (block of rows, 16 K steps): blocks of 128 rows (8 fragments of 16 rows, 16
+// bytes per lane and step) for both operands.  16 steps are 128 scale bytes of a
 // row, one cache line: the rows are read once, 8 bytes per thread and fully coalesced, into LDS (row stride 136
 // bytes, so that the 16 rows of a fragment fall into 16 different banks), and each wave then builds the words
 // of every fourth step from byte reads of LDS.  (Gathering the bytes straight from global memory, two per row
 // and lane, took 9.5 us per call at 8192^3, 4 % of the product.)
-constexpr uint32_t kLayoutSteps = 16, kLayoutStride = 136;
+constexpr uint32_t kLayoutSteps = 16, kLayoutStride = 136, kLayoutFrags = 8;
 
 __global__ void __launch_bounds__(256)
 mx_scale_layout_kernel(const uint8_t *__restrict__ SA, const uint8_t *__restrict__ SB, uint8_t *__restrict__ out_a,
@@ -38,8 +39,8 @@ mx_scale_layout_kernel(const uint8_t *__restrict__ SA, const uint8_t *__restrict
   if (grp >= groups_a + groups_b) return;
   const uint8_t *S = SA;
   uint8_t *out = out_a;
-  uint32_t frags = 8;
-  if (grp >= groups_a) { grp -= groups_a; S = SB; out = out_b; frags = 4; }
+  constexpr uint32_t frags = kLayoutFrags;
+  if (grp >= groups_a) { grp -= groups_a; S = SB; out = out_b; }
   const uint32_t rb = grp / chunks, s0 = (grp % chunks) * kLayoutSteps;
   const uint32_t ns = steps - s0 < kLayoutSteps ? steps - s0 : kLayoutSteps, nrows = 16u * frags;
   for (uint32_t u = threadIdx.x; u < nrows * ns; u += blockDim.x) {
@@ -52,16 +53,14 @@ mx_scale_layout_kernel(const uint8_t *__restrict__ SA, const uint8_t *__restrict
   for (uint32_t st = wave; st < ns; st += blockDim.x / 64u) {
     uint32_t word[4] = {0, 0, 0, 0};
 #pragma unroll
-    for (uint32_t i = 0; i < 8; i++) {
-      if (i >= frags) break;
+    for (uint32_t i = 0; i < frags; i++) {
       const uint8_t *p = rows + (16u * i + r) * kLayoutStride + st * 8u + g;
       const uint32_t pair = (uint32_t)p[0] | ((uint32_t)p[4] << 8);   // K halves 0 and 1 of fragment i
       if (i % 2 == 0) word[i / 2] = pair;
       else word[i / 2] |= pair << 16;
     }
     const size_t unit = (size_t)rb * steps + s0 + st;
-    if (frags == 8) *reinterpret_cast<uint4 *>(out + (unit * 64u + lane) * 16u) = make_uint4(word[0], word[1], word[2], word[3]);
-    else *reinterpret_cast<uint2 *>(out + (unit * 64u + lane) * 8u) = make_uint2(word[0], word[1]);
+    *reinterpret_cast<uint4 *>(out + (unit * 64u + lane) * 16u) = make_uint4(word[0], word[1], word[2], word[3]);
   }
 }
 
@@ -83,10 +82,10 @@ int run_mx(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *sc
   const uint32_t k32 = K / 32u, steps = K / 256u;
   uint8_t *sal = lane_scales, *sbl = sal + (size_t)M * k32;
   const uint32_t chunks = (steps + kLayoutSteps - 1) / kLayoutSteps;
-  const uint32_t groups_a = M / 128u * chunks, groups_b = N / 64u * chunks;
+  const uint32_t groups_a = M / 128u * chunks, groups_b = N / 128u * chunks;
   mx_scale_layout_kernel<<<groups_a + groups_b, 256, 0, dev->stream>>>(scale_a, scale_b, sal, sbl, k32, steps, groups_a, groups_b);
   MI355_LAUNCH_CHECK(dev, "mx_scale_layout");
-  return mi355_launch_gemm_mx_ring(dev, A, B, sal, sbl, C, M, N, K);
+  return mi355_launch_gemm_quad_mx(dev, A, B, sal, sbl, C, M, N, K);
 }
 
 }  // namespace

@@ -37,6 +37,7 @@ constexpr uint32_t kSlotA0 = 0, kSlotB0 = 3u * kSlabBytes;   // three A slots, t
 struct QuadFrags {
   i32x4v b_lo[2][8], b_hi[2][8];   // two register sets of B fragments (current step / next step)
   i32x4v a_lo[4], a_hi[4];         // four rotating A fragment slots: row i lives in slot i mod 4
+  i32x4v sa[2], sb[2];             // block-scaled kind: the scale bytes of the current / next step (see quad_mx_scales)
 };
 
 struct QuadWalk {
@@ -50,18 +51,11 @@ struct QuadWalk {
   uint64_t ga, gb;           // global addresses of this wave's first A / B row of slab s+2 (uniform)
   uint32_t voff[8];          // this lane's byte offset from ga / gb for each of the wave's 8 loads of a slab
   uint32_t first;            // the step is the first of a tile (uniform)
+  uint64_t sa_next, sb_next; // block-scaled kind: addresses of the next step's 1 KiB of A / B scale bytes (uniform)
+  uint32_t s_off;            // ... and this lane's offset there
 };
 
-#ifdef QUAD_NO_READS
-#define Q_DS_READ(dst, addr, off) asm volatile("" : "=v"(dst) : "v"(addr), "n"(off))
-#else
 #define Q_DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
-#endif
-#ifdef QUAD_NO_LOADS
-#define Q_GLOAD ";"
-#else
-#define Q_GLOAD "global_load_lds_dwordx4"
-#endif
 #define Q_WAIT_LGKM(n) asm volatile("s_waitcnt lgkmcnt(%0)" :: "n"(n) : "memory")
 
 // The accumulators are the accumulation registers a[0:255], named in the instruction text: tile (i, j) of the wave is
@@ -85,7 +79,7 @@ __device__ __forceinline__ void q_mfma(const i32x4v &b, const i32x4v &a) {
 template <int OP, int T, int IMM>
 __device__ __forceinline__ void q_mfma_load(const i32x4v &b, const i32x4v &a, uint32_t dst, uint32_t voff, uint64_t base) {
 #define Q_WITH_LOAD(insn)                                                                                              \
-  asm volatile("s_add_u32 m0, %4, %5\n " insn " a[%2:%3], %0, %1, a[%2:%3]\n " Q_GLOAD " %6, %7"           \
+  asm volatile("s_add_u32 m0, %4, %5\n " insn " a[%2:%3], %0, %1, a[%2:%3]\n global_load_lds_dwordx4 %6, %7"           \
                :: "v"(b), "v"(a), "n"(4 * T), "n"(4 * T + 3), "s"(dst), "n"(IMM), "v"(voff), "s"(base) : "memory", "m0", "scc")
   if constexpr (OP == kQuadBf16) Q_WITH_LOAD(Q_INSN_BF16);
   else if constexpr (OP == kQuadF16) Q_WITH_LOAD(Q_INSN_F16);
@@ -102,11 +96,31 @@ __device__ __forceinline__ void q_mfma8(const i32x8v &b, const i32x8v &a) {
 template <int OP, int T, int IMM>
 __device__ __forceinline__ void q_mfma8_load(const i32x8v &b, const i32x8v &a, uint32_t dst, uint32_t voff, uint64_t base) {
 #define Q_WITH_LOAD8(fmt)                                                                                              \
-  asm volatile("s_add_u32 m0, %4, %5\n " Q_INSN_F8 " a[%2:%3], %0, %1, a[%2:%3]" fmt "\n " Q_GLOAD " %6, %7"            \
+  asm volatile("s_add_u32 m0, %4, %5\n " Q_INSN_F8 " a[%2:%3], %0, %1, a[%2:%3]" fmt "\n global_load_lds_dwordx4 %6, %7" \
                :: "v"(b), "v"(a), "n"(4 * T), "n"(4 * T + 3), "s"(dst), "n"(IMM), "v"(voff), "s"(base) : "memory", "m0", "scc")
   if constexpr (OP == kQuadE5m2) Q_WITH_LOAD8(" blgp:1");
   else Q_WITH_LOAD8("");
 #undef Q_WITH_LOAD8
+}
+
+// Block-scaled e2m1 (OCP MXFP4): a lane's 16-byte chunk is the 32 codes of one scale block, so a slot is again a pair of
+// K=128 instructions on the two K halves, each with the scale bytes of its blocks.  A wave's scale bytes of a step are
+// 16 bytes per lane and operand, byte 2i+h belonging to fragment i, K half h: the instruction takes byte
+// (op_sel + 2 * op_sel_hi) of the register it is given: op_sel = K half, op_sel_hi = parity of the fragment, register =
+// fragment / 2.  They do not pass through LDS: a pre-pass (gemm_mxfp4.hip) has written them in this order, and a step
+// loads those of the next step with one instruction per operand, its oldest loads.
+#define Q_INSN_MX "v_mfma_scale_f32_16x16x128_f8f6f4"
+template <int T, int H, int JB, int IB>
+__device__ __forceinline__ void q_mfma_mx(const i32x4v &b, const i32x4v &a, int sb, int sa) {
+  asm volatile(Q_INSN_MX " a[%2:%3], %0, %1, a[%2:%3], %4, %5 op_sel:[%6,%6,0] op_sel_hi:[%7,%8,0] cbsz:4 blgp:4"
+               :: "v"(b), "v"(a), "n"(4 * T), "n"(4 * T + 3), "v"(sb), "v"(sa), "n"(H), "n"(JB), "n"(IB));
+}
+template <int T, int JB, int IB, int IMM>
+__device__ __forceinline__ void q_mfma_mx_load(const i32x4v &b, const i32x4v &a, int sb, int sa, uint32_t dst, uint32_t voff, uint64_t base) {
+  asm volatile("s_add_u32 m0, %8, %9\n " Q_INSN_MX " a[%2:%3], %0, %1, a[%2:%3], %4, %5 op_sel:[0,0,0] op_sel_hi:[%6,%7,0] cbsz:4 blgp:4\n"
+               " global_load_lds_dwordx4 %10, %11"
+               :: "v"(b), "v"(a), "n"(4 * T), "n"(4 * T + 3), "v"(sb), "v"(sa), "n"(JB), "n"(IB), "s"(dst), "n"(IMM), "v"(voff), "s"(base)
+               : "memory", "m0", "scc");
 }
 
 constexpr bool quad_is_fp8(int op) { return op == kQuadE4m3 || op == kQuadE5m2; }
@@ -122,30 +136,54 @@ constexpr bool quad_is_fp8(int op) { return op == kQuadE4m3 || op == kQuadE5m2; 
 //   slots 23, 46, 47    the fetch addresses and the A slots move on; slot 57: the fragment addresses
 //   slot 60             every read has arrived; barrier Y of the NEXT step
 #define Q_PIN() __builtin_amdgcn_sched_barrier(0)
+constexpr int kLoadEvery = 3;   // the wave's 16 loads of a slab ride on slots 0, 3, 6, .. 45 (every 2: 5 % slower; 4: the same)
+constexpr int kAhead = 2;       // rows between the read of an A fragment and its use (at most 3: four register slots; 3: the same)
+constexpr int kSlotX = 40;      // barrier X follows this slot; the 16 reads of the burst follow it, one per slot (36, 43: the same)
+constexpr int quad_burst_reads(int from, int to) {   // reads of the burst issued in slots from..to
+  int n = 0;
+  for (int p = from; p <= to; p++) n += p > kSlotX && p <= kSlotX + 16;
+  return n;
+}
+// loads of the step's own slab that are issued before barrier X (they are the ones that may still be in flight there)
+constexpr int kKeepAtX = kSlotX / kLoadEvery + 1 < 16 ? kSlotX / kLoadEvery + 1 : 16;
+static_assert(15 * kLoadEvery + 2 <= 57, "the loads of a step and the bookkeeping behind them end before the addresses move on");
+static_assert(kAhead >= 1 && kAhead <= 3 && kSlotX + 16 < 60 && kSlotX >= 46 - 16, "schedule of a step");
 template <int OP, int PAR, int P>
 __device__ __forceinline__ void quad_slot(QuadFrags &f, QuadWalk &w) {
   constexpr int i = P / 8, j = P % 8, sl = i % 4, T = P;
   if constexpr (j == 0) {
-    // (reads return in order: the count is that of the reads issued behind the one waited for)
-    if constexpr (i <= 5) {
-      Q_DS_READ(f.a_lo[(i + 2) % 4], w.a_cur, (i + 2) * 2048);
-      Q_DS_READ(f.a_hi[(i + 2) % 4], w.a_cur_hi, (i + 2) * 2048);
+    // the reads of the A row kAhead rows on go out (past row 7: of the next slab), then this row's fragment must have
+    // arrived: reads return in order, so the count is that of the reads issued behind it (the counter holds 15)
+    constexpr int r = i + kAhead;
+    if constexpr (r <= 7) {
+      Q_DS_READ(f.a_lo[r % 4], w.a_cur, r * 2048);
+      Q_DS_READ(f.a_hi[r % 4], w.a_cur_hi, r * 2048);
     } else {
-      Q_DS_READ(f.a_lo[i - 6], w.a_nxt, (i - 6) * 2048);
-      Q_DS_READ(f.a_hi[i - 6], w.a_nxt_hi, (i - 6) * 2048);
+      Q_DS_READ(f.a_lo[r % 4], w.a_nxt, (r - 8) * 2048);
+      Q_DS_READ(f.a_hi[r % 4], w.a_nxt_hi, (r - 8) * 2048);
     }
-    if constexpr (i >= 1 && i <= 5) Q_WAIT_LGKM(4);
-    if constexpr (i == 6) Q_WAIT_LGKM(11);   // behind row 6: row 7, 7 reads of the burst, row 0 of the next slab
-    if constexpr (i == 7) Q_WAIT_LGKM(15);   // behind row 7 there are 19; the counter holds 15
+    if constexpr (i >= kAhead) {
+      constexpr int behind = 2 * kAhead + quad_burst_reads(8 * (i - kAhead), 8 * i - 1);
+      Q_WAIT_LGKM(behind < 15 ? behind : 15);
+    }
   }
-  constexpr int q = P / 3;
-  constexpr bool with_load = P % 3 == 0 && q < 16;
+  constexpr int q = P / kLoadEvery;
+  constexpr bool with_load = P % kLoadEvery == 0 && q < 16;
   if constexpr (quad_is_fp8(OP)) {
     const i32x8v b8 = __builtin_shufflevector(f.b_lo[PAR][j], f.b_hi[PAR][j], 0, 1, 2, 3, 4, 5, 6, 7);
     const i32x8v a8 = __builtin_shufflevector(f.a_lo[sl], f.a_hi[sl], 0, 1, 2, 3, 4, 5, 6, 7);
     if constexpr (with_load && q < 8) q_mfma8_load<OP, T, kSlotB0 + PAR * kSlabBytes + q * 1024>(b8, a8, w.dst_wave, w.voff[q], w.gb);
     else if constexpr (with_load) q_mfma8_load<OP, T, (q - 8) * 1024>(b8, a8, w.dst_a, w.voff[q - 8], w.ga);
     else q_mfma8<OP, T>(b8, a8);
+  } else if constexpr (OP == kQuadMx) {
+    const int sb = f.sb[PAR][j / 2], sa = f.sa[PAR][i / 2];
+    if constexpr (with_load && q < 8)
+      q_mfma_mx_load<T, j % 2, i % 2, kSlotB0 + PAR * kSlabBytes + q * 1024>(f.b_lo[PAR][j], f.a_lo[sl], sb, sa, w.dst_wave, w.voff[q], w.gb);
+    else if constexpr (with_load)
+      q_mfma_mx_load<T, j % 2, i % 2, (q - 8) * 1024>(f.b_lo[PAR][j], f.a_lo[sl], sb, sa, w.dst_a, w.voff[q - 8], w.ga);
+    else
+      q_mfma_mx<T, 0, j % 2, i % 2>(f.b_lo[PAR][j], f.a_lo[sl], sb, sa);
+    q_mfma_mx<T, 1, j % 2, i % 2>(f.b_hi[PAR][j], f.a_hi[sl], sb, sa);
   } else {
     if constexpr (with_load && q < 8)
       q_mfma_load<OP, T, kSlotB0 + PAR * kSlabBytes + q * 1024>(f.b_lo[PAR][j], f.a_lo[sl], w.dst_wave, w.voff[q], w.gb);
@@ -155,22 +193,22 @@ __device__ __forceinline__ void quad_slot(QuadFrags &f, QuadWalk &w) {
       q_mfma<OP, T>(f.b_lo[PAR][j], f.a_lo[sl]);
     q_mfma<OP, T>(f.b_hi[PAR][j], f.a_hi[sl]);
   }
-  if constexpr (P == 40) {
+  if constexpr (P == kSlotX) {
     // barrier X: this wave's loads of slab s+1 have landed (the 16 of slab s+2 may be in flight).  In the first step
     // of a tile that wait was done before the stores of the tile before, which must not be counted here.
-#ifndef QUAD_NO_BARRIER
-    asm volatile("s_cmp_lg_u32 %0, 0\n s_cbranch_scc1 1f\n s_waitcnt vmcnt(16)\n1:\n s_barrier" :: "s"(w.first) : "memory", "scc");
-#endif
+    asm volatile("s_cmp_lg_u32 %0, 0\n s_cbranch_scc1 1f\n s_waitcnt vmcnt(%1)\n1:\n s_barrier" :: "s"(w.first), "n"(kKeepAtX + (OP == kQuadMx ? 2 : 0)) : "memory", "scc");
   }
-  if constexpr (P >= 41 && P <= 56) {
+  if constexpr (P > kSlotX && P <= kSlotX + 16) {
     // the burst: B fragment r/2, K half r%2 of slab s+1 into the other register set
-    constexpr int r = P - 41, jb = r / 2;
+    constexpr int r = P - kSlotX - 1, jb = r / 2;
     if constexpr (r % 2 == 0) Q_DS_READ(f.b_lo[PAR ^ 1][jb], w.b_base, (PAR ^ 1) * kSlabBytes + jb * 2048);
     else Q_DS_READ(f.b_hi[PAR ^ 1][jb], w.b_base_hi, (PAR ^ 1) * kSlabBytes + jb * 2048);
   }
-  if constexpr (P == 23) { Q_PIN(); w.gb += kRowBytes; w.first = 0; Q_PIN(); }
-  if constexpr (P == 46) { Q_PIN(); w.ga += kRowBytes; Q_PIN(); }
-  if constexpr (P == 47) {
+  if constexpr (P == 7 * kLoadEvery + 1) { Q_PIN(); w.gb += kRowBytes; Q_PIN(); }
+  if constexpr (OP == kQuadMx && P == 5) { Q_PIN(); w.sa_next += 1024; w.sb_next += 1024; Q_PIN(); }
+  if constexpr (P == kSlotX + 1) { Q_PIN(); w.first = 0; Q_PIN(); }
+  if constexpr (P == 15 * kLoadEvery + 1) { Q_PIN(); w.ga += kRowBytes; Q_PIN(); }
+  if constexpr (P == 15 * kLoadEvery + 2) {
     Q_PIN();
     const uint32_t t = w.off_cur;
     w.off_cur = w.off_nxt; w.off_nxt = w.off_dst; w.off_dst = t;
@@ -188,18 +226,26 @@ __device__ __forceinline__ void quad_slot(QuadFrags &f, QuadWalk &w) {
     // compiler might place where control flow joins, the next step) can come before the wait.  Then barrier Y of the
     // next step: every wave has read B(s+1) and all of A(s), whose slots the loads of the next step overwrite.
 #define Q_TIE8(x) "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7])
-#ifndef QUAD_NO_BARRIER
     asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier"
-#else
-    asm volatile("s_waitcnt lgkmcnt(0)"
-#endif
-                 : Q_TIE8(f.b_lo[PAR ^ 1]), Q_TIE8(f.b_hi[PAR ^ 1]), "+v"(f.a_lo[0]), "+v"(f.a_hi[0]), "+v"(f.a_lo[1]), "+v"(f.a_hi[1])
+                 : Q_TIE8(f.b_lo[PAR ^ 1]), Q_TIE8(f.b_hi[PAR ^ 1]), "+v"(f.a_lo[0]), "+v"(f.a_hi[0]), "+v"(f.a_lo[1]), "+v"(f.a_hi[1]),
+                   "+v"(f.a_lo[2]), "+v"(f.a_hi[2])
                  :: "memory");
   }
 }
 
+__device__ __forceinline__ void quad_mx_scales(i32x4v &sa, i32x4v &sb, const QuadWalk &w) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(sa) : "v"(w.s_off), "s"(w.sa_next) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(sb) : "v"(w.s_off), "s"(w.sb_next) : "memory");
+}
+
 template <int OP, int PAR, int... Ps>
 __device__ __forceinline__ void quad_step(std::integer_sequence<int, Ps...>, QuadFrags &f, QuadWalk &w) {
+  if constexpr (OP == kQuadMx) {
+    // this step's scale bytes were requested at the top of the step before, ahead of its 16 loads into LDS (in the first
+    // step of a tile they were waited for before the stores of the tile before); then those of the next step go out
+    asm volatile("s_cmp_lg_u32 %2, 0\n s_cbranch_scc1 1f\n s_waitcnt vmcnt(16)\n1:" : "+v"(f.sa[PAR]), "+v"(f.sb[PAR]) : "s"(w.first) : "scc");
+    quad_mx_scales(f.sa[PAR ^ 1], f.sb[PAR ^ 1], w);
+  }
   (quad_slot<OP, PAR, Ps>(f, w), ...);
 }
 
@@ -274,7 +320,8 @@ __device__ __forceinline__ void quad_store(std::integer_sequence<int, Qs...>, vo
 template <int OP>
 __global__ void __launch_bounds__(kQuadThreads)
 gemm_quad_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, void *__restrict__ C, uint32_t N, uint32_t k_bytes,
-                 float scale, uint32_t tiles_m, uint32_t tiles_n) {
+                 float scale, uint32_t tiles_m, uint32_t tiles_n, const uint8_t *__restrict__ scales_a,
+                 const uint8_t *__restrict__ scales_b) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const uint32_t tid = threadIdx.x, lane = tid % 64;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
@@ -301,12 +348,18 @@ gemm_quad_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
 
   // the fetch stream: slabs numbered through all tiles of the workgroup (after the last tile it runs on into the
   // first tile again, two slabs that nobody reads, so that every step is the same code)
-  uint32_t f_round = 0, f_left = steps;
+  // Workgroups of different XCDs walk K from different starting points (and wrap around): at any moment the part then
+  // reads eight different places of every row instead of the same one.
+  uint32_t f_round = 0, f_left = steps, w_left = steps;
+  const uint32_t k_rot = (grid.first % 8u) * (steps / 8u);
   auto rows_of = [&](uint32_t rnd) {
     uint32_t tm, tn;
     tile_at(grid, rnd, tm, tn);
     w.ga = a_origin + (uint64_t)tm * kTile * k_bytes;
     w.gb = b_origin + (uint64_t)tn * kTile * k_bytes;
+    w.ga += k_rot * kRowBytes;
+    w.gb += k_rot * kRowBytes;
+    w_left = steps - k_rot;
   };
   auto next_fetch_tile = [&]() {
     f_round = f_round + 1u == grid.mine ? 0u : f_round + 1u;
@@ -320,16 +373,38 @@ gemm_quad_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
     for (uint32_t q = 0; q < 8; q++) MI355_LOAD_LDS(w.voff[q], w.ga, w.dst_wave + kSlotA0 + slot_a * kSlabBytes + q * 1024u);
     w.ga += kRowBytes;
     w.gb += kRowBytes;
+    if (--w_left == 0u) { w.ga -= k_bytes; w.gb -= k_bytes; w_left = steps; }
     if (--f_left == 0u) next_fetch_tile();
   };
+  // block-scaled kind: the stream of scale bytes, one step ahead of the multiplication and walking K the same way
+  // (per block of 128 rows and step 1 KiB, the steps of a block consecutive)
+  uint32_t s_round = 0, s_left = steps, sw_left = steps;
+  auto scales_of = [&](uint32_t rnd) {
+    uint32_t tm, tn;
+    tile_at(grid, rnd, tm, tn);
+    w.sa_next = (uint64_t)(uintptr_t)(scales_a + ((size_t)(tm * 2u + wm) * steps + k_rot) * 1024u);
+    w.sb_next = (uint64_t)(uintptr_t)(scales_b + ((size_t)(tn * 2u + wn) * steps + k_rot) * 1024u);
+    sw_left = steps - k_rot;
+    s_left = steps;
+  };
+  auto scales_wrap = [&]() { w.sa_next -= (uint64_t)steps * 1024u; w.sb_next -= (uint64_t)steps * 1024u; sw_left = steps; };
+  auto next_scale_tile = [&]() { s_round = s_round + 1u == grid.mine ? 0u : s_round + 1u; scales_of(s_round); };
+  QuadFrags f;
+  if constexpr (OP == kQuadMx) {   // the first step's scales go out first; the start below waits for every load
+    w.s_off = lane * 16u;
+    scales_of(0);
+    quad_mx_scales(f.sa[0], f.sb[0], w);
+    w.sa_next += 1024; w.sb_next += 1024;
+    if (--sw_left == 0u) scales_wrap();
+    if (--s_left == 0u) next_scale_tile();
+  }
   rows_of(0);
   fetch(0, 0);
   fetch(1, 1);
-  asm volatile("s_waitcnt vmcnt(16)\n s_barrier" ::: "memory");   // slab 0 has landed
+  asm volatile("s_waitcnt vmcnt(16)\n s_barrier" ::: "memory");   // slab 0 (and, older, the first scale bytes) has landed
 
   quad_claim_accumulators();
   quad_zero_accumulators(std::make_integer_sequence<int, 256>{});
-  QuadFrags f;
   w.off_cur = 0; w.off_nxt = kSlabBytes; w.off_dst = 2u * kSlabBytes;
   w.dst_a = w.dst_wave + w.off_dst;
   w.a_cur = w.lane_a; w.a_cur_hi = w.a_cur ^ 64u;
@@ -339,20 +414,35 @@ gemm_quad_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
       // its barrier Y behind it
 #pragma unroll
     for (int j = 0; j < 8; j++) { Q_DS_READ(f.b_lo[0][j], w.b_base, j * 2048); Q_DS_READ(f.b_hi[0][j], w.b_base_hi, j * 2048); }
-    Q_DS_READ(f.a_lo[0], w.a_cur, 0); Q_DS_READ(f.a_hi[0], w.a_cur_hi, 0);
-    Q_DS_READ(f.a_lo[1], w.a_cur, 2048); Q_DS_READ(f.a_hi[1], w.a_cur_hi, 2048);
+#pragma unroll
+    for (int r = 0; r < kAhead; r++) { Q_DS_READ(f.a_lo[r], w.a_cur, r * 2048); Q_DS_READ(f.a_hi[r], w.a_cur_hi, r * 2048); }
     asm volatile("s_waitcnt lgkmcnt(0)\n s_barrier"
-                 : Q_TIE8(f.b_lo[0]), Q_TIE8(f.b_hi[0]), "+v"(f.a_lo[0]), "+v"(f.a_hi[0]), "+v"(f.a_lo[1]), "+v"(f.a_hi[1]) :: "memory");
+                 : Q_TIE8(f.b_lo[0]), Q_TIE8(f.b_hi[0]), "+v"(f.a_lo[0]), "+v"(f.a_hi[0]), "+v"(f.a_lo[1]), "+v"(f.a_hi[1]),
+                   "+v"(f.a_lo[2]), "+v"(f.a_hi[2]) :: "memory");
   }
 
   // One countdown to the next event: the fetch stream moves on to its next tile (f_left steps from now), or the tile
   // being multiplied is complete (left steps from now).
   uint32_t round = 0, left = steps;
-  uint32_t span = left < f_left ? left : f_left, ev = span;
+  auto next_span = [&]() {
+    uint32_t m = left < f_left ? left : f_left;
+    m = m < w_left ? m : w_left;
+    if constexpr (OP == kQuadMx) { m = m < s_left ? m : s_left; m = m < sw_left ? m : sw_left; }
+    return m;
+  };
+  uint32_t span = next_span(), ev = span;
   auto event = [&]() -> bool {   // true after the last tile
     left -= span;
     f_left -= span;
+    w_left -= span;
+    if (w_left == 0u) { w.ga -= k_bytes; w.gb -= k_bytes; w_left = steps; }   // the fetch stream wraps around to the row's start
     if (f_left == 0u) next_fetch_tile();   // (the step has already moved ga / gb on by a slab: overwritten here)
+    if constexpr (OP == kQuadMx) {
+      s_left -= span;
+      sw_left -= span;
+      if (sw_left == 0u) scales_wrap();
+      if (s_left == 0u) next_scale_tile();
+    }
     bool done = false;
     if (left == 0u) {
       // the wait states the compiler cannot know about, then every load of this wave (the next barrier X then needs
@@ -365,7 +455,7 @@ gemm_quad_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
       w.first = 1;
       done = ++round == grid.mine;
     }
-    span = left < f_left ? left : f_left;
+    span = next_span();
     ev = span;
     return done;
   };
@@ -381,11 +471,11 @@ gemm_quad_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
 
 template <int OP>
 int launch_quad(mi355_dev *dev, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N, uint32_t k_bytes,
-                float scale) {
+                float scale, const uint8_t *scales_a = nullptr, const uint8_t *scales_b = nullptr) {
   if (int rc = allow_full_lds(dev, &gemm_quad_kernel<OP>, kLdsQuad0 + OP)) return rc;
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
   gemm_quad_kernel<OP><<<gemm_workgroups(dev, tiles_m * tiles_n), kQuadThreads, kRingBytes, dev->stream>>>(
-      (const uint8_t *)A, (const uint8_t *)B, C, N, k_bytes, scale, tiles_m, tiles_n);
+      (const uint8_t *)A, (const uint8_t *)B, C, N, k_bytes, scale, tiles_m, tiles_n, scales_a, scales_b);
   MI355_LAUNCH_CHECK(dev, what);
   return MI355_OK;
 }
@@ -402,4 +492,11 @@ int mi355_launch_gemm_quad(mi355_dev *dev, int op, const char *what, const void 
     case kQuadI8: return launch_quad<kQuadI8>(dev, what, A, B, C, M, N, k_bytes, scale);
   }
   return mi355_fail(dev, MI355_ERR_ARG, "gemm: unknown operand kind %d", op);
+}
+
+// The block-scaled FP4 product; the caller (gemm_mxfp4.hip) has checked the shapes and laid the scale bytes out per
+// lane, both operands in blocks of 128 rows (16 bytes per lane and step).
+int mi355_launch_gemm_quad_mx(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scales_a, const uint8_t *scales_b,
+                              uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
+  return launch_quad<kQuadMx>(dev, "gemm_mxfp4", A, B, C, M, N, K / 2u, 1.0f, scales_a, scales_b);
 }

@@ -1,5 +1,5 @@
-// The tile walk shared by the GEMM kernels (gemm.hip; gemm_f64.hip borrows the tile mapping and the loads): 256x256 tiles of C, K in steps of
-// 128 bytes per row, a ring of five 32 KiB LDS slots fed by direct global->LDS loads, persistent workgroups.
+// Shared by the GEMM kernels: 256x256 tiles of C and their order (every kernel), the direct global->LDS load (every
+// kernel), and the ring of five 32 KiB LDS slots with its persistent-workgroup tile walk (the fp32 kernel of gemm.hip).
 #pragma once
 #include "internal.h"
 
@@ -193,7 +193,7 @@ constexpr size_t kRingBytes = 5 * (size_t)kSlabBytes;   // five 32 KiB slots: al
 
 // A kernel that takes the whole LDS must be allowed to, once per device handle (the attribute belongs to
 // the function on the handle's device).  `bit` names the kernel within mi355_dev::full_lds_allowed.
-enum { kLdsF32 = 0, kLdsRing0 /* + the operand kind of gemm_ring_kernel, six of them */ };
+enum { kLdsF32 = 0 /* gemm_quad.h: kLdsQuad0 + the operand kind of gemm_quad_kernel */ };
 template <typename Kernel>
 inline int allow_full_lds(mi355_dev *dev, Kernel kernel, unsigned bit) {
   if (dev->full_lds_allowed & (1u << bit)) return MI355_OK;
@@ -202,10 +202,6 @@ inline int allow_full_lds(mi355_dev *dev, Kernel kernel, unsigned bit) {
   dev->full_lds_allowed |= 1u << bit;
   return MI355_OK;
 }
-
-// gemm.hip: the block-scaled FP4 product on the ring kernel (scale bytes already in per-lane order).
-int mi355_launch_gemm_mx_ring(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scales_a,
-                              const uint8_t *scales_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K);
 
 // One persistent workgroup per CU (a workgroup takes the whole LDS of one), never more than tiles.
 inline uint32_t gemm_workgroups(const mi355_dev *dev, uint32_t tiles) {

@@ -1,9 +1,9 @@
 """Properties of the generated gfx950 code that the hand-scheduled kernels rely on.
 
-The GEMM loop issues its LDS reads as inline assembly whose results arrive asynchronously; a
-register spill of such a result would be stored before the data has landed.  The kernel is therefore
-only correct when it fits the register file, which the compiler reports in the code object
-metadata.  hipcc cross-compiles without a GPU, so this runs on the CPU.
+The GEMM loops issue their LDS reads as inline assembly whose results arrive asynchronously; a
+register spill (or copy) of such a result would be taken before the data has landed.  The kernels are
+therefore only correct when they fit the register file, which the compiler reports in the code object
+metadata, and the four-wave kernel names its accumulation registers itself, which the instruction text shows.  hipcc cross-compiles without a GPU, so this runs on the CPU.
 """
 import os
 import re
@@ -49,41 +49,74 @@ def kernel_body(asm, name):
     return asm[start:asm.index(".Lfunc_end", start)]
 
 
+QUAD_KINDS = {  # instantiation tag in the mangled name -> (matrix instruction of the loop, how many per step and parity)
+    "ILi0E": ("v_mfma_f32_16x16x128_f8f6f4", 64),
+    "ILi1E": ("v_mfma_f32_16x16x128_f8f6f4", 64),
+    "ILi2E": ("v_mfma_f32_16x16x32_bf16", 128),
+    "ILi3E": ("v_mfma_f32_16x16x32_f16", 128),
+    "ILi4E": ("v_mfma_i32_16x16x64_i8", 128),
+    "ILi5E": ("v_mfma_scale_f32_16x16x128_f8f6f4", 128),
+}
+
+
+def _acc_range(text):
+    lo, hi = (int(x, 0) for x in text.split(":"))
+    return lo, hi
+
+
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
-def test_gemm_kernels_fit_the_register_file(tmp_path):
-    asm = device_asm(tmp_path, "gemm.hip")
+def test_gemm_quad_kernels(tmp_path):
+    """The four-wave kernel: the loop is written once per parity of the step, every matrix instruction accumulates in
+    the accumulation registers the source names (all 256 of them, tile T in a[4T:4T+3]), nothing spills, and the
+    compiler neither copies a fragment register nor touches an accumulation register of its own accord."""
+    asm = device_asm(tmp_path, "gemm_quad.hip")
     meta = kernel_metadata(asm)
-    # (kernel template, instantiation tag in the mangled name) -> the matrix instruction of its loop and how
-    # many of them the one instance of the step holds: 32 slots, one fp8 instruction or a pair per slot
-    expect = {("gemm_ring_kernel", "ILi0E"): ("v_mfma_f32_16x16x128_f8f6f4", 32),
-              ("gemm_ring_kernel", "ILi1E"): ("v_mfma_f32_16x16x128_f8f6f4", 32),
-              ("gemm_ring_kernel", "ILi2E"): ("v_mfma_f32_16x16x32_bf16", 64),
-              ("gemm_ring_kernel", "ILi3E"): ("v_mfma_f32_16x16x32_f16", 64),
-              ("gemm_ring_kernel", "ILi4E"): ("v_mfma_i32_16x16x64_i8", 64)}
-    for (kernel, tag), (insn, count) in expect.items():
-        name = next(k for k in meta if kernel + tag in k)
+    for tag, (insn, per_step) in QUAD_KINDS.items():
+        name = next(k for k in meta if "gemm_quad_kernel" + tag in k)
         m = meta[name]
-        assert m["vgpr_spill_count"] == 0, (name, m)
-        assert m["private_segment_fixed_size"] == 0, (name, m)
-        # 8 waves per workgroup, 2 per SIMD: at most 256 registers each
-        assert m["vgpr_count"] <= 256, (name, m)
-        # the whole LDS of a CU is requested at launch (dynamic), none statically
-        assert m.get("group_segment_fixed_size", 0) == 0, (name, m)
+        assert m["vgpr_spill_count"] == 0 and m.get("sgpr_spill_count", 0) == 0 and m["private_segment_fixed_size"] == 0, (name, m)
+        # one wave per SIMD: up to 512 registers, 256 of them the accumulators
+        assert m["agpr_count"] == 256 and m["vgpr_count"] <= 512, (name, m)
+        assert m.get("group_segment_fixed_size", 0) == 0, (name, m)   # the whole LDS of a CU is requested at launch
         body = kernel_body(asm, name)
-        assert body.count(insn) == count, (name, body.count(insn))
+        acc = [_acc_range(x) for x in re.findall(insn + r" a\[([0-9a-fx]+:[0-9a-fx]+)\]", body)]
+        assert len(acc) == 2 * per_step, (name, len(acc))
+        for half in (acc[:per_step], acc[per_step:]):   # the step of parity 0, then of parity 1
+            per_tile = per_step // 64
+            assert [r for r in half[::per_tile]] == [(4 * t, 4 * t + 3) for t in range(64)], name
+            if per_tile == 2:   # a pair is issued back to back on one accumulator
+                assert half[0::2] == half[1::2], name
+        # destination and addend are the same registers in every instruction
+        assert len(re.findall(insn + r" a\[([0-9a-fx:]+)\], v\[\d+:\d+\], v\[\d+:\d+\], a\[\1\]", body)) == 2 * per_step, name
         if tag == "ILi1E":
-            assert body.count("blgp:1") == count      # the e5m2 operand is the second source
-        if count == 64:   # a pair is issued back to back on one accumulator: same destination twice in a row
-            dst = re.findall(insn + r" (v\[\d+:\d+\]),", body)
-            assert len(dst) == 64 and all(dst[2 * k] == dst[2 * k + 1] for k in range(32)), name
-        # the direct-to-LDS loads: 20 in the prologue (five ring slots) + 8 per steady-state step
-        assert body.count("global_load_lds_dwordx4") >= 20 + 8, name
-        # no LDS stores at all on this path
-        assert "ds_write" not in body, name
-        # the accumulators leave through the packed conversions, two values per instruction
+            assert body.count("blgp:1") == 2 * per_step      # the e5m2 operand is the second source
+        if tag == "ILi5E":
+            assert body.count("cbsz:4 blgp:4") == 2 * per_step
+            ops = re.findall(insn + r" .* op_sel:\[(\d),(\d),0\]", body)
+            assert ops[0::2] == [("0", "0")] * per_step and ops[1::2] == [("1", "1")] * per_step, name
+            # per step one 16-byte load of scale bytes per operand (+ the same two before the loop)
+            assert len(re.findall(r"global_load_dwordx4 v\[", body)) == 2 * 3, name
+        # direct-to-LDS loads: 32 before the loop (two slabs), 16 per step
+        assert body.count("global_load_lds_dwordx4") == 32 + 2 * 16, (name, body.count("global_load_lds_dwordx4"))
+        assert "ds_write" not in body and "scratch_" not in body, name
+        # LDS reads: 16 + 2 * 2 before the loop, 32 per step
+        assert body.count("ds_read_b128") == 16 + 4 + 2 * 32, (name, body.count("ds_read_b128"))
+        # accumulation registers are read and cleared by the epilogue (one copy behind the step of either parity) and
+        # cleared once at the start, nowhere else
+        assert body.count("v_accvgpr_read_b32") == 2 * 256 and body.count("v_accvgpr_write_b32") == 3 * 256, name
+        assert "v_accvgpr_mov" not in body, name
+        # two barriers per step (+ two before the loop)
+        assert len(re.findall(r"^\s*s_barrier", body, re.M)) == 2 + 2 * 2, name
         if tag != "ILi4E":
             cvt = "v_cvt_pk_f16_f32" if tag == "ILi3E" else "v_cvt_pk_bf16_f32"
-            assert body.count(cvt) == 64, (name, body.count(cvt))   # 32 tiles x 4 values per lane
+            assert body.count(cvt) == 2 * 128, (name, body.count(cvt))   # 64 tiles x 4 values per lane, two per instruction
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_gemm_mxfp4_prepass(tmp_path):
+    meta = kernel_metadata(device_asm(tmp_path, "gemm_mxfp4.hip"))
+    name = next(k for k in meta if "mx_scale_layout_kernel" in k)
+    assert meta[name]["vgpr_spill_count"] == 0 and meta[name]["private_segment_fixed_size"] == 0
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
@@ -94,30 +127,6 @@ def test_peak_loops_do_not_spill(tmp_path, source):
     for name, m in meta.items():
         assert m.get("vgpr_spill_count", 0) == 0, (name, m)
         assert m.get("private_segment_fixed_size", 0) == 0, (name, m)
-
-
-@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
-def test_gemm_mxfp4_instantiation_of_the_ring_kernel(tmp_path):
-    """The block-scaled kind adds 12 scale registers (this step's and the next step's, written asynchronously by
-    loads) to the 128 accumulators and 96 fragment registers: it must still fit 256 without a spill."""
-    asm = device_asm(tmp_path, "gemm.hip")
-    meta = kernel_metadata(asm)
-    name = next(k for k in meta if "gemm_ring_kernelILi5E" in k)
-    m = meta[name]
-    assert m["vgpr_spill_count"] == 0 and m["private_segment_fixed_size"] == 0 and m["vgpr_count"] <= 256, m
-    body = kernel_body(asm, name)
-    insn = "v_mfma_scale_f32_16x16x128_f8f6f4"
-    assert body.count(insn) == 64 and body.count("cbsz:4 blgp:4") == 64
-    # a slot is its two K halves back to back on one accumulator, scale byte picked by op_sel
-    ops = re.findall(insn + r" (v\[\d+:\d+\]), .* op_sel:\[(\d),(\d),0\]", body)
-    assert len(ops) == 64
-    assert all(ops[2 * k][0] == ops[2 * k + 1][0] and ops[2 * k][1:] == ("0", "0") and ops[2 * k + 1][1:] == ("1", "1") for k in range(32))
-    # per step: one 16-byte load of A scales and one 8-byte load of B scales (+ the same two before the loop)
-    assert len(re.findall(r"global_load_dwordx4 v\[", body)) == 2 and len(re.findall(r"global_load_dwordx2 v\[", body)) == 2
-    assert body.count("v_cvt_pk_bf16_f32") == 64 and "ds_write" not in body
-    # the pre-pass and the entry point live in gemm_mxfp4.hip
-    meta = kernel_metadata(device_asm(tmp_path, "gemm_mxfp4.hip"))
-    assert any("mx_scale_layout_kernel" in k for k in meta)
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
