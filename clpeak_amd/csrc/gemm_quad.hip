@@ -281,7 +281,8 @@ __device__ __forceinline__ void quad_zero_accumulators(std::integer_sequence<int
 // tile j+1), after which a lane holds 8 consecutive elements: 16 bytes per lane, 64 contiguous bytes per row and
 // instruction.
 template <int OP, int I, int JP>
-__device__ __forceinline__ void quad_store_pair(void *__restrict__ Cout, uint32_t N, uint32_t row0, uint32_t col0, uint32_t lane, float scale) {
+__device__ __forceinline__ void quad_store_pair(void *__restrict__ Cout, uint32_t N, uint32_t row0, uint32_t col0, uint32_t lane, float scale,
+                                                bool c_streams) {
   const i32x4v t0 = quad_take_tile<I * 8 + JP>(), t1 = quad_take_tile<I * 8 + JP + 1>();
   if constexpr (OP == kQuadI8) {
     int32_t *dst = static_cast<int32_t *>(Cout) + (size_t)(row0 + I * 16u) * N + col0 + 4u * (lane / 16u) + JP * 16u;
@@ -306,14 +307,18 @@ __device__ __forceinline__ void quad_store_pair(void *__restrict__ Cout, uint32_
     const auto q01 = __builtin_amdgcn_permlane16_swap(p[0][0], p[1][0], false, false);
     const auto q23 = __builtin_amdgcn_permlane16_swap(p[0][1], p[1][1], false, false);
     const uint4 packed = make_uint4(q01[0], q23[0], q01[1], q23[1]);
-    *reinterpret_cast<uint4 *>(static_cast<uint16_t *>(Cout) + (size_t)(row0 + I * 16u) * N + col + JP * 16u) = packed;
+    i32x4v *dst = reinterpret_cast<i32x4v *>(static_cast<uint16_t *>(Cout) + (size_t)(row0 + I * 16u) * N + col + JP * 16u);
+    const i32x4v bits = {(int)packed.x, (int)packed.y, (int)packed.z, (int)packed.w};
+    // (as text: the compiler merges the two arms of a branch that differ only in the cache policy of a store)
+    if (c_streams) asm volatile("global_store_dwordx4 %0, %1, off nt" :: "v"(dst), "v"(bits) : "memory");
+    else *dst = bits;
   }
   __builtin_amdgcn_sched_barrier(0);   // one pair of tiles at a time: the fragment registers stay live, few are free
 }
 template <int OP, int... Qs>
 __device__ __forceinline__ void quad_store(std::integer_sequence<int, Qs...>, void *__restrict__ Cout, uint32_t N, uint32_t row0,
-                                           uint32_t col0, uint32_t lane, float scale) {
-  (quad_store_pair<OP, Qs / 4, 2 * (Qs % 4)>(Cout, N, row0, col0, lane, scale), ...);
+                                           uint32_t col0, uint32_t lane, float scale, bool c_streams) {
+  (quad_store_pair<OP, Qs / 4, 2 * (Qs % 4)>(Cout, N, row0, col0, lane, scale, c_streams), ...);
   asm volatile("s_nop 7");   // accumulation registers written by the vector unit, read next by the matrix unit
 }
 
@@ -321,7 +326,7 @@ template <int OP>
 __global__ void __launch_bounds__(kQuadThreads)
 gemm_quad_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, void *__restrict__ C, uint32_t N, uint32_t k_bytes,
                  float scale, uint32_t tiles_m, uint32_t tiles_n, const uint8_t *__restrict__ scales_a,
-                 const uint8_t *__restrict__ scales_b) {
+                 const uint8_t *__restrict__ scales_b, uint32_t c_streams) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const uint32_t tid = threadIdx.x, lane = tid % 64;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
@@ -450,7 +455,7 @@ gemm_quad_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, v
       asm volatile("s_nop 15\n s_nop 15\n s_waitcnt vmcnt(0)" ::: "memory");
       uint32_t tm, tn;
       tile_at(grid, round, tm, tn);
-      quad_store<OP>(std::make_integer_sequence<int, 32>{}, C, N, tm * kTile + wm * 128u + lane % 16u, tn * kTile + wn * 128u, lane, scale);
+      quad_store<OP>(std::make_integer_sequence<int, 32>{}, C, N, tm * kTile + wm * 128u + lane % 16u, tn * kTile + wn * 128u, lane, scale, c_streams != 0u);
       left = steps;
       w.first = 1;
       done = ++round == grid.mine;
@@ -474,8 +479,12 @@ int launch_quad(mi355_dev *dev, const char *what, const void *A, const void *B, 
                 float scale, const uint8_t *scales_a = nullptr, const uint8_t *scales_b = nullptr) {
   if (int rc = allow_full_lds(dev, &gemm_quad_kernel<OP>, kLdsQuad0 + OP)) return rc;
   const uint32_t tiles_m = M / kTile, tiles_n = N / kTile;
+  // A 16-bit C goes past the caches (non-temporal stores) when the operands alone fill the 256 MiB last-level cache: C
+  // lines kept there would only push out operand rows that the next round of tiles reads again (bf16 8192^3: 524 ->
+  // 512 us on constant, 671 -> 663 us on seeded operands; smaller operands, fp8 8192^3: 2 % slower; a 4-byte C: 10 %).
+  const uint32_t c_streams = OP != kQuadI8 && ((uint64_t)M + N) * k_bytes >= (256ull << 20) ? 1u : 0u;
   gemm_quad_kernel<OP><<<gemm_workgroups(dev, tiles_m * tiles_n), kQuadThreads, kRingBytes, dev->stream>>>(
-      (const uint8_t *)A, (const uint8_t *)B, C, N, k_bytes, scale, tiles_m, tiles_n, scales_a, scales_b);
+      (const uint8_t *)A, (const uint8_t *)B, C, N, k_bytes, scale, tiles_m, tiles_n, scales_a, scales_b, c_streams);
   MI355_LAUNCH_CHECK(dev, what);
   return MI355_OK;
 }
