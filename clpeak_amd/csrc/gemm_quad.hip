@@ -1,28 +1,35 @@
 // The 4-, 8- and 16-bit GEMM kernel:  C[M][N] = scale * A[M][K] . B[N][K]^T, both operands K-contiguous, fp32 (int32)
 // accumulation.  One workgroup of FOUR waves, one per SIMD, owns a 256x256 tile of C; a wave owns 128x128 of it,
 // 8x8 tiles of 16x16, its 256 accumulators in the accumulation registers.  K is walked in steps of one 128-byte row
-// segment (a slab: 256 rows x 128 B = 32 KiB per operand).
+// segment (a slab: 256 rows x 128 B = 32 KiB per operand).  Tiles, their order, the LDS layout of a slab (rows
+// XOR-swizzled in 16-byte chunks) and the direct global->LDS load are those of gemm_ring.h / gemm.hip.
 //
 // What this arrangement is for.  A workgroup's slab stream (64 KiB per step, 2048 cycles of the matrix pipe) is bound
 // by latency, not by bandwidth: with the real addresses and tile order the part delivers a step's 64 KiB in 0.94 us
 // when a CU keeps 0..64 KiB in flight, in 0.67 us at 32..96 KiB and in 0.65 us from 64..128 KiB on, against 0.85 us for
 // the matrix instructions.  LDS holds 160 KiB, so at most 32 KiB of it may be "being read" at any time:
 //   * the B fragments of a step (8 fragments x 32 bytes per lane) are read in ONE BURST into a second register set
-//     during the last three rows of the step before, and their slot is free again at the next barrier;
+//     during rows 5..7 of the step before, and their slot is free again at the barrier that follows;
 //   * the A fragments are streamed, row by row, two rows ahead of the matrix instructions, through four rotating
 //     register slots; the A slab being streamed is the only resident slab that is not in flight.
 // LDS is three A slots and two B slots of 32 KiB.  Slab s has its A rows in A slot s mod 3, its B rows in B slot
 // s mod 2.  A step has two barriers:
-//   Y (top of step s):    every wave has read B(s) into registers and all of A(s-1): the wave's loads of slab s+2 go
-//                         out, all 16 of them in the first row of the step, into B slot s mod 2 and A slot (s-1) mod 3;
-//   X (row 5 of step s):  every wave's loads of slab s+1 (issued a step and a half before) have landed: the burst of
-//                         B(s+1) and the reads of rows 0,1 of A(s+1) follow.
-// Between Y of one step and X of the next, 128 KiB are in flight; never less than 64 KiB.
+//   X (slot 40, row 5 of step s):  every wave's loads of slab s+1 (issued a step and a half before) have landed: the
+//                         burst of B(s+1) and the reads of rows 0,1 of A(s+1) follow;
+//   Y (slot 60 of step s):  every wave has read B(s+1) into registers and all of A(s): the wave's 16 loads of slab s+3
+//                         go out from the top of step s+1 on, into B slot (s+1) mod 2 and A slot s mod 3.
+// Between Y and the next X, 128 KiB are in flight; never less than 64 KiB.
 //
 // A step of a wave is 64 slots (row i = 0..7 of A fragments against the 8 B fragments), each slot the pair of
 // instructions on the two K halves of the slab, back to back on one accumulator (one K=128 instruction for fp8).  The
 // loop body is inline assembly; every s_waitcnt in it is part of the schedule.  The step is written once per parity
-// of s (which B register set is current), so no register is ever copied.
+// of s (which B register set is current), so no register is ever copied.  With one wave per SIMD nothing hides a
+// bubble, so everything a step does besides its matrix instructions rides on fixed slots (see quad_slot) and the
+// boundary between two steps is one countdown and a branch that is not taken.
+//
+// Workgroups of different XCDs walk K from different starting points (XCD x at step x * steps / 8, wrapping around),
+// so that at any moment the part reads eight places of every row instead of one; sums are order-independent up to
+// rounding, the int8 kind exactly.
 #include "internal.h"
 #include "mfma_common.h"
 #include "gemm_ring.h"
