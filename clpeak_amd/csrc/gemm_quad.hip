@@ -498,8 +498,12 @@ int launch_quad(mi355_dev *dev, const char *what, const void *A, const void *B, 
 
 }  // namespace
 
+// A lane's offsets within its wave's 64 rows of a slab are 32-bit: a row may be at most 64 MiB long.
+constexpr uint32_t kMaxRowBytes = 64u << 20;
+
 int mi355_launch_gemm_quad(mi355_dev *dev, int op, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N,
                            uint32_t k_bytes, float scale) {
+  MI355_REQUIRE(dev, k_bytes <= kMaxRowBytes, "%s: a row of K is %u bytes, the kernel takes at most %u", what, k_bytes, kMaxRowBytes);
   switch (op) {
     case kQuadE4m3: return launch_quad<kQuadE4m3>(dev, what, A, B, C, M, N, k_bytes, scale);
     case kQuadE5m2: return launch_quad<kQuadE5m2>(dev, what, A, B, C, M, N, k_bytes, scale);
@@ -514,5 +518,6 @@ int mi355_launch_gemm_quad(mi355_dev *dev, int op, const char *what, const void 
 // lane, both operands in blocks of 128 rows (16 bytes per lane and step).
 int mi355_launch_gemm_quad_mx(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scales_a, const uint8_t *scales_b,
                               uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
+  MI355_REQUIRE(dev, K / 2u <= kMaxRowBytes, "gemm_mxfp4: a row of K is %u bytes, the kernel takes at most %u", K / 2u, kMaxRowBytes);
   return launch_quad<kQuadMx>(dev, "gemm_mxfp4", A, B, C, M, N, K / 2u, 1.0f, scales_a, scales_b);
 }

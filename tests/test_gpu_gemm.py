@@ -106,11 +106,13 @@ def test_gemm_non_square_grid_visits_every_tile_once(dev, fp8):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
-@pytest.mark.parametrize("steps", [1, 2, 5])
+@pytest.mark.parametrize("steps", [1, 2, 5, 9, 16, 19])
 def test_gemm_workgroups_walk_several_tiles(dev, fp8, steps):
     """17 x 16 = 272 tiles on a 256-CU part: workgroups are persistent, 16 of them own two tiles and the
-    ring runs through the tile boundary (with 1 and 2 steps per tile the fetch streams are a whole tile
-    or more ahead of the tile being multiplied).  Every 256x256 tile is checked on one 128x128 quarter,
+    fetch stream runs through the tile boundary (with 1 and 2 steps per tile it is a whole tile
+    or more ahead of the tile being multiplied).  From 8 steps on, every XCD starts its walk along K at a place of
+    its own and wraps around inside the tile; an odd number of steps makes a workgroup's second tile start on the
+    other copy of the step.  Every 256x256 tile is checked on one 128x128 quarter,
     and no element of C keeps the NaN pattern it started with."""
     M, N, K = 17 * 256, 16 * 256, steps * (128 if fp8 else 64)
     assert (M // 256) * (N // 256) > dev.props.num_cus
@@ -326,7 +328,7 @@ def test_gemm_mxfp4_grids_and_full_size(dev):
     _check_mx(dev, 8192, 8192, 8192, tiles)
 
 
-@pytest.mark.parametrize("steps", [1, 2, 5])
+@pytest.mark.parametrize("steps", [1, 2, 5, 9, 16])
 def test_gemm_mxfp4_workgroups_walk_several_tiles(dev, steps):
     """272 tiles on a 256-CU part (see test_gemm_workgroups_walk_several_tiles): the A, B and scale streams
     each cross the tile boundary at their own distance ahead of the tile being multiplied."""
@@ -334,6 +336,17 @@ def test_gemm_mxfp4_workgroups_walk_several_tiles(dev, steps):
     assert (M // 256) * (N // 256) > dev.props.num_cus
     tiles = [(m + 128 * ((m // 256 + n // 256) % 2), n + 128 * ((m // 256) % 2)) for m in range(0, M, 256) for n in range(0, N, 256)]
     _check_mx(dev, M, N, K, tiles, whole_output_finite=True)
+
+
+def test_gemm_refuses_rows_longer_than_its_offsets_reach(dev):
+    """A lane addresses its wave's 64 rows of a slab with 32-bit offsets: rows of K longer than 64 MiB are refused
+    before anything is launched (the buffers here are never touched)."""
+    small = dev.alloc(1 << 20)
+    K = (64 << 20) // 2 + 64      # bf16: 64 MiB + 128 bytes per row
+    with pytest.raises(capi.Mi355Error) as err:
+        dev.gemm_bf16(small, small, small, 256, 256, K)
+    assert err.value.code == capi.ERR_ARG and "at most" in str(err.value)
+    small.free()
 
 
 # --- the reference's own GEMM inputs ---------------------------------------------------------------------
