@@ -247,7 +247,9 @@ int mi355_mfma_raw(mi355_dev *dev, int sparse, int kind,
  * (src/rocm/rocblas.cpp:122-342 row "bf16"; src/rocm/hipblaslt_gemm.cpp:214-525 row
  * "fp8_e4m3"; both with K contiguous in A and B, fp32 accumulation, bf16 output).
  *   A[M][K] row-major, B[N][K] (column-major B), C[M][N] row-major bf16.
- * M, N multiples of 256, K a multiple of 64.  fp8: C = scale_a*scale_b * (A.B). */
+ * M, N multiples of 256, K a multiple of 128 bytes (64 bf16 values, 128 fp8 values) and a row of
+ * K at most 64 MiB; buffers 16-byte aligned.  fp8: C = scale_a*scale_b * (A.B).  Sums along K are
+ * formed in an order that depends on the tile (results agree within rounding; int8 exactly). */
 int mi355_gemm_bf16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C,
                     uint32_t M, uint32_t N, uint32_t K);
 int mi355_gemm_fp8_e4m3(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C,
