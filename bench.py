@@ -77,6 +77,8 @@ def bench_rows(dev, quick, only):
         _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=False, one_set=True, reference=True)
     if "gemm" in only:
         _gemm_rows(dev, capi, wl, add, budget, constant=False)
+    if "vendor" in only:
+        _vendor_rows(dev, capi, wl, add, budget)
     if "gemm_const" in only:
         _gemm_rows(dev, capi, wl, add, budget, constant=True)
     if "lds" in only:
@@ -237,6 +239,78 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
             metric += " constant operands"
         us, _ = timed(dev, fn, **budget)
         add(test, metric, 2.0 * M * N * K / us / 1e6, unit, us, PEAK[peak], shape="8192x8192x8192")
+        for b in (dA, dB, dC):
+            b.free()
+
+
+def _vendor_rows(dev, capi, wl, add, budget):
+    """The vendor library the reference's GEMM rows call (rocBLAS / hipBLASLt, reached here through torch.matmul,
+    torch._scaled_mm and torch._int_mm), timed in this process on this board right beside this library's kernel of the
+    same row, on operands of the same distribution (uniform [-1,1) rounded to the type; int8 uniform in [-8,7]) and on
+    the reference's constant fill.  Not part of the default rows: it needs torch, whose first import takes a minute."""
+    import time
+    import torch
+    M = N = K = 8192
+    flops = 2.0 * M * N * K
+
+    def t_torch(fn):
+        torch.cuda.synchronize()
+        t0 = time.time()
+        while time.time() - t0 < budget.get("warm_us", 300e3) / 1e6:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+        reps = max(10, int(budget.get("min_us", 300e3) / 600.0))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    g = torch.Generator(device="cuda")
+    g.manual_seed(SEED & 0x7fffffff)
+    one = torch.ones((), device="cuda")
+    cases = [("rocblas-fp", "bf16", torch.bfloat16, "bf16", "tflops", 0x3f), ("rocblas-fp", "fp16", torch.float16, "f16", "tflops", 0x3f),
+             ("hipblaslt-fp8", "fp8_e4m3", torch.float8_e4m3fn, "fp8", "tflops", 0x38), ("rocblas-int", "int8", torch.int8, "int8", "tops", 0x3f)]
+    for test, metric, dt, peak, unit, const_byte in cases:
+        if dt == torch.int8:
+            A = torch.randint(-8, 8, (M, K), device="cuda", dtype=dt, generator=g); B = torch.randint(-8, 8, (N, K), device="cuda", dtype=dt, generator=g)
+            fn = lambda: torch._int_mm(A, B.t())
+        elif dt == torch.float8_e4m3fn:
+            A = ((torch.rand(M, K, device="cuda", generator=g) * 2 - 1) * 448).to(dt); B = ((torch.rand(N, K, device="cuda", generator=g) * 2 - 1) * 448).to(dt)
+            fn = lambda: torch._scaled_mm(A, B.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+        else:
+            A = (torch.rand(M, K, device="cuda", generator=g) * 2 - 1).to(dt); B = (torch.rand(N, K, device="cuda", generator=g) * 2 - 1).to(dt)
+            fn = lambda: torch.matmul(A, B.t())
+        for what in ("uniform random operands", "constant operands"):
+            if what.startswith("constant"):
+                A.view(torch.uint8).fill_(const_byte); B.view(torch.uint8).fill_(const_byte)
+            us = t_torch(fn)
+            add(test, f"{metric} vendor library, {what}", flops / us / 1e6, unit, us, PEAK[peak], shape="8192x8192x8192")
+        del A, B
+        torch.cuda.empty_cache()
+        # this library's kernel of the same row, right behind it on the same board
+        eb, ob = (2, 2) if dt in (torch.bfloat16, torch.float16) else (1, 4 if dt == torch.int8 else 2)
+        dA, dB, dC = dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * ob)
+        if metric == "bf16":
+            dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            mine = lambda: dev.gemm_bf16(dA, dB, dC, M, N, K)
+        elif metric == "fp16":
+            dev.fill_f16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_f16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            mine = lambda: dev.gemm_f16(dA, dB, dC, M, N, K)
+        elif metric == "fp8_e4m3":
+            dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, 448.0); dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, 448.0)
+            mine = lambda: dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1.0, 1.0)
+        else:
+            dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
+            mine = lambda: dev.gemm_i8(dA, dB, dC, M, N, K)
+        for what in ("seeded operands", "constant operands"):
+            if what.startswith("constant"):
+                dev.memset(dA, const_byte); dev.memset(dB, const_byte)
+            us, _ = timed(dev, mine, **budget)
+            add(test, f"{metric} this library, {what}", flops / us / 1e6, unit, us, PEAK[peak], shape="8192x8192x8192")
         for b in (dA, dB, dC):
             b.free()
 
@@ -584,8 +658,13 @@ def main():
                     help="run only the power / clock telemetry: each matrix workload for SECONDS while board power and "
                          "shader clock are sampled from sysfs every 10 ms; one JSON line per workload")
     ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer",
-                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer")
+                    help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer; "
+                         "and, not among the defaults, vendor: the vendor library's GEMM beside this library's (needs torch)")
     args = ap.parse_args()
+    if "vendor" in args.only.split(","):
+        # torch brings a HIP runtime of its own: it has to be the one that initialises the device in this process
+        import torch
+        torch.cuda.init()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; the hot path has no multi-GPU step "
                  "(every kernel is independent per device), run with --gpus 1")
