@@ -120,7 +120,7 @@ def test_gemm_workgroups_walk_several_tiles(dev, fp8, steps):
     _check_tiles(dev, fp8, M, N, K, tiles, whole_output_finite=True)
 
 
-@pytest.mark.parametrize("M, N, K", [(4096, 4096, 128), (4096, 8192, 128), (8192, 4096, 384)])
+@pytest.mark.parametrize("M, N, K", [(4096, 4096, 128), (4096, 8192, 128), (8192, 4096, 384), (4096, 4096, 19 * 128)])
 def test_gemm_rounds_of_16x16_tiles(dev, M, N, K):
     """Grids whose sides are multiples of 16 tiles on a 256-CU part: a round of the part is a square of 16 x 16
     tiles, the squares in serpentine order (one, two side by side, two on top of each other).  Every tile is
