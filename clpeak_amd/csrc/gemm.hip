@@ -183,6 +183,8 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
   MI355_REQUIRE(dev, A && B && C, "gemm: null buffer");
   MI355_REQUIRE(dev, M > 0 && N > 0 && K > 0, "gemm: empty problem");
   MI355_REQUIRE(dev, M % kTile == 0 && N % kTile == 0, "gemm: M (%u) and N (%u) must be multiples of 256", M, N);
+  MI355_REQUIRE(dev, (uint64_t)K * elem <= (64u << 20), "gemm: a row of K is %llu bytes, the kernels take at most 64 MiB (32-bit lane offsets)",
+                (unsigned long long)K * elem);
   MI355_REQUIRE(dev, (K * elem) % kRowBytes == 0, "gemm: K (%u) must be a multiple of %u", K, kRowBytes / elem);
   MI355_REQUIRE(dev, (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) == 0, "gemm: buffers must be 16-byte aligned");
   return MI355_OK;

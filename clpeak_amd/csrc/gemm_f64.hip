@@ -142,6 +142,8 @@ extern "C" int mi355_gemm_f64(mi355_dev *dev, const double *A, const double *B, 
   MI355_REQUIRE(dev, A && B && C, "gemm_f64: null buffer");
   MI355_REQUIRE(dev, M > 0 && N > 0 && K > 0, "gemm_f64: empty problem");
   MI355_REQUIRE(dev, M % kTile64 == 0 && N % kTile64 == 0, "gemm_f64: M (%u) and N (%u) must be multiples of 128", M, N);
+  MI355_REQUIRE(dev, (uint64_t)K * 8u <= (64u << 20), "gemm_f64: a row of K is %llu bytes, the kernel takes at most 64 MiB (32-bit lane offsets)",
+                (unsigned long long)K * 8u);
   MI355_REQUIRE(dev, K % 16 == 0, "gemm_f64: K (%u) must be a multiple of 16", K);
   MI355_REQUIRE(dev, (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 31u) == 0, "gemm_f64: buffers must be 32-byte aligned");
   const uint32_t tiles_m = M / kTile64, tiles_n = N / kTile64;
