@@ -112,6 +112,91 @@ def test_gemm_quad_kernels(tmp_path):
             assert body.count(cvt) == 2 * 128, (name, body.count(cvt))   # 64 tiles x 4 values per lane, two per instruction
 
 
+def _reg_range(text):
+    """'v[10:13]' -> range(10, 14); 'v7' -> range(7, 8)"""
+    m = re.match(r"v\[(\d+):(\d+)\]$", text)
+    if m:
+        return range(int(m.group(1)), int(m.group(2)) + 1)
+    return range(int(text[1:]), int(text[1:]) + 1)
+
+
+def _steps_of(body, insn):
+    """The two copies of the step (parity 0, parity 1) as lists of instruction lines: a step runs from behind the last
+    matrix instruction of what precedes it to its own last one (on the last accumulator tile, a[252:255])."""
+    lines = [l.strip() for l in body.splitlines()]
+    lines = [l for l in lines if l and not l.startswith(";")]
+    last = [i for i, l in enumerate(lines) if l.startswith(insn) and re.search(r"a\[(0xfc|252):(0xff|255)\]", l)]
+    first = [i for i, l in enumerate(lines) if l.startswith(insn) and re.search(r" a\[0:3\]", l)]
+    ends = [i for k, i in enumerate(last) if k + 1 == len(last) or last[k + 1] != i + 1]     # last of a run on that tile
+    assert len(ends) == 2, ends
+    starts = [first[0], next(i for i in first if i > ends[0])]
+    steps = []
+    for k in range(2):
+        begin = starts[k]
+        while not (lines[begin - 1].startswith(insn) or lines[begin - 1].startswith("s_barrier") or re.match(r"\.LBB", lines[begin - 1])
+                   or lines[begin - 1].startswith("s_cbranch") or lines[begin - 1].startswith("s_branch")):
+            begin -= 1          # the reads and address arithmetic in front of the step's first matrix instruction
+        steps.append(lines[begin:ends[k] + 1])
+    return steps
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+@pytest.mark.parametrize("tag", ["ILi2E", "ILi0E", "ILi5E"])
+def test_gemm_quad_schedule_waits_for_what_it_uses(tmp_path, tag):
+    """A replay of the step as the compiler emitted it, with the two in-order queues the hardware keeps: LDS reads
+    (lgkmcnt) and vector-memory loads (vmcnt).  No matrix instruction may name a register that a read or load still in
+    flight will write; at barrier X exactly the loads the step itself has issued may be in flight; and the registers the
+    burst of one step fills are the B operands of the other step."""
+    asm = device_asm(tmp_path, "gemm_quad.hip")
+    meta = kernel_metadata(asm)
+    insn, per_step = QUAD_KINDS[tag]
+    name = next(k for k in meta if "gemm_quad_kernel" + tag in k)
+    steps = _steps_of(kernel_body(asm, name), insn)
+    b_sources, burst_dests = [], []
+    for step in steps:
+        lgkm, vm = [], []          # destinations (register ranges) of the operations in flight, oldest first
+        mfma_seen = loads_before_x = x_seen = 0
+        b_src, dests_after_x = set(), set()
+        for line in step:
+            op = line.split()[0]
+            if op == "ds_read_b128":
+                dest = _reg_range(line.split()[1].rstrip(","))
+                lgkm.append(dest)
+                if x_seen:
+                    dests_after_x.update(dest)
+            elif op.startswith("global_load_lds"):
+                vm.append(range(0))
+                loads_before_x += not x_seen
+            elif op.startswith("global_load_dword"):
+                vm.append(_reg_range(line.split()[1].rstrip(",")))
+                loads_before_x += not x_seen
+            elif op == "s_waitcnt":
+                m = re.search(r"lgkmcnt\((\d+)\)", line)
+                if m:
+                    lgkm = lgkm[max(0, len(lgkm) - int(m.group(1))):]
+                m = re.search(r"vmcnt\((\d+)\)", line)
+                if m:
+                    keep = int(m.group(1))
+                    if mfma_seen:      # the wait of barrier X (the block-scaled kind's wait at the top comes before any)
+                        assert keep == loads_before_x, (name, keep, loads_before_x)
+                        x_seen = 1
+                    vm = vm[max(0, len(vm) - keep):]
+            elif op == insn:
+                mfma_seen += 1
+                srcs = re.findall(r"v\[\d+:\d+\]|\bv\d+\b", line)
+                in_flight = {r for d in lgkm + vm for r in d}
+                for src in srcs:
+                    assert not in_flight & set(_reg_range(src)), (name, mfma_seen, line)
+                b_src.update(_reg_range(srcs[0]))
+        assert mfma_seen == per_step and x_seen, (name, mfma_seen, x_seen)
+        assert not lgkm, (name, "reads still in flight at the end of the step", len(lgkm))
+        b_sources.append(b_src)
+        burst_dests.append(dests_after_x)
+    # behind X a step reads the other step's B fragments (16 x 4 registers) and rows 0, 1 of its A fragments (16 more)
+    for k in range(2):
+        assert len(b_sources[k]) == 64 and b_sources[k] <= burst_dests[1 - k] and len(burst_dests[1 - k]) == 64 + 16, name
+
+
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
 def test_gemm_mxfp4_prepass(tmp_path):
     meta = kernel_metadata(device_asm(tmp_path, "gemm_mxfp4.hip"))
