@@ -207,6 +207,58 @@ def test_gemm_other_types_8192_sampled_tiles(dev, kind):
     _check_kind(dev, kind, 8192, 8192, 8192, tiles)
 
 
+def _decode(fmt, codes):
+    """Codes of one of the oracle's formats as float64 (through the oracle's own decoder, which the CPU tests pin)."""
+    return orc.decode(fmt, codes).astype(np.float64)
+
+
+@pytest.mark.parametrize("kind", ["bf16", "f16", "e4m3", "i8"])
+def test_gemm_random_shapes_every_element(dev, kind):
+    """Six seeded shapes (tile grids from 1 x 1 to 6 x 5, K walks of 1 to 40 steps, mostly odd): the WHOLE of C against a
+    numpy float64 product of the decoded operands.  Catches what sampled tiles cannot: a tile or a K step visited twice
+    or never, anywhere in the grid."""
+    rng = np.random.default_rng(11)
+    eb = 2 if kind in ("bf16", "f16") else 1
+    for _ in range(6):
+        M, N = 256 * int(rng.integers(1, 7)), 256 * int(rng.integers(1, 6))
+        K = int(rng.integers(1, 41)) * (128 // eb)
+        dA, dB, dC = dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * (4 if kind == "i8" else 2))
+        dev.memset(dC, 0xff)
+        if kind == "bf16":
+            dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            dev.gemm_bf16(dA, dB, dC, M, N, K); fmt, scale = orc.FMT_BF16, 1.0
+        elif kind == "f16":
+            dev.fill_f16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_f16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            dev.gemm_f16(dA, dB, dC, M, N, K); fmt, scale = orc.FMT_F16, 1.0
+        elif kind == "e4m3":
+            dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, FP8_SCALE); dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, FP8_SCALE)
+            dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1.0 / FP8_SCALE, 1.0 / FP8_SCALE); fmt, scale = orc.FMT_E4M3, 1.0 / (FP8_SCALE * FP8_SCALE)
+        else:
+            dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
+            dev.gemm_i8(dA, dB, dC, M, N, K); fmt, scale = None, 1.0
+        if kind == "i8":
+            a = dA.download(np.int8, M * K).astype(np.float64).reshape(M, K)
+            b = dB.download(np.int8, N * K).astype(np.float64).reshape(N, K)
+        else:
+            in_dt = np.uint16 if eb == 2 else np.uint8
+            codes = np.arange(1 << (8 * eb), dtype=np.uint32)
+            table = _decode(fmt, codes)            # every code of the format once, then a lookup
+            a = table[dA.download(in_dt, M * K)].reshape(M, K)
+            b = table[dB.download(in_dt, N * K)].reshape(N, K)
+        ref = (a @ b.T) * scale
+        if kind == "i8":
+            got = dC.download(np.int32, M * N).reshape(M, N).astype(np.float64)
+            assert np.array_equal(got, ref), (M, N, K)
+        else:
+            raw = dC.download(np.uint16, M * N)
+            got = (raw.view(np.float16) if kind == "f16" else (raw.astype(np.uint32) << 16).view(np.float32)).astype(np.float64).reshape(M, N)
+            rms = float(np.sqrt((ref ** 2).mean()))
+            assert np.all(np.isfinite(got)), (M, N, K)
+            assert np.all(np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-2 * rms), (M, N, K, float(np.abs(got - ref).max()), rms)
+        for buf in (dA, dB, dC):
+            buf.free()
+
+
 # --- fp32 and fp64: the accumulation type is the operand type ---------------------------------------------
 def _check_wide(dev, kind, M, N, K, tiles, tile=128):
     """kind in f32 / f64.  Bar: |gpu - ref| <= 4 sqrt(K) eps (|ref| + rms(ref tile)), eps = 2^-24 / 2^-53: K
