@@ -15,7 +15,9 @@ of the workload list).  `value` is its throughput in GB/s.  The same line carrie
   fracs         one fraction of datasheet peak per target kernel (taken from the rows below);
   rows (file)   every other kernel of the backend (float/float2 reads, MAD chains, launch
                 latency, dense MFMA, 2:4 SMFMAC, GEMM, LDS, PCIe transfers) with its absolute figure, the
-                MI355X datasheet peak it is compared with and the fraction reached.
+                MI355X datasheet peak it is compared with and the fraction reached; and, measured first by a
+                child process on the same board, the vendor library's bf16 / fp8 GEMM of the same shape (what the
+                reference's GEMM rows call; skipped without torch or with --no-vendor).
 
 One GPU only: the path has no exchange step, every unit of work is independent, so more
 GPUs would simply run the same kernels side by side.
@@ -62,26 +64,34 @@ def bench_rows(dev, quick, only):
         r.update(extra)
         rows.append(r)
 
+    progress("rows: " + ",".join(sorted(only)))
     if "mad" in only:
         _mad_rows(dev, capi, add, budget)
     if "latency" in only:
         us = dev.launch_roundtrip(2, 10000)
         add("kernel_launch_latency", "roundtrip", us, "us", us)
     if "mfma" in only or "smfmac" in only:
+        progress("mfma rows")
         _matrix_rows(dev, wl, add, budget, only, zero=False, one_set=True)
     if "matrix_distinct" in only:
+        progress("matrix_distinct rows")
         _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=False, one_set=False)
     if "matrix_zero" in only:
+        progress("matrix_zero rows")
         _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=True, one_set=True)
     if "matrix_ref" in only:
+        progress("matrix_ref rows")
         _matrix_rows(dev, wl, add, budget, ("mfma", "smfmac"), zero=False, one_set=True, reference=True)
     if "gemm" in only:
+        progress("gemm rows")
         _gemm_rows(dev, capi, wl, add, budget, constant=False)
     if "vendor" in only:
         _vendor_rows(dev, capi, wl, add, budget)
     if "gemm_const" in only:
+        progress("gemm_const rows")
         _gemm_rows(dev, capi, wl, add, budget, constant=True)
     if "lds" in only:
+        progress("lds rows")
         _lds_rows(dev, add, budget)
     if "transfer" in only:
         _transfer_rows(dev, capi, add, budget)
@@ -366,6 +376,73 @@ class _Telemetry:
         m = [c for t, _, c in self.samples if c is not None and t - t0 >= skip_s]
         return {"samples": len(w), "watts_mean": round(sum(w) / len(w), 1) if w else None, "watts_max": round(max(w), 1) if w else None,
                 "sclk_mhz_mean": round(sum(m) / len(m), 0) if m else None, "sclk_mhz_min": min(m) if m else None}
+
+
+def _vendor_child():
+    """Child-process leg: the vendor library's bf16 and fp8 GEMM at 8192^3 on uniform random operands, through
+    torch.matmul / torch._scaled_mm (hipBLASLt), one JSON line {"bf16": us, "fp8_e4m3": us}.  A process of its own
+    because torch brings a HIP runtime that has to be the one to initialise the device in its process."""
+    import torch
+    M = N = K = 8192
+    g = torch.Generator(device="cuda")
+    g.manual_seed(SEED & 0x7fffffff)
+    one = torch.ones((), device="cuda")
+    out = {}
+
+    def t_torch(fn, warm_s=0.3, run_s=0.3):
+        torch.cuda.synchronize()
+        t0 = time.time()
+        while time.time() - t0 < warm_s:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+        reps = max(10, int(run_s * 1e6 / 600.0))
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    A = (torch.rand(M, K, device="cuda", generator=g) * 2 - 1).to(torch.bfloat16)
+    B = (torch.rand(N, K, device="cuda", generator=g) * 2 - 1).to(torch.bfloat16)
+    out["bf16"] = t_torch(lambda: torch.matmul(A, B.t()))
+    del A, B
+    try:
+        A = ((torch.rand(M, K, device="cuda", generator=g) * 2 - 1) * 448).to(torch.float8_e4m3fn)
+        B = ((torch.rand(N, K, device="cuda", generator=g) * 2 - 1) * 448).to(torch.float8_e4m3fn)
+        out["fp8_e4m3"] = t_torch(lambda: torch._scaled_mm(A, B.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16))
+    except Exception as e:   # an older torch without the fp8 product: the bf16 figure stands alone
+        sys.stderr.write(f"bench.py: vendor fp8 product not available: {e!r}\n")
+    print(json.dumps(out), flush=True)
+
+
+def vendor_beside(timeout_s=150):
+    """Rows of the vendor library's GEMM (what the reference's rocblas-fp / hipblaslt-fp8 rows call) measured on this
+    board by a child process, or [] when torch is missing, slow to load or fails: a comparison, never a dependency.
+    Runs before this process touches the GPU."""
+    import subprocess
+    try:
+        r = subprocess.run([sys.executable, os.path.abspath(__file__), "--vendor-child"], capture_output=True, text=True, timeout=timeout_s)
+        got = json.loads(r.stdout.strip().splitlines()[-1]) if r.returncode == 0 and r.stdout.strip() else {}
+    except (subprocess.TimeoutExpired, OSError, ValueError) as e:
+        sys.stderr.write(f"bench.py: vendor library leg skipped: {e!r}\n")
+        return []
+    rows, flops = [], 2.0 * 8192 ** 3
+    for key, test, peak in (("bf16", "rocblas-fp", "bf16"), ("fp8_e4m3", "hipblaslt-fp8", "fp8")):
+        if key in got:
+            us = float(got[key])
+            rows.append({"test": test, "metric": f"{key} vendor library, uniform random operands", "value": round(flops / us / 1e6, 2),
+                         "unit": "tflops", "us_per_launch": round(us, 2), "peak": PEAK[peak], "frac": round(flops / us / 1e6 / PEAK[peak], 4),
+                         "shape": "8192x8192x8192"})
+    return rows
+
+
+def progress(what):
+    """A line on stderr per phase: a reader that takes a silent run for a hung one sees this one move."""
+    sys.stderr.write(f"bench.py [{time.strftime('%H:%M:%S')}] {what}\n")
+    sys.stderr.flush()
 
 
 def power_table(dev, seconds):
@@ -660,7 +737,12 @@ def main():
     ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer",
                     help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer; "
                          "and, not among the defaults, vendor: the vendor library's GEMM beside this library's (needs torch)")
+    ap.add_argument("--no-vendor", action="store_true", help="skip the vendor library's bf16 / fp8 GEMM beside this library's (a child process that imports torch)")
+    ap.add_argument("--vendor-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
+    if args.vendor_child:
+        _vendor_child()
+        return
     if "vendor" in args.only.split(","):
         # torch brings a HIP runtime of its own: it has to be the one that initialises the device in this process
         import torch
@@ -669,6 +751,10 @@ def main():
         sys.exit("bench.py: this build measures one GPU; the hot path has no multi-GPU step "
                  "(every kernel is independent per device), run with --gpus 1")
 
+    vendor = []
+    if not (args.no_rows or args.no_vendor or args.power_table or args.calibrate_copy or "gemm" not in args.only.split(",")):
+        progress("vendor library's bf16 / fp8 GEMM in a child process (torch)")
+        vendor = vendor_beside()
     from clpeak_amd import capi
     from clpeak_amd import workloads as wl
     dev = capi.Device(0)
@@ -717,7 +803,10 @@ def main():
     src.free(); out.free()
     if not args.no_rows:
         rows += bench_rows(dev, args.quick, set(args.only.split(",")))
+    rows += vendor
     dev.close()
+    if not args.no_cpu:
+        progress("CPU baseline leg")
 
     achieved = n * 4 / kernel_us / 1e3
     full = {
@@ -773,6 +862,8 @@ FRAC_KEYS = [("hbm_float", "global_memory_bandwidth", "float"), ("hbm_float2", "
              ("gemm_fp8_e4m3_seeded", "hipblaslt-fp8", "fp8_e4m3"), ("gemm_fp8_e5m2_seeded", "hipblaslt-fp8", "fp8_e5m2"),
              ("gemm_mxfp4_seeded", "hipblaslt-fp8", "mxf4_e2m1"), ("gemm_int8_seeded", "rocblas-int", "int8"),
              ("gemm_bf16_const", "rocblas-fp", "bf16 constant operands"),
+             ("gemm_bf16_vendor", "rocblas-fp", "bf16 vendor library, uniform random operands"),
+             ("gemm_fp8_vendor", "hipblaslt-fp8", "fp8_e4m3 vendor library, uniform random operands"),
              ("lds_float4", "local_memory_bandwidth", "float4")]
 
 
