@@ -463,3 +463,42 @@ def test_gemm_on_the_reference_fills(dev, kind):
         assert np.all(dC.download(np.uint16, M * N) == _bf16_bits_of(total)), (kind, total)
     for b in (dA, dB, dC):
         b.free()
+
+
+@pytest.mark.parametrize("kind", ["bf16", "e4m3", "i8", "mx"])
+def test_gemm_same_bits_from_launch_to_launch(dev, kind):
+    """4096^3 (256 tiles: every workgroup busy, 64 / 32 / 16 K steps per tile), launched three times back to back, six
+    times over: C is the same bits every time.  Nothing in the kernel depends on timing unless a wave reads a slab or
+    a fragment before it has landed, or a slot is overwritten while another wave still reads it; such a launch would
+    differ from its neighbours now and then."""
+    import zlib
+    M = N = K = 4096
+    eb, cb = (2 if kind == "bf16" else 1), (4 if kind == "i8" else 2)
+    if kind == "mx":
+        bufs = [dev.alloc(M * K // 2), dev.alloc(N * K // 2), dev.alloc(M * N * 2), dev.alloc(M * K // 32), dev.alloc(N * K // 32)]
+        dA, dB, dC, dSA, dSB = bufs
+        dev.fill_bytes(dA, M * K // 2, SEED, wl.STREAM_GEMM_A, 0, 256); dev.fill_bytes(dB, N * K // 2, SEED, wl.STREAM_GEMM_B, 0, 256)
+        dev.fill_bytes(dSA, M * K // 32, SEED, wl.STREAM_SCALE_A, 123, 9); dev.fill_bytes(dSB, N * K // 32, SEED, wl.STREAM_SCALE_B, 123, 9)
+        launch = lambda: dev.gemm_mxfp4(dA, dB, dSA, dSB, dC, M, N, K)
+    else:
+        bufs = [dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * cb)]
+        dA, dB, dC = bufs
+        if kind == "bf16":
+            dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            launch = lambda: dev.gemm_bf16(dA, dB, dC, M, N, K)
+        elif kind == "e4m3":
+            dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, FP8_SCALE); dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, FP8_SCALE)
+            launch = lambda: dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1.0 / FP8_SCALE, 1.0 / FP8_SCALE)
+        else:
+            dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
+            launch = lambda: dev.gemm_i8(dA, dB, dC, M, N, K)
+    seen = set()
+    for _ in range(6):
+        dev.memset(dC, 0xff)
+        for _ in range(3):
+            launch()
+        dev.sync()
+        seen.add(zlib.crc32(dC.download(np.uint8, M * N * cb).tobytes()))
+    assert len(seen) == 1, seen
+    for b in bufs:
+        b.free()
