@@ -16,7 +16,7 @@ of the workload list).  `value` is its throughput in GB/s.  The same line carrie
   rows (file)   every other kernel of the backend (float/float2 reads, MAD chains, launch
                 latency, dense MFMA, 2:4 SMFMAC, GEMM, LDS, PCIe transfers) with its absolute figure, the
                 MI355X datasheet peak it is compared with and the fraction reached; and, measured first by a
-                child process on the same board, the vendor library's bf16 / fp8 GEMM of the same shape (what the
+                child process on the same board, the vendor library's bf16 / fp8 / block-scaled FP4 GEMM of the same shape (what the
                 reference's GEMM rows call; skipped without torch or with --no-vendor).
 
 One GPU only: the path has no exchange step, every unit of work is independent, so more
@@ -379,8 +379,9 @@ class _Telemetry:
 
 
 def _vendor_child():
-    """Child-process leg: the vendor library's bf16 and fp8 GEMM at 8192^3 on uniform random operands, through
-    torch.matmul / torch._scaled_mm (hipBLASLt), one JSON line {"bf16": us, "fp8_e4m3": us}.  A process of its own
+    """Child-process leg: the vendor library's bf16, fp8 and block-scaled FP4 GEMM at 8192^3 on uniform random operands
+    (FP4: uniform codes under scales 2^-4 .. 2^4, as this library's row), through torch.matmul / torch._scaled_mm
+    (hipBLASLt), one JSON line {"bf16": us, "fp8_e4m3": us, "mxf4_e2m1": us}.  A process of its own
     because torch brings a HIP runtime that has to be the one to initialise the device in its process."""
     import torch
     M = N = K = 8192
@@ -415,6 +416,15 @@ def _vendor_child():
         out["fp8_e4m3"] = t_torch(lambda: torch._scaled_mm(A, B.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16))
     except Exception as e:   # an older torch without the fp8 product: the bf16 figure stands alone
         sys.stderr.write(f"bench.py: vendor fp8 product not available: {e!r}\n")
+    try:
+        del A, B
+        A = torch.randint(0, 256, (M, K // 2), device="cuda", dtype=torch.uint8, generator=g).view(torch.float4_e2m1fn_x2)
+        B = torch.randint(0, 256, (N, K // 2), device="cuda", dtype=torch.uint8, generator=g).view(torch.float4_e2m1fn_x2)
+        sa = torch.randint(123, 132, (M, K // 32), device="cuda", dtype=torch.uint8, generator=g).view(torch.float8_e8m0fnu)
+        sb = torch.randint(123, 132, (N, K // 32), device="cuda", dtype=torch.uint8, generator=g).view(torch.float8_e8m0fnu)
+        out["mxf4_e2m1"] = t_torch(lambda: torch._scaled_mm(A, B.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16))
+    except Exception as e:
+        sys.stderr.write(f"bench.py: vendor block-scaled FP4 product not available: {e!r}\n")
     print(json.dumps(out), flush=True)
 
 
@@ -430,7 +440,7 @@ def vendor_beside(timeout_s=150):
         sys.stderr.write(f"bench.py: vendor library leg skipped: {e!r}\n")
         return []
     rows, flops = [], 2.0 * 8192 ** 3
-    for key, test, peak in (("bf16", "rocblas-fp", "bf16"), ("fp8_e4m3", "hipblaslt-fp8", "fp8")):
+    for key, test, peak in (("bf16", "rocblas-fp", "bf16"), ("fp8_e4m3", "hipblaslt-fp8", "fp8"), ("mxf4_e2m1", "hipblaslt-fp8", "fp4")):
         if key in got:
             us = float(got[key])
             rows.append({"test": test, "metric": f"{key} vendor library, uniform random operands", "value": round(flops / us / 1e6, 2),
@@ -737,7 +747,7 @@ def main():
     ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer",
                     help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer; "
                          "and, not among the defaults, vendor: the vendor library's GEMM beside this library's (needs torch)")
-    ap.add_argument("--no-vendor", action="store_true", help="skip the vendor library's bf16 / fp8 GEMM beside this library's (a child process that imports torch)")
+    ap.add_argument("--no-vendor", action="store_true", help="skip the vendor library's bf16 / fp8 / FP4 GEMM beside this library's (a child process that imports torch)")
     ap.add_argument("--vendor-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
     if args.vendor_child:
@@ -753,7 +763,7 @@ def main():
 
     vendor = []
     if not (args.no_rows or args.no_vendor or args.power_table or args.calibrate_copy or "gemm" not in args.only.split(",")):
-        progress("vendor library's bf16 / fp8 GEMM in a child process (torch)")
+        progress("vendor library's bf16 / fp8 / block-scaled FP4 GEMM in a child process (torch)")
         vendor = vendor_beside()
     from clpeak_amd import capi
     from clpeak_amd import workloads as wl
@@ -864,6 +874,7 @@ FRAC_KEYS = [("hbm_float", "global_memory_bandwidth", "float"), ("hbm_float2", "
              ("gemm_bf16_const", "rocblas-fp", "bf16 constant operands"),
              ("gemm_bf16_vendor", "rocblas-fp", "bf16 vendor library, uniform random operands"),
              ("gemm_fp8_vendor", "hipblaslt-fp8", "fp8_e4m3 vendor library, uniform random operands"),
+             ("gemm_mxfp4_vendor", "hipblaslt-fp8", "mxf4_e2m1 vendor library, uniform random operands"),
              ("lds_float4", "local_memory_bandwidth", "float4")]
 
 
