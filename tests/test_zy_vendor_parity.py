@@ -2,9 +2,9 @@
 
 The reference's GEMM rows call rocBLAS / hipBLASLt (src/rocm/rocblas.cpp:122-342, src/rocm/hipblaslt_gemm.cpp:262-520);
 the hand-written kernels take their place, so their results are held to that library's here: torch.matmul,
-torch._scaled_mm and torch._int_mm reach the same hipBLASLt on this image.  1024 x 768 x 4096, every element of C:
-int8 equal, the floating kinds within 1e-2 (relative to the element and to the rms of C: the two sum in different
-orders and round once to the 16-bit output).  The block-scaled FP4 case also says that both read the scale bytes as
+torch._scaled_mm and torch._int_mm reach the same libraries on this image.  All eight rows (bf16, fp16, fp32, fp64, fp8 e4m3, e5m2 x e4m3, int8, block-scaled
+FP4), 1024 x 768 x 4096, every element of C: int8 equal, the 16-bit outputs within 1e-2 (relative to the element and to
+the rms of C: the two sum in different orders and round once to the output type), fp32 within 1e-5, fp64 within 1e-13.  The block-scaled FP4 case also says that both read the scale bytes as
 plain row-major [rows][K / 32] arrays.
 
 The comparison runs in a child process (tests/vendor_parity_child.py): torch's HIP runtime has to be the one that
