@@ -6,8 +6,12 @@
 // 128x128 tiles, 4 waves of 64x64 (16 accumulator tiles of 4 doubles per lane = 128 registers), two LDS
 // buffers of 32 KiB per workgroup, two workgroups per CU, one barrier per step (in its middle, between the
 // two K halves, so that every LDS read lands under 32 matrix instructions), and the loads of the next slab
-// in flight for a whole step.  It shares the LDS layout with its siblings (rows of 128
-// bytes, chunk c of row r at position c ^ (r & 7), global memory straight into LDS).
+// in flight for a whole step.  The fragment reads of one K half ride on the matrix instructions of the other, one
+// read behind every second of its first 16 instructions (all 8 in a burst in front of them: 1 % slower; with no
+// reads at all the loop would be another 1 % faster, with no barrier not at all), which fixes the order of the
+// instructions: they are written as text, the accumulators in the accumulation registers.  It shares the LDS
+// layout with its siblings (rows of 128 bytes, chunk c of row r at position c ^ (r & 7), global memory straight
+// into LDS).
 //
 // A lane's 16-byte fragment read is chunk lane/16 (+4 for the second K half) of its row, two doubles;
 // double t of it is the operand of the t-th of two instructions, so lane group g supplies
@@ -35,22 +39,38 @@ typedef double f64x4v __attribute__((ext_vector_type(4)));
 #define MI355_WAIT_FRAGS64(fa, fb)                                                                 \
   asm volatile("s_waitcnt lgkmcnt(0)"                                                              \
                : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]))
-#define MI355_WAIT_FRAGS64_BUT8(fa, fb)                                                            \
-  asm volatile("s_waitcnt lgkmcnt(8)"                                                              \
-               : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]), "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]))
 #define MI355_READ_FRAGS64(fa, fb, a_addr, b_addr)                                                 \
   MI355_DS_READ64(fb[0], b_addr, 0); MI355_DS_READ64(fb[1], b_addr, 2048);                         \
   MI355_DS_READ64(fb[2], b_addr, 4096); MI355_DS_READ64(fb[3], b_addr, 6144);                      \
   MI355_DS_READ64(fa[0], a_addr, 0); MI355_DS_READ64(fa[1], a_addr, 2048);                         \
   MI355_DS_READ64(fa[2], a_addr, 4096); MI355_DS_READ64(fa[3], a_addr, 6144)
 
-__device__ __forceinline__ void mfma_sweep(f64x4v (&acc)[4][4], const f64x2v (&fa)[4], const f64x2v (&fb)[4]) {
+// The 32 matrix instructions of one K half (fragments fa, fb), and riding on the first 16 of them, one behind every
+// second, the 8 reads of the other fragment set (ra, rb) for the half after this one.
+__device__ __forceinline__ void mfma_sweep(f64x4v (&acc)[4][4], const f64x2v (&fa)[4], const f64x2v (&fb)[4], f64x2v (&ra)[4],
+                                           f64x2v (&rb)[4], uint32_t a_addr, uint32_t b_addr, bool reads) {
 #pragma unroll
   for (int t = 0; t < 2; t++)
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-      for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fb[j][t], fa[i][t], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < 4; j++) {
+        const double b = fb[j][t], a = fa[i][t];
+        asm volatile("v_mfma_f64_16x16x4_f64 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b), "v"(a));
+        const int n = t * 16 + i * 4 + j;
+        if (n % 2 == 0 && n < 16 && reads) {
+          switch (n / 2) {
+            case 0: MI355_DS_READ64(rb[0], b_addr, 0); break;
+            case 1: MI355_DS_READ64(rb[1], b_addr, 2048); break;
+            case 2: MI355_DS_READ64(rb[2], b_addr, 4096); break;
+            case 3: MI355_DS_READ64(rb[3], b_addr, 6144); break;
+            case 4: MI355_DS_READ64(ra[0], a_addr, 0); break;
+            case 5: MI355_DS_READ64(ra[1], a_addr, 2048); break;
+            case 6: MI355_DS_READ64(ra[2], a_addr, 4096); break;
+            default: MI355_DS_READ64(ra[3], a_addr, 6144); break;
+          }
+        }
+      }
 }
 
 __global__ void __launch_bounds__(kThreads64, 2)
@@ -95,10 +115,10 @@ gemm_f64_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, do
   f64x2v fa0[4], fb0[4], fa1[4], fb1[4];
 
   // Two fragment sets, one per K half of a slab, refilled while the other is being multiplied: the reads of
-  // the second half go out at the top of a step and land under the 32 instructions of the first half; in the
-  // middle of the step this wave's loads of the next slab have landed and, after the barrier, everybody's, and
-  // everybody has read all of this slab: its buffer takes the slab after the next, and the first half of the
-  // next slab is read under the 32 instructions of the second half.
+  // the second half go out under the instructions of the first half; in the middle of the step this wave's loads
+  // of the next slab have landed and, after the barrier, everybody's, and everybody has read all of this slab: its
+  // buffer takes the slab after the next, and the first half of the next slab is read under the instructions of
+  // the second half.
   const uint32_t steps = k_bytes / kRowBytes;
   fetch(0);
   asm volatile("s_waitcnt vmcnt(0)\n s_barrier" ::: "memory");
@@ -106,26 +126,17 @@ gemm_f64_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, do
   MI355_READ_FRAGS64(fa0, fb0, lane_a, lane_b);
   for (uint32_t s = 0; s < steps; s++) {
     const uint32_t cur = (s & 1u) * 2u * kSlab64, nxt = cur ^ (2u * kSlab64);
-    const uint32_t a1 = (lane_a + cur) ^ 64u, b1 = (lane_b + cur) ^ 64u;
-    MI355_READ_FRAGS64(fa1, fb1, a1, b1);
-    MI355_WAIT_FRAGS64_BUT8(fa0, fb0);   // reads return in order: the 8 just issued may still be in flight
-    mfma_sweep(acc, fa0, fb0);
-    // The accumulators ride along as operands so that the first half's matrix instructions stay ahead of the
-    // waits (the reads and the loads are meant to fly under them), the second fragment set so that none of
-    // the second half's can be placed before them.
+    MI355_WAIT_FRAGS64(fa0, fb0);
+    mfma_sweep(acc, fa0, fb0, fa1, fb1, (lane_a + cur) ^ 64u, (lane_b + cur) ^ 64u, true);
+    // (the second fragment set rides along as an operand so that nothing that uses it can be placed before the wait)
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n s_barrier"
-                 : "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]), "+v"(acc[1][1]),
-                   "+v"(acc[1][2]), "+v"(acc[1][3]), "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[2][2]), "+v"(acc[2][3]),
-                   "+v"(acc[3][0]), "+v"(acc[3][1]), "+v"(acc[3][2]), "+v"(acc[3][3]),
-                   "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fa1[2]), "+v"(fa1[3]), "+v"(fb1[0]), "+v"(fb1[1]), "+v"(fb1[2]), "+v"(fb1[3])
+                 : "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fa1[2]), "+v"(fa1[3]), "+v"(fb1[0]), "+v"(fb1[1]), "+v"(fb1[2]), "+v"(fb1[3])
                  :: "memory");
     if (s + 2 < steps) fetch(s & 1u);
-    if (s + 1 < steps) {
-      const uint32_t a0 = lane_a + nxt, b0 = lane_b + nxt;
-      MI355_READ_FRAGS64(fa0, fb0, a0, b0);
-    }
-    mfma_sweep(acc, fa1, fb1);
+    mfma_sweep(acc, fa1, fb1, fa0, fb0, lane_a + nxt, lane_b + nxt, s + 1 < steps);
   }
+  // the matrix instructions are text to the compiler: the wait states between the last of them and the stores
+  asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
   const uint32_t row0 = tm * kTile64 + wm * 64u + lane % 16u, col0 = tn * kTile64 + wn * 64u + 4u * (lane / 16u);
 #pragma unroll

@@ -217,8 +217,8 @@ def test_peak_loops_do_not_spill(tmp_path, source):
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
 def test_gemm_fp32_and_fp64_kernels(tmp_path):
     """fp32: the ring kernel with four 16x16x4 instructions per 16-byte fragment read, 256 per step.
-    fp64: 64 instructions per step in two halves around the barrier, two 32 KiB buffers (64 KiB static LDS, two
-    workgroups per CU)."""
+    fp64: 64 instructions per step in two halves around the barrier, on the accumulation registers, the fragment reads
+    riding on them; two 32 KiB buffers (64 KiB static LDS, two workgroups per CU)."""
     asm = device_asm(tmp_path, "gemm.hip")
     meta = kernel_metadata(asm)
     name = next(k for k in meta if "gemm_f32_kernel" in k)
@@ -231,18 +231,23 @@ def test_gemm_fp32_and_fp64_kernels(tmp_path):
     assert meta[name]["vgpr_spill_count"] == 0 and meta[name]["private_segment_fixed_size"] == 0 and meta[name]["vgpr_count"] <= 256
     assert meta[name]["group_segment_fixed_size"] == 65536
     body = kernel_body(asm, name)
-    assert body.count("v_mfma_f64_16x16x4_f64") == 64 and "ds_write" not in body
-    # the order of a step: the 8 reads of the second K half, a counted wait, the 32 instructions of the first
-    # half ahead of the wait for everything and the barrier; then the next slab's loads and first-half reads
-    # under the 32 instructions of the second half
+    assert meta[name]["agpr_count"] == 128 and "ds_write" not in body
+    mfmas = re.findall(r"v_mfma_f64_16x16x4_f64 (\S+), \S+, \S+, (\S+)", body)
+    # 32 per K half; the compiler keeps a second copy of (part of) the second half, without reads, for the last step
+    assert len(mfmas) in (64, 80, 96) and all(d == c and d.startswith("a[") for d, c in mfmas), mfmas[:4]
+    # the order of a step: the fragments of the first K half have arrived; its 32 instructions with the 8 reads of
+    # the second half behind every second of the first 16; the wait for everything and the barrier; the next slab's
+    # 8 loads; the 32 instructions of the second half with the next slab's first-half reads riding the same way
     marks = []
     for line in body.split("\n"):
         t = line.strip()
         marks.append("M" if t.startswith("v_mfma_f64") else "B" if t.startswith("s_barrier") else "r" if t.startswith("ds_read_b128")
                      else "w" if t.startswith("s_waitcnt") else "L" if t.startswith("global_load_lds") else "")
     order = "".join(marks)
-    assert "r" * 8 + "w" + "M" * 32 + "wB" in order, order
-    assert order.count("M" * 32) == 2 and order.count("B") == 2
+    half = "MrM" * 8 + "M" * 16
+    assert "w" + half + "wB" in order, order
+    assert "B" + "L" * 8 + "MrM" * 7 + "Mr" in order, order   # (its last 17 instructions are shared with the copy without reads)
+    assert order.count("B") == 2
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
