@@ -762,7 +762,9 @@ def main():
                  "(every kernel is independent per device), run with --gpus 1")
 
     vendor = []
-    if not (args.no_rows or args.no_vendor or args.power_table or args.calibrate_copy or "gemm" not in args.only.split(",")):
+    # (not under a profiler, which would follow the child and report its kernels among this library's)
+    profiled = any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ)
+    if not (args.no_rows or args.no_vendor or profiled or args.power_table or args.calibrate_copy or "gemm" not in args.only.split(",")):
         progress("vendor library's bf16 / fp8 / block-scaled FP4 GEMM in a child process (torch)")
         vendor = vendor_beside()
     from clpeak_amd import capi
@@ -916,7 +918,7 @@ HEADLINE_BLOCKS_PER_CU = 1
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in
 # KiB per dispatch), each scaled by what the counter reads for the plain copy kernel of known size
 # (FETCH_SIZE x 2.0000, WRITE_SIZE x 1.0000): profiles/hbm_float4_read_4GiB_traffic.md.
-TRAFFIC_BYTES_PER_LAUNCH = 4295176192
+TRAFFIC_BYTES_PER_LAUNCH = 4295168000
 
 if __name__ == "__main__":
     main()
