@@ -212,7 +212,7 @@ def _decode(fmt, codes):
     return orc.decode(fmt, codes).astype(np.float64)
 
 
-@pytest.mark.parametrize("kind", ["bf16", "f16", "e4m3", "i8"])
+@pytest.mark.parametrize("kind", ["bf16", "f16", "e4m3", "e5m2", "i8", "mx"])
 def test_gemm_random_shapes_every_element(dev, kind):
     """Six seeded shapes (tile grids from 1 x 1 to 6 x 5, K walks of 1 to 40 steps, mostly odd): the WHOLE of C against a
     numpy float64 product of the decoded operands.  Catches what sampled tiles cannot: a tile or a K step visited twice
@@ -222,6 +222,9 @@ def test_gemm_random_shapes_every_element(dev, kind):
     for _ in range(6):
         M, N = 256 * int(rng.integers(1, 7)), 256 * int(rng.integers(1, 6))
         K = int(rng.integers(1, 41)) * (128 // eb)
+        if kind == "mx":
+            _check_mx_whole(dev, M, N, 2 * K)
+            continue
         dA, dB, dC = dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * (4 if kind == "i8" else 2))
         dev.memset(dC, 0xff)
         if kind == "bf16":
@@ -233,6 +236,9 @@ def test_gemm_random_shapes_every_element(dev, kind):
         elif kind == "e4m3":
             dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, FP8_SCALE); dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, FP8_SCALE)
             dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1.0 / FP8_SCALE, 1.0 / FP8_SCALE); fmt, scale = orc.FMT_E4M3, 1.0 / (FP8_SCALE * FP8_SCALE)
+        elif kind == "e5m2":   # e5m2 A times e4m3 B, as the reference's row
+            dev.fill_fp8_e5m2(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, 57344.0); dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, FP8_SCALE)
+            dev.gemm_fp8_e5m2(dA, dB, dC, M, N, K, 1.0 / 57344.0, 1.0 / FP8_SCALE); fmt, scale = orc.FMT_E5M2, 1.0 / (57344.0 * FP8_SCALE)
         else:
             dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
             dev.gemm_i8(dA, dB, dC, M, N, K); fmt, scale = None, 1.0
@@ -244,7 +250,7 @@ def test_gemm_random_shapes_every_element(dev, kind):
             codes = np.arange(1 << (8 * eb), dtype=np.uint32)
             table = _decode(fmt, codes)            # every code of the format once, then a lookup
             a = table[dA.download(in_dt, M * K)].reshape(M, K)
-            b = table[dB.download(in_dt, N * K)].reshape(N, K)
+            b = (_decode(orc.FMT_E4M3, codes) if kind == "e5m2" else table)[dB.download(in_dt, N * K)].reshape(N, K)
         ref = (a @ b.T) * scale
         if kind == "i8":
             got = dC.download(np.int32, M * N).reshape(M, N).astype(np.float64)
@@ -351,6 +357,36 @@ def _check_mx(dev, M, N, K, tiles, tile=128, whole_output_finite=False):
         err = np.abs(got - ref)
         assert np.all(np.isfinite(got)), (m0, n0)
         assert np.all(err <= 1e-2 * np.abs(ref) + 1e-2 * rms), (m0, n0, float(err.max()), rms)
+    for b in (dA, dB, dSA, dSB, dC):
+        b.free()
+
+
+def _check_mx_whole(dev, M, N, K):
+    """The block-scaled FP4 product, the whole of C against a numpy float64 product of decoded codes times 2^(scale - 127)
+    (low nibble = even element; one scale byte per 32 elements of a row; the oracle's tile routine, which the CPU tests
+    pin, says the same on the sampled tiles of the other tests)."""
+    dA, dB = dev.alloc(M * K // 2), dev.alloc(N * K // 2)
+    dSA, dSB = dev.alloc(M * K // 32), dev.alloc(N * K // 32)
+    dC = dev.alloc(M * N * 2)
+    dev.memset(dC, 0xff)
+    dev.fill_bytes(dA, M * K // 2, SEED, wl.STREAM_GEMM_A, 0, 256); dev.fill_bytes(dB, N * K // 2, SEED, wl.STREAM_GEMM_B, 0, 256)
+    dev.fill_bytes(dSA, M * K // 32, SEED, wl.STREAM_SCALE_A, 123, 9); dev.fill_bytes(dSB, N * K // 32, SEED, wl.STREAM_SCALE_B, 123, 9)
+    dev.gemm_mxfp4(dA, dB, dSA, dSB, dC, M, N, K)
+    e2m1 = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], dtype=np.float64)
+    e2m1 = np.concatenate([e2m1, -e2m1])
+
+    def operand(buf, sbuf, rows):
+        raw = buf.download(np.uint8, rows * K // 2).reshape(rows, K // 2)
+        x = np.empty((rows, K), dtype=np.float64)
+        x[:, 0::2], x[:, 1::2] = e2m1[raw & 15], e2m1[raw >> 4]
+        sc = np.exp2(sbuf.download(np.uint8, rows * K // 32).astype(np.float64) - 127.0).reshape(rows, K // 32)
+        return x * np.repeat(sc, 32, axis=1)
+
+    ref = operand(dA, dSA, M) @ operand(dB, dSB, N).T
+    got = (dC.download(np.uint16, M * N).astype(np.uint32) << 16).view(np.float32).astype(np.float64).reshape(M, N)
+    rms = float(np.sqrt((ref ** 2).mean()))
+    assert np.all(np.isfinite(got)), (M, N, K)
+    assert np.all(np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-2 * rms), (M, N, K, float(np.abs(got - ref).max()), rms)
     for b in (dA, dB, dSA, dSB, dC):
         b.free()
 
