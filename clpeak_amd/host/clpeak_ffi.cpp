@@ -45,13 +45,6 @@ void emitDone(ClpeakEventCallback cb, void *ud, int status, bool cancelled) {
   ffiEmitJson(cb, ud, "{\"t\":\"done\",\"status\":" + std::to_string(status) + ",\"cancelled\":" + (cancelled ? "true" : "false") + "}");
 }
 
-// The stand-in device can be selected from the environment too, so that a front end which passes
-// only reference flags can be exercised on a machine without a GPU.
-bool fakeFromEnv() {
-  const char *v = std::getenv("CLPEAK_FAKE_DEVICES");
-  return v && *v;
-}
-
 std::atomic<bool> g_running{false};
 }  // namespace
 
@@ -83,8 +76,7 @@ extern "C" {
 const char *clpeak_version(void) { return CLPEAK_MI355_VERSION; }
 
 char *clpeak_copy_backend_catalog_json(void) {
-  const Mi355Api &api = fakeFromEnv() ? mi355_fake_api() : mi355_real_api();
-  return copyString(inventoryToJson({Mi355Peak::enumerate(api)}));
+  return copyString(inventoryToJson({Mi355Peak::enumerate(mi355_api())}));
 }
 
 void clpeak_free_string(char *s) { std::free(s); }
@@ -122,7 +114,7 @@ int clpeak_launch(int argc, const char **argv, ClpeakEventCallback on_event, voi
   DeviceInfoStore combinedDevices;
   int status = 0;
   if (!opts.skipRocm && !clpeak::cancelRequested()) {
-    Mi355Peak peak(extras.fakeDevice || fakeFromEnv() ? mi355_fake_api() : mi355_real_api());
+    Mi355Peak peak(mi355_api());
     peak.workload = extras.shape;
     peak.log.reset(new LoggerFfi(on_event, user_data));
     peak.applyOptions(opts);

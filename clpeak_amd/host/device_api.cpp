@@ -1,6 +1,7 @@
 #include "device_api.h"
 
-const Mi355Api &mi355_real_api() {
+// The entry points of libclpeak_mi355.so.
+const Mi355Api &mi355_api() {
   static const Mi355Api api = {
       mi355_device_count, mi355_open, mi355_close, mi355_get_props, mi355_last_error, mi355_alloc, mi355_free,
       mi355_upload, mi355_download, mi355_sync, mi355_timer_start, mi355_timer_stop, mi355_fill_f32,

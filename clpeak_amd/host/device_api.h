@@ -1,7 +1,7 @@
 // The C ABI of libclpeak_mi355.so as a table of function pointers.  The backend class talks
-// to the GPU only through such a table: the real one binds the library's entry points, the
-// fake one (fake_device.cpp) stands in for a GPU so that the row set, ordering, gating and
-// file output can be exercised on a machine without one.
+// to the GPU only through such a table.  The program and the library that ship bind the entry
+// points of libclpeak_mi355.so (device_api.cpp) and nothing else; the host-logic tests link the
+// same classes against a table of their own instead of device_api.cpp.
 #pragma once
 #include "../../include/clpeak_mi355.h"
 
@@ -45,5 +45,4 @@ struct Mi355Api {
   decltype(&mi355_gemm_f64) gemm_f64;
 };
 
-const Mi355Api &mi355_real_api();   // the entry points of libclpeak_mi355.so
-const Mi355Api &mi355_fake_api();   // one pretend gfx950 device, host memory, fixed timings
+const Mi355Api &mi355_api();   // the table this binary is linked with

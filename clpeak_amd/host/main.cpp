@@ -22,7 +22,7 @@ int main(int argc, char **argv) {
   }
   clpeak::setVerbose(opts.verbose);
 
-  const Mi355Api &api = extras.fakeDevice ? mi355_fake_api() : mi355_real_api();
+  const Mi355Api &api = mi355_api();
   if (opts.listDevices) {
     Mi355Peak::printInventory(Mi355Peak::enumerate(api), std::cout);
     return 0;

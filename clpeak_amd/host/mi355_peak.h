@@ -16,13 +16,13 @@ class Mi355Peak : public Peak {
  public:
   std::vector<int> deviceIndices;   // empty = run every device
 
-  explicit Mi355Peak(const Mi355Api &api = mi355_real_api());
+  explicit Mi355Peak(const Mi355Api &api = mi355_api());
   void applyOptions(const CliOptions &opts) override;
   int runAll() override;
 
   // What the front ends call for --list-devices and the backend catalog
   // (RocmPeak::enumerate / printInventory, src/rocm/rocm_peak.cpp:231-278).
-  static BackendInventory enumerate(const Mi355Api &api = mi355_real_api());
+  static BackendInventory enumerate(const Mi355Api &api = mi355_api());
   static void printInventory(const BackendInventory &inv, std::ostream &os);
 
   // Shapes of the seeded workloads.  Defaults are the configured ones; tests shrink them.

@@ -152,7 +152,6 @@ ParseResult parseCliCore(int argc, char **argv, CliOptions &opts, HostExtras &ex
     else if (a == "--describe") opts.describe = true;
     else if (a == "--list-devices") opts.listDevices = true;
     else if (a == "--verbose") opts.verbose = true;
-    else if (a == "--fake-device") extras.fakeDevice = true;
     else if (a == "--reference-operands") extras.shape.referenceOperands = true;
     else if (a == "--small-shapes") {
       Mi355Peak::Workload &s = extras.shape;

@@ -8,9 +8,9 @@
 
 enum class ParseResult { Ok, Help, Version, Error };
 
-// Not part of clpeak's grammar: a stand-in device and reduced shapes, for tests of the host logic.
+// Not part of clpeak's grammar: the shapes of the workloads (reduced ones for quick runs, the
+// reference's constant operands).
 struct HostExtras {
-  bool fakeDevice = false;
   Mi355Peak::Workload shape;
 };
 

@@ -19,3 +19,15 @@ def dev():
     d = capi.Device(0)
     yield d
     d.close()
+
+
+def ensure_host_double():
+    """Build the host layer's test target (tests/host_double: the host sources against a pretend device) when
+    it is not there yet."""
+    import subprocess
+    d = os.path.join(ROOT, "tests", "host_double")
+    if all(os.path.exists(os.path.join(d, f)) for f in ("clpeak-mi355-double", "libclpeak_host_double.so")):
+        return
+    r = subprocess.run(["make", "-C", d, "-j8"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("tests/host_double did not build:\n" + r.stdout[-4000:])

@@ -1,4 +1,7 @@
-// A pretend device behind the Mi355Api table: no GPU, no arithmetic.  Allocations are sizes
+// TEST DOUBLE, never linked into the program or the library that ship: a pretend device behind
+// the Mi355Api table, built only into tests/host_double/clpeak-mi355-double and
+// libclpeak_host_double.so, where it takes the place of clpeak_amd/host/device_api.cpp.
+// No GPU, no arithmetic.  Allocations are sizes
 // only (nothing is dereferenced), every launch "takes" a fixed time, and environment
 // variables can inject failures so that the backend's degrade paths can be tested:
 //   CLPEAK_FAKE_DEVICES=n          number of devices (default 1)
@@ -6,7 +9,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <string>
-#include "device_api.h"
+#include "../../clpeak_amd/host/device_api.h"
 
 struct mi355_dev {
   std::string error;
@@ -91,7 +94,7 @@ int f_gemm_f32(mi355_dev *d, const float *, const float *, float *, uint32_t, ui
 int f_gemm_f64(mi355_dev *d, const double *, const double *, double *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_f64"); return MI355_OK; }
 }  // namespace
 
-const Mi355Api &mi355_fake_api() {
+const Mi355Api &mi355_api() {
   static const Mi355Api api = {
       f_device_count, f_open, f_close, f_get_props, f_last_error, f_alloc, f_free, f_upload, f_download, f_sync,
       f_timer_start, f_timer_stop, f_fill_f32, f_fill_bf16, f_fill_fp8, f_global_bandwidth, f_compute_mad,

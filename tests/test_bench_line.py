@@ -69,3 +69,28 @@ def test_emit_prints_the_compact_record_last(tmp_path):
     # the full record, every row of it, is in the file; the rows are listed for a human on stderr
     assert len(json.loads(rows_file.read_text())["rows"]) == len(full["rows"])
     assert err.getvalue().count("\n") == len(full["rows"])
+
+
+def test_traffic_figure_is_the_committed_profile():
+    """`roofline.traffic` is a measured figure carried as a constant: it must be the one the committed counter
+    summary derives, so that a changed kernel with a stale profile (or the other way round) fails here."""
+    import re
+    text = open(os.path.join(ROOT, "profiles", "hbm_float4_read_4GiB_traffic.md")).read()
+    m = re.search(r"=\s*\*\*(\d+) bytes\*\*", text)
+    assert m, "no scaled traffic figure in the profile"
+    assert int(m.group(1)) == bench.TRAFFIC_BYTES_PER_LAUNCH
+    # and the figure follows from the table's own rows: FETCH_SIZE x 2 + WRITE_SIZE x 1, KiB per dispatch
+    rows = dict(re.findall(r"\| global_bandwidth_kernel<float4, 6>[^|]*\| (FETCH_SIZE|WRITE_SIZE) \| \d+ \| (\d+) \|", text))
+    assert int(rows["FETCH_SIZE"]) * 1024 * 2 + int(rows["WRITE_SIZE"]) * 1024 == bench.TRAFFIC_BYTES_PER_LAUNCH
+    # the profile names the grid it measured; it is the grid the headline launches
+    assert "65536 threads" in text and bench.HEADLINE_BLOCKS_PER_CU * 256 * 256 == 65536
+
+
+def test_headline_grid_is_the_parity_tested_one():
+    """One 256-thread workgroup per CU: bench.py's headline launch, the host layer's default, and the grid the
+    4 GiB GPU parity test runs first."""
+    assert bench.HEADLINE_BLOCKS_PER_CU == 1
+    header = open(os.path.join(ROOT, "clpeak_amd", "host", "mi355_peak.h")).read()
+    assert "bwBlocksPerCU = 1;" in header
+    gpu_test = open(os.path.join(ROOT, "tests", "test_gpu_basic.py")).read()
+    assert "for blocks_per_cu in (1, 8):" in gpu_test

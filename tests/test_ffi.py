@@ -13,15 +13,23 @@ import re
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HOSTLIB = os.path.join(ROOT, "clpeak_amd", "libclpeak_host.so")
+# the embedding ABI built from the host layer's own sources against the pretend device (tests/host_double)
+HOSTLIB = os.path.join(ROOT, "tests", "host_double", "libclpeak_host_double.so")
+SHIPPED = os.path.join(ROOT, "clpeak_amd", "libclpeak_host.so")
 HEADER = os.path.join(ROOT, "include", "clpeak_ffi.h")
 
 CALLBACK = C.CFUNCTYPE(None, C.c_void_p, C.c_void_p)
 RUN_OK, RUN_BAD_ARGS, RUN_CANCELLED, RUN_BUSY = 0, -1, -2, -3
 
 
+@pytest.fixture(scope="module", autouse=True)
+def _host_double():
+    from conftest import ensure_host_double
+    ensure_host_double()
+
+
 @pytest.fixture(scope="module")
-def ffi():
+def ffi(_host_double):
     lib = C.CDLL(HOSTLIB)
     lib.clpeak_version.restype = C.c_char_p
     lib.clpeak_copy_backend_catalog_json.restype = C.c_void_p
@@ -83,7 +91,7 @@ def test_version_and_catalog(ffi, monkeypatch):
 
 def test_quick_run_streams_events_and_saves_xml(ffi, tmp_path):
     xml = tmp_path / "run.xml"
-    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "-i", "1", "--xml-file", str(xml)])
+    rc, raw = launch(ffi, ["--small-shapes", "-i", "1", "--xml-file", str(xml)])
     events = [json.loads(r) for r in raw]
     assert rc == RUN_OK
     assert events[-1] == {"t": "done", "status": 0, "cancelled": False}
@@ -144,7 +152,7 @@ def test_cancel_stops_the_run_and_still_saves(ffi, tmp_path):
             if seen["metrics"] == 3:
                 ffi.clpeak_request_cancel()     # any thread may call this; here: the run's own
 
-    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "--xml-file", str(xml)], on_event)
+    rc, raw = launch(ffi, ["--small-shapes", "--xml-file", str(xml)], on_event)
     events = [json.loads(r) for r in raw]
     assert rc == RUN_CANCELLED
     assert events[-1] == {"t": "done", "status": RUN_CANCELLED, "cancelled": True}
@@ -153,7 +161,7 @@ def test_cancel_stops_the_run_and_still_saves(ffi, tmp_path):
     doc = json.loads(take_string(ffi, ffi.clpeak_load_result_file_json(str(xml).encode())))
     assert [e["test"] for e in doc["entries"]] == ["single_precision_compute"] * 3
     # the flag resets at the start of the next launch
-    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "--kernel-launch-latency"])
+    rc, raw = launch(ffi, ["--small-shapes", "--kernel-launch-latency"])
     assert rc == RUN_OK and json.loads(raw[-1])["cancelled"] is False
 
 
@@ -162,15 +170,15 @@ def test_second_launch_while_running_is_busy_and_silent(ffi):
 
     def on_event(e):
         if e["t"] == "device" and "rc" not in inner:
-            inner["rc"], inner["raw"] = launch(ffi, ["--fake-device", "--small-shapes"])
+            inner["rc"], inner["raw"] = launch(ffi, ["--small-shapes"])
 
-    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "--kernel-launch-latency"], on_event)
+    rc, raw = launch(ffi, ["--small-shapes", "--kernel-launch-latency"], on_event)
     assert inner["rc"] == RUN_BUSY and inner["raw"] == []
     assert rc == RUN_OK and json.loads(raw[-1])["t"] == "done"
 
 
 def test_skipped_backend_runs_nothing(ffi):
-    rc, raw = launch(ffi, ["--fake-device", "--no-rocm"])
+    rc, raw = launch(ffi, ["--no-rocm"])
     assert rc == RUN_OK and [json.loads(r)["t"] for r in raw] == ["done"]
 
 
@@ -207,7 +215,7 @@ def test_arguments_the_gui_builds_for_a_partial_selection(ffi):
     args = ["--no-opencl", "--no-vulkan", "--rocm-device", "0", "--no-cpu",
             "--fp-compute", "--int-compute", "--crypto", "--string", "--bandwidth",
             "--max-time", "200", "--max-time-cpu", "500"]
-    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "-i", "1"] + args)
+    rc, raw = launch(ffi, ["--small-shapes", "-i", "1"] + args)
     events = [json.loads(r) for r in raw]
     assert rc == RUN_OK and events[-1] == {"t": "done", "status": 0, "cancelled": False}
     tags = {e["test"] for e in events if e["t"] == "test_begin"}
@@ -226,7 +234,7 @@ def test_arguments_the_gui_builds_for_a_partial_selection(ffi):
     (["--crypto"], False),                                 # a category with no test here
 ])
 def test_flags_of_the_other_backends_parse_with_their_meaning(ffi, args, runs):
-    rc, raw = launch(ffi, ["--fake-device", "--small-shapes", "-i", "1"] + args)
+    rc, raw = launch(ffi, ["--small-shapes", "-i", "1"] + args)
     events = [json.loads(r) for r in raw]
     assert rc == RUN_OK, (args, events[:1])
     began = [e for e in events if e["t"] == "test_begin"]
@@ -236,5 +244,5 @@ def test_flags_of_the_other_backends_parse_with_their_meaning(ffi, args, runs):
 @pytest.mark.parametrize("args", [["--max-time-cpu"], ["--max-time-cpu", "0"], ["--max-time", "0"], ["--iters", "0"],
                                   ["--cuda-device", "a"], ["--cl-platform"], ["--integer-compute-wide"]])
 def test_malformed_values_of_those_flags_are_still_refused(ffi, args):
-    rc, raw = launch(ffi, ["--fake-device"] + args)
+    rc, raw = launch(ffi, args)
     assert rc == RUN_BAD_ARGS and json.loads(raw[0])["message"].startswith("clpeak:")

@@ -148,18 +148,22 @@ def test_global_bandwidth_full_size_4GiB(dev):
     n = 1 << 30
     src = dev.alloc(n * 4)
     dev.fill_f32(src, n, SEED, wl.STREAM_BW, capi.DIST_U01)
-    blocks, bs = dev.props.num_cus * 8, 256
-    T = blocks * bs
-    out = dev.alloc(T * 4)
+    bs = 256
+    out = dev.alloc(dev.props.num_cus * 8 * bs * 4)
     ref_total = orc.sum_u01(SEED, wl.STREAM_BW, n)
     rng = np.random.default_rng(0)
-    for width in (1, 2, 4):
-        dev.global_bandwidth(width, src, n, out, blocks, bs)
-        got = out.download(np.float32, T)
-        for t in [0, 1, T - 1] + list(rng.integers(0, T, 13)):
-            assert got[t] == orc.global_bandwidth_thread(width, SEED, wl.STREAM_BW, n, T, int(t)), (width, t)
-        total = float(got.astype(np.float64).sum())
-        assert abs(total - ref_total) <= 1e-5 * ref_total, (width, total, ref_total)
+    # one workgroup per CU is the launch bench.py and the command-line program time; eight per CU the
+    # shape with eight times as many, shorter, partial sums
+    for blocks_per_cu in (1, 8):
+        blocks = dev.props.num_cus * blocks_per_cu
+        T = blocks * bs
+        for width in (1, 2, 4):
+            dev.global_bandwidth(width, src, n, out, blocks, bs)
+            got = out.download(np.float32, T)
+            for t in [0, 1, T - 1] + list(rng.integers(0, T, 13)):
+                assert got[t] == orc.global_bandwidth_thread(width, SEED, wl.STREAM_BW, n, T, int(t)), (blocks_per_cu, width, t)
+            total = float(got.astype(np.float64).sum())
+            assert abs(total - ref_total) <= 1e-5 * ref_total, (blocks_per_cu, width, total, ref_total)
     src.free(); out.free()
 
 
@@ -197,6 +201,27 @@ def test_compute_mad_f32_full_size_sampled(dev):
     for first in (0, 123457, n - 64):
         assert np.array_equal(got[first:first + 64], orc.compute_mad(0, 4, SEED, first, 64, steps)), first
     assert np.all(np.isfinite(got))
+    out.free()
+
+
+FULL_SIZE_MAD = [(capi.MAD_F16, 1, np.uint16), (capi.MAD_F16, 2, np.uint16), (capi.MAD_F64, 1, np.float64),
+                 (capi.MAD_F64, 4, np.float64), (capi.MAD_MP, 1, np.float32), (capi.MAD_BF16, 1, np.float32),
+                 (capi.MAD_I32, 1, np.uint32), (capi.MAD_I32, 4, np.uint32), (capi.MAD_I8DP, 1, np.int32),
+                 (capi.MAD_I8DP, 8, np.int32)]
+
+
+@pytest.mark.parametrize("kind,width,dtype", FULL_SIZE_MAD)
+def test_compute_mad_full_size_sampled(dev, kind, width, dtype):
+    """Every other MAD kind at the launch that is timed (2^20 work-items x 4096 steps, 256 per workgroup):
+    three 64-item windows of the output, bit for bit against the oracle (the driver behind every kind is
+    the reference's src/rocm/compute_kernel.cpp:7-94)."""
+    n, steps = 1 << 20, 4096
+    out = dev.alloc(n * np.dtype(dtype).itemsize)
+    dev.compute_mad(kind, width, SEED, n, steps, out, 256)
+    got = out.download(dtype, n)
+    for first in (0, 654321, n - 64):
+        ref = orc.compute_mad(kind, width, SEED, first, 64, steps)
+        assert np.array_equal(got[first:first + 64].view(np.uint8), ref.view(np.uint8)), (kind, width, first)
     out.free()
 
 

@@ -15,14 +15,21 @@ from oracle import pyoracle as orc
 from oracle import workloads as wl
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-CLI = os.path.join(ROOT, "clpeak_amd", "clpeak-mi355")
+# the host layer's own sources linked against the pretend device (tests/host_double), not the program that ships
+CLI = os.path.join(ROOT, "tests", "host_double", "clpeak-mi355-double")
 HOSTLIB = os.path.join(ROOT, "clpeak_amd", "libclpeak_host.so")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _host_double():
+    from conftest import ensure_host_double
+    ensure_host_double()
 
 
 def run_cli(*args, env=None):
     e = dict(os.environ)
     e.update(env or {})
-    return subprocess.run([CLI, "--fake-device", "--small-shapes", *args], capture_output=True, text=True, env=e, timeout=120)
+    return subprocess.run([CLI, "--small-shapes", *args], capture_output=True, text=True, env=e, timeout=120)
 
 
 # The rows a ROCm device reports, in order: (test tag, unit, metrics).  Tags, units and metric
@@ -369,3 +376,20 @@ def test_shipped_mi355x_result_file_has_the_row_contract():
     measured = {(t, m[0]): float(m[2]) for _, t, _, ms in rows for m in ms if m[1] is None}
     assert measured[("global_memory_bandwidth", "float4")] > 6800.0          # 85 % of 8 TB/s
     assert measured[("mfma_bf16", "mfma_bf16")] > 2125.0 and measured[("mfma_int8", "mfma_int8")] > 4250.0
+
+
+def test_the_product_holds_no_pretend_device(tmp_path):
+    """The program and the library that ship know one device table, the entry points of libclpeak_mi355.so:
+    no symbol or string of the tests' pretend device, no flag and no environment switch that selects one."""
+    shipped_cli = os.path.join(ROOT, "clpeak_amd", "clpeak-mi355")
+    for binary in (shipped_cli, HOSTLIB, os.path.join(ROOT, "clpeak_amd", "libclpeak_mi355.so")):
+        syms = subprocess.run(["nm", "-D", "--defined-only", binary], capture_output=True, text=True).stdout
+        assert "fake" not in syms.lower(), binary
+        blob = open(binary, "rb").read().lower()
+        assert b"fake" not in blob and b"clpeak_fake" not in blob, binary
+    r = subprocess.run([shipped_cli, "--fake-device"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 1 and "--fake-device" in r.stderr
+    # and the environment cannot conjure a device: on a machine without a GPU the shipped program lists none
+    e = dict(os.environ, CLPEAK_FAKE_DEVICES="2")
+    r = subprocess.run([shipped_cli, "--list-devices"], capture_output=True, text=True, env=e, timeout=60)
+    assert "Fake" not in r.stdout
