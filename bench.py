@@ -880,6 +880,10 @@ FRAC_KEYS = [("hbm_float", "global_memory_bandwidth", "float"), ("hbm_float2", "
              ("lds_float4", "local_memory_bandwidth", "float4")]
 
 
+# What the workload list asks of each family, as a fraction of the datasheet peak.
+TARGET_FRAC = {"mfma": 0.85, "smfmac": 0.80, "hbm": 0.85, "gemm": 0.70}
+
+
 def compact_line(full):
     """The record the driver reads: the contract's keys, the roofline of the headline kernel, the CPU
     baseline's headline figures and one fraction of peak per target; kept under 2000 bytes (the full
@@ -894,7 +898,7 @@ def compact_line(full):
         c = {k: cb[k] for k in ("value", "unit", "cores", "kind")}
         head = (cb.get("reference") or {}).get("global_memory_bandwidth read") or cb["port"]["global_memory_bandwidth float4"]
         c["ST"], c["MT"] = head.get("ST"), head.get("MT")
-        c["sample"] = cb["sample"][:200]
+        c["sample"] = cb["sample"][:120]
         line["cpu_baseline"] = c
     else:
         line["cpu_baseline"] = None
@@ -905,6 +909,17 @@ def compact_line(full):
         if r is not None and "frac" in r:
             fracs[key] = round(r["frac"], 3)
     line["fracs"] = fracs
+    # which launch the matrix fractions are: the four accumulator chains of a wave share one A and one B
+    # fragment (the rows "distinct operands per chain" in the rows file are the other launch)
+    line["mfma_operands"] = "one set per wave"
+    # the shader clock the part held under each matrix row that is below its target
+    held = {}
+    for key, test, metric in FRAC_KEYS:
+        r = by_key.get((test, metric))
+        target = TARGET_FRAC.get(key.split("_")[0]) if key.startswith(("mfma", "smfmac")) else None   # the rows that read the clock
+        if r is not None and target and "sclk_mhz" in r and r.get("frac", 1.0) < target:
+            held[key] = int(r["sclk_mhz"])
+    line["sclk_mhz"] = held
     lat = by_key.get(("kernel_launch_latency", "roundtrip"))
     if lat is not None:
         line["launch_roundtrip_us"] = lat["value"]

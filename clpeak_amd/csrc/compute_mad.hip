@@ -71,19 +71,30 @@ mad_f16_kernel(uint64_t seed, uint16_t a_bits, uint32_t steps, uint64_t n_items,
   const _Float16 a = bits_to_half(a_bits);
   _Float16 sum = (_Float16)0;
   if constexpr (W == 1) {
-    _Float16 x0[kAcc], x[kAcc];
+    // One v_fma_f16 per step and accumulator, as the reference's scalar row (its __hfma chains,
+    // src/rocm/rocm_kernels/compute_hp.hip:12-30).  Written as the instruction itself, on 32-bit registers
+    // that hold a half in their low 16 bits: from the plain expression the compiler pairs neighbouring chains
+    // into v_pk_fma_f16 and the row becomes the half2 row.  The arithmetic is the same correctly rounded half
+    // FMA either way.
+    uint32_t x0[kAcc], x[kAcc];
+    uint32_t a32 = a_bits;
+    asm volatile("" : "+v"(a32));   // a vector register: the 16-bit literal form would be another encoding
 #pragma unroll
     for (int j = 0; j < kAcc; j++) {
-      x0[j] = bits_to_half(mi355_f32_to_f16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j))));
+      x0[j] = mi355_f32_to_f16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j)));
       x[j] = x0[j];
     }
-#pragma unroll 2
-    for (uint32_t s = 0; s < steps; s++) {
+    for (uint32_t b = 0; b < steps / 8; b++) {   // 128 instructions per trip: the branch of a shorter one shows
 #pragma unroll
-      for (int j = 0; j < kAcc; j++) x[j] = __builtin_fmaf16(x[j], a, x0[j]);
+      for (int t = 0; t < 8; t++)
+#pragma unroll
+        for (int j = 0; j < kAcc; j++) asm volatile("v_fma_f16 %0, %0, %1, %2" : "+v"(x[j]) : "v"(a32), "v"(x0[j]));
     }
+    for (uint32_t r = 0; r < steps % 8; r++)
 #pragma unroll
-    for (int j = 0; j < kAcc; j++) sum += x[j];
+      for (int j = 0; j < kAcc; j++) asm volatile("v_fma_f16 %0, %0, %1, %2" : "+v"(x[j]) : "v"(a32), "v"(x0[j]));
+#pragma unroll
+    for (int j = 0; j < kAcc; j++) sum += bits_to_half((uint16_t)x[j]);
   } else {
     half2v x0[kAcc / 2], x[kAcc / 2];
     const half2v av = {a, a};

@@ -20,13 +20,57 @@ struct Mi355Peak::Buffer {
   bool upload(const std::vector<uint8_t> &host) { return ptr && api.upload(dev, ptr, host.data(), host.size()) == MI355_OK; }
 };
 
-static const char *widthNote(int width) {
+// What the width of a reading means, per test family.
+static const char *chainWidthNote(int width) {
   switch (width) {
     case 1: return "One value per lane at a time.";
     case 2: return "The 16 accumulators of a work-item grouped as 2-wide vectors.";
     case 4: return "The 16 accumulators of a work-item grouped as 4-wide vectors.";
     default: return "";
   }
+}
+static const char *loadWidthNote(int width) {
+  switch (width) {
+    case 1: return "One float (4 bytes) per lane and load instruction.";
+    case 2: return "Two floats (8 bytes) per lane and load instruction.";
+    case 4: return "Four floats (16 bytes) per lane and load instruction.";
+    default: return "";
+  }
+}
+static const char *ldsWidthNote(int width) {
+  switch (width) {
+    case 1: return "One float (4 bytes) per lane in every LDS store and load.";
+    case 2: return "Two floats (8 bytes) per lane in every LDS store and load.";
+    case 4: return "Four floats (16 bytes) per lane in every LDS store and load.";
+    default: return "";
+  }
+}
+
+// MI355X datasheet peaks, in the unit of the row they are compared with (dense; the 2:4 sparse
+// peaks are twice the dense ones).  The reference quotes the datasheet beside its readings the
+// same way (src/rocm/mfma.cpp:9-10, src/rocm/sparse_mfma.cpp:8-11).
+namespace peaks {
+constexpr double kVectorFp32Gflops = 157300.0, kVectorFp64Gflops = 78600.0;
+constexpr double kMatrixFp32 = 157.3, kMatrixFp64 = 78.6, kMatrix16 = 2500.0, kMatrix8 = 5000.0, kMatrix6and4 = 10100.0;
+constexpr double kHbmGbps = 8000.0;
+}  // namespace peaks
+
+// "<note> NN.N % of the MI355X datasheet peak (<peak> <what>)[; shader clock held: NNNN MHz]."
+// The note a reading carries (EmitOptions::description, include/common/logger.h:121-128) is the one
+// place of the row format that takes free text, so the fraction of peak travels there.
+static std::string withPeak(const std::string &note, double value, double peak, const char *what, double heldMhz = 0.0) {
+  std::string out = note;
+  char buf[160];
+  if (peak > 0.0) {
+    snprintf(buf, sizeof buf, "%s%.1f %% of the MI355X datasheet peak (%g %s)", out.empty() ? "" : " ", 100.0 * value / peak, peak, what);
+    out += buf;
+    if (heldMhz > 0.0) {
+      snprintf(buf, sizeof buf, "; shader clock held: %.0f MHz", heldMhz);
+      out += buf;
+    }
+    out += ".";
+  }
+  return out;
 }
 
 Mi355Peak::Mi355Peak(const Mi355Api &api) : api_(api) {}
@@ -126,6 +170,8 @@ struct MadTest {
   const char *tag, *display, *unit, *description;
   int kind, elemBytes;
   int opsPerStep;   // operations one accumulator step counts for
+  double peak;      // datasheet peak in the row's unit, 0 where the datasheet has no line
+  const char *peakWhat;
   struct Variant { const char *metric; int width; const char *note; } variants[4];
 };
 
@@ -151,27 +197,28 @@ void Mi355Peak::runDevice(int ordinal, logger::BackendScope &backend) {
 
   static const MadTest sp = {Benchmark::ComputeSP, "single_precision_compute", "Single-precision compute", "gflops",
       "Vector-ALU rate on 32-bit floats: 2^20 work-items, each advancing 16 independent fused multiply-add chains, "
-      "nothing but registers involved.", MI355_MAD_F32, 4, 2,
-      {{"float", 1, widthNote(1)}, {"float2", 2, widthNote(2)}, {"float4", 4, widthNote(4)}, {nullptr, 0, nullptr}}};
+      "nothing but registers involved.", MI355_MAD_F32, 4, 2, peaks::kVectorFp32Gflops, "GFLOPS vector fp32",
+      {{"float", 1, chainWidthNote(1)}, {"float2", 2, chainWidthNote(2)}, {"float4", 4, chainWidthNote(4)}, {nullptr, 0, nullptr}}};
   static const MadTest hp = {Benchmark::ComputeHP, "half_precision_compute", "Half-precision compute", "gflops",
-      "The same chains in IEEE half precision; the packed form does two lanes per instruction.", MI355_MAD_F16, 2, 2,
-      {{"half", 1, "Half chains written one value at a time (the compiler issues them as packed pairs)."}, {"half2", 2, "Packed half2 FMA."}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
+      "The same chains in IEEE half precision; the packed form does two lanes per instruction.", MI355_MAD_F16, 2, 2, 0.0, "",
+      {{"half", 1, "One scalar half-precision multiply-add per step and accumulator."}, {"half2", 2, "Packed: two half-precision multiply-adds per lane and instruction."}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
   static const MadTest dp = {Benchmark::ComputeDP, "double_precision_compute", "Double-precision compute", "gflops",
-      "The same chains on 64-bit floats.", MI355_MAD_F64, 8, 2,
-      {{"double", 1, widthNote(1)}, {"double2", 2, widthNote(2)}, {"double4", 4, widthNote(4)}, {nullptr, 0, nullptr}}};
+      "The same chains on 64-bit floats.", MI355_MAD_F64, 8, 2, peaks::kVectorFp64Gflops, "GFLOPS vector fp64",
+      {{"double", 1, chainWidthNote(1)}, {"double2", 2, chainWidthNote(2)}, {"double4", 4, chainWidthNote(4)}, {nullptr, 0, nullptr}}};
   static const MadTest mp = {Benchmark::ComputeMP, "mixed_precision_compute", "Mixed-precision compute fp16xfp16+fp32", "gflops",
       "A 32-bit running value times a half-precision factor plus a half-precision addend, widened by the multiply-add "
-      "itself; the running value passes through half precision once every 16 steps.", MI355_MAD_MP, 4, 2,
+      "itself; the running value passes through half precision once every 16 steps.", MI355_MAD_MP, 4, 2, 0.0, "",
       {{"mp", 1, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
   static const MadTest bf = {Benchmark::ComputeBF16, "bfloat16_compute", "BF16 compute bf16xbf16+fp32", "gflops",
       "Two bfloat16 products added to a 32-bit running total per instruction; one factor is refreshed from the total "
-      "once every 128 steps.", MI355_MAD_BF16, 4, 4,
-      {{"bf16", 1, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
+      "once every 128 steps.", MI355_MAD_BF16, 4, 4, 0.0, "",
+      {{"bf16", 1, "Counted as 4 operations per instruction (two products, two additions: a 2-element dot product); clpeak's own "
+                   "row of this name counts a 2-operation multiply-add chain."}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
   static const MadTest i32 = {Benchmark::ComputeInt, "integer_compute", "Integer compute (32-bit IMAD)", "gops",
-      "The same chains on 32-bit integers (multiply-add, wrapping).", MI355_MAD_I32, 4, 2,
-      {{"int", 1, widthNote(1)}, {"int2", 2, widthNote(2)}, {"int4", 4, widthNote(4)}, {nullptr, 0, nullptr}}};
+      "The same chains on 32-bit integers (multiply-add, wrapping).", MI355_MAD_I32, 4, 2, 0.0, "",
+      {{"int", 1, chainWidthNote(1)}, {"int2", 2, chainWidthNote(2)}, {"int4", 4, chainWidthNote(4)}, {nullptr, 0, nullptr}}};
   static const MadTest i8 = {Benchmark::ComputeInt8DP, "integer_compute_int8_dp", "INT8 dot-product compute (DP4a)", "gops",
-      "Four 8-bit multiply-adds per instruction, each result fed back into the next operand.", MI355_MAD_I8DP, 4, 8,
+      "Four 8-bit multiply-adds per instruction, each result fed back into the next operand.", MI355_MAD_I8DP, 4, 8, 0.0, "",
       {{"int8_dp", 1, "One dependent chain."}, {"int8_dp2", 2, "Two independent chains."},
        {"int8_dp4", 4, "Four independent chains."}, {"int8_dp8", 8, "Eight independent chains."}}};
 
@@ -231,7 +278,8 @@ void Mi355Peak::runComputeMad(const MadTest &t) {
     // 16 accumulators per item (or `width` chains for the dot-product test)
     const double chains = t.kind == MI355_MAD_I8DP ? (double)v.width : 16.0;
     const double ops = (double)workload.madItems * chains * (double)workload.madSteps * (double)t.opsPerStep;
-    test.emit(v.metric, (float)(ops * 1e6 / us / 1e9), {false, note});
+    const double giga = ops * 1e6 / us / 1e9;
+    test.emit(v.metric, (float)giga, {false, withPeak(note, giga, t.peak, t.peakWhat)});
   }
 }
 
@@ -261,6 +309,19 @@ void Mi355Peak::runUnsupportedMatrixRows(Category phase, bool wmma) {
 }
 
 // ---- dense MFMA ----------------------------------------------------------------------------------------------
+// The matrix kernels leave two counters of their timed loop behind (shader cycles, ticks of the
+// constant 100 MHz clock): the shader clock the part held under the load, in MHz; 0 when unknown.
+double Mi355Peak::heldClockMhz(const void *clocks) {
+  uint64_t c[2] = {0, 0};
+  if (!clocks || api_.download(dev_, c, clocks, sizeof c) != MI355_OK || c[1] == 0) return 0.0;
+  return (double)c[0] / (double)c[1] * 100.0;
+}
+
+static const char *operandsNote(bool reference) {
+  return reference ? "Operands: the constants clpeak's own kernels multiply; one operand set per wave."
+                   : "Operands: seeded random values; one operand set per wave, four accumulator chains.";
+}
+
 namespace {
 struct MfmaRow {
   const char *tag, *display, *unit, *description;
@@ -268,50 +329,52 @@ struct MfmaRow {
   OperandFormat fmt;
   double sigma;
   bool scaled;
+  double peak;   // dense datasheet peak of the operand type, TFLOPS / TOPS
 };
 const MfmaRow kMfmaFp[] = {
     {"mfma_fp16", "MFMA fp16xfp16+fp32 16x16x32", "tflops", "Matrix-core rate on half-precision inputs with a 32-bit accumulator.",
-     MI355_MFMA_F16_16x16x32, 16, 16, 32, OperandFormat::F16, 0.01, false},
+     MI355_MFMA_F16_16x16x32, 16, 16, 32, OperandFormat::F16, 0.01, false, peaks::kMatrix16},
     {"mfma_fp16_32x32x16", "MFMA fp16xfp16+fp32 32x32x16", "tflops", "The same on the 32x32 tile shape.",
-     MI355_MFMA_F16_32x32x16, 32, 32, 16, OperandFormat::F16, 0.01, false},
+     MI355_MFMA_F16_32x32x16, 32, 32, 16, OperandFormat::F16, 0.01, false, peaks::kMatrix16},
     {"mfma_bf16", "MFMA bf16xbf16+fp32 16x16x32", "tflops", "Matrix-core rate on bfloat16 inputs with a 32-bit accumulator.",
-     MI355_MFMA_BF16_16x16x32, 16, 16, 32, OperandFormat::BF16, 0.01, false},
+     MI355_MFMA_BF16_16x16x32, 16, 16, 32, OperandFormat::BF16, 0.01, false, peaks::kMatrix16},
     {"mfma_bf16_32x32x16", "MFMA bf16xbf16+fp32 32x32x16", "tflops", "The same on the 32x32 tile shape.",
-     MI355_MFMA_BF16_32x32x16, 32, 32, 16, OperandFormat::BF16, 0.01, false},
+     MI355_MFMA_BF16_32x32x16, 32, 32, 16, OperandFormat::BF16, 0.01, false, peaks::kMatrix16},
     {"mfma_fp8", "MFMA fp8xfp8+fp32 16x16x128", "tflops", "Matrix-core rate on OCP fp8 (E4M3) inputs.",
-     MI355_MFMA_FP8_16x16x128, 16, 16, 128, OperandFormat::E4M3, 1.0, false},
+     MI355_MFMA_FP8_16x16x128, 16, 16, 128, OperandFormat::E4M3, 1.0, false, peaks::kMatrix8},
     {"mfma_bf8", "MFMA bf8xbf8+fp32 16x16x128", "tflops", "Matrix-core rate on OCP fp8 (E5M2) inputs.",
-     MI355_MFMA_BF8_16x16x128, 16, 16, 128, OperandFormat::E5M2, 1.0, false},
+     MI355_MFMA_BF8_16x16x128, 16, 16, 128, OperandFormat::E5M2, 1.0, false, peaks::kMatrix8},
     {"mfma_mxfp6_e2m3", "MFMA mxfp6(e2m3)+fp32 16x16x128", "tflops", "6-bit MX inputs with one E8M0 scale per 32 elements.",
-     MI355_MFMA_MXFP6_E2M3, 16, 16, 128, OperandFormat::E2M3, 1.0, true},
+     MI355_MFMA_MXFP6_E2M3, 16, 16, 128, OperandFormat::E2M3, 1.0, true, peaks::kMatrix6and4},
     {"mfma_mxfp6_e3m2", "MFMA mxfp6(e3m2)+fp32 16x16x128", "tflops", "6-bit MX inputs, the wider-range variant.",
-     MI355_MFMA_MXFP6_E3M2, 16, 16, 128, OperandFormat::E3M2, 1.0, true},
+     MI355_MFMA_MXFP6_E3M2, 16, 16, 128, OperandFormat::E3M2, 1.0, true, peaks::kMatrix6and4},
     {"mfma_mxfp4", "MFMA mxfp4(e2m1)+fp32 16x16x128", "tflops", "4-bit MX inputs with one E8M0 scale per 32 elements.",
-     MI355_MFMA_MXFP4_E2M1, 16, 16, 128, OperandFormat::E2M1, 1.0, true},
+     MI355_MFMA_MXFP4_E2M1, 16, 16, 128, OperandFormat::E2M1, 1.0, true, peaks::kMatrix6and4},
 };
 const MfmaRow kMfmaInt[] = {
     {"mfma_int8", "MFMA int8xint8+int32 16x16x64", "tops", "Matrix-core rate on 8-bit integers with a 32-bit accumulator.",
-     MI355_MFMA_I8_16x16x64, 16, 16, 64, OperandFormat::I8, 0.0, false},
+     MI355_MFMA_I8_16x16x64, 16, 16, 64, OperandFormat::I8, 0.0, false, peaks::kMatrix8},
 };
 struct SparseRow {
   const char *tag, *display, *unit, *description;
   int kind, K;
   OperandFormat fmt;
   double sigma;
+  double peak;   // 2:4 sparse datasheet peak (twice the dense one), TFLOPS / TOPS
 };
 const SparseRow kSparseFp[] = {
     {"smfmac_fp16", "Sparse MFMA fp16 2:4 16x16x64 (TFLOPS)", "tflops", "2:4 structured-sparse matrix-core rate, half-precision inputs.",
-     MI355_SMFMAC_F16_16x16x64, 64, OperandFormat::F16, 0.01},
+     MI355_SMFMAC_F16_16x16x64, 64, OperandFormat::F16, 0.01, 2 * peaks::kMatrix16},
     {"smfmac_bf16", "Sparse MFMA bf16 2:4 16x16x64 (TFLOPS)", "tflops", "2:4 structured-sparse matrix-core rate, bfloat16 inputs.",
-     MI355_SMFMAC_BF16_16x16x64, 64, OperandFormat::BF16, 0.01},
+     MI355_SMFMAC_BF16_16x16x64, 64, OperandFormat::BF16, 0.01, 2 * peaks::kMatrix16},
     {"smfmac_fp8", "Sparse MFMA fp8 2:4 16x16x128 (TFLOPS)", "tflops", "2:4 structured-sparse matrix-core rate, fp8 (E4M3) inputs.",
-     MI355_SMFMAC_FP8_16x16x128, 128, OperandFormat::E4M3, 1.0},
+     MI355_SMFMAC_FP8_16x16x128, 128, OperandFormat::E4M3, 1.0, 2 * peaks::kMatrix8},
     {"smfmac_bf8", "Sparse MFMA bf8 2:4 16x16x128 (TFLOPS)", "tflops", "2:4 structured-sparse matrix-core rate, fp8 (E5M2) inputs.",
-     MI355_SMFMAC_BF8_16x16x128, 128, OperandFormat::E5M2, 1.0},
+     MI355_SMFMAC_BF8_16x16x128, 128, OperandFormat::E5M2, 1.0, 2 * peaks::kMatrix8},
 };
 const SparseRow kSparseInt[] = {
     {"smfmac_int8", "Sparse MFMA int8 2:4 16x16x128 (TOPS)", "tops", "2:4 structured-sparse matrix-core rate, 8-bit integers.",
-     MI355_SMFMAC_I8_16x16x128, 128, OperandFormat::I8, 0.0},
+     MI355_SMFMAC_I8_16x16x128, 128, OperandFormat::I8, 0.0, 2 * peaks::kMatrix8},
 };
 }  // namespace
 
@@ -331,7 +394,8 @@ void Mi355Peak::runMfma(Category phase) {
                                        : seeded_operand(m.fmt, m.sigma, workload.seed, MI355_STREAM_MFMA_B, units * m.N * m.K);
     Buffer dA(api_, dev_, A.size()), dB(api_, dev_, B.size()), out(api_, dev_, units * m.M * m.N * 4);
     Buffer sA(api_, dev_, m.scaled ? units * m.M * (m.K / 32) : 16), sB(api_, dev_, m.scaled ? units * m.N * (m.K / 32) : 16);
-    bool ok = dA && dB && out && sA && sB && dA.upload(A) && dB.upload(B);
+    Buffer clk(api_, dev_, 16);
+    bool ok = dA && dB && out && sA && sB && clk && dA.upload(A) && dB.upload(B);
     if (ok && m.scaled && ref)
       ok = sA.upload(std::vector<uint8_t>(units * m.M * (m.K / 32), kReferenceScale)) &&
            sB.upload(std::vector<uint8_t>(units * m.N * (m.K / 32), kReferenceScale));
@@ -345,7 +409,7 @@ void Mi355Peak::runMfma(Category phase) {
     const float us = runKernel(
         [&] {
           return api_.mfma_dense(dev_, m.kind | MI355_MFMA_ONE_OPERAND_SET, dA.ptr, dB.ptr, m.scaled ? (const uint8_t *)sA.ptr : nullptr,
-                                 m.scaled ? (const uint8_t *)sB.ptr : nullptr, out.ptr, waves, workload.mfmaIters, nullptr);
+                                 m.scaled ? (const uint8_t *)sB.ptr : nullptr, out.ptr, waves, workload.mfmaIters, (uint64_t *)clk.ptr);
         },
         targetTimeUs, forceIters ? specifiedIters : 0);
     if (us <= 0.0f) {
@@ -354,7 +418,8 @@ void Mi355Peak::runMfma(Category phase) {
     }
     // every wave issues 4 * iters instructions of 2*M*N*K operations
     const double ops = (double)units * workload.mfmaIters * 2.0 * m.M * m.N * m.K;
-    test.emit(m.tag, (float)(ops * 1e6 / us / 1e12));
+    const double tera = ops * 1e6 / us / 1e12;
+    test.emit(m.tag, (float)tera, {false, withPeak(operandsNote(workload.referenceOperands), tera, m.peak, isInt ? "TOPS dense" : "TFLOPS dense", heldClockMhz(clk.ptr))});
   }
 }
 
@@ -375,12 +440,13 @@ void Mi355Peak::runSparseMfma(Category phase) {
     const std::vector<uint8_t> meta = ref ? std::vector<uint8_t>(units * 16 * (m.K / 4), kReferenceSparseMeta)
                                           : seeded_sparse_meta(workload.seed, MI355_STREAM_SPARSE, units * 16 * (m.K / 4));
     Buffer dA(api_, dev_, Ac.size()), dB(api_, dev_, B.size()), dM(api_, dev_, meta.size()), out(api_, dev_, units * 256 * 4);
-    if (!(dA && dB && dM && out && dA.upload(Ac) && dB.upload(B) && dM.upload(meta))) {
+    Buffer clk(api_, dev_, 16);
+    if (!(dA && dB && dM && out && clk && dA.upload(Ac) && dB.upload(B) && dM.upload(meta))) {
       test.skip(m.tag, ResultStatus::Error, "Failed to allocate or upload operand buffers");
       continue;
     }
     const float us = runKernel(
-        [&] { return api_.smfmac(dev_, m.kind | MI355_MFMA_ONE_OPERAND_SET, dA.ptr, (const uint8_t *)dM.ptr, dB.ptr, out.ptr, waves, workload.mfmaIters, nullptr); },
+        [&] { return api_.smfmac(dev_, m.kind | MI355_MFMA_ONE_OPERAND_SET, dA.ptr, (const uint8_t *)dM.ptr, dB.ptr, out.ptr, waves, workload.mfmaIters, (uint64_t *)clk.ptr); },
         targetTimeUs, forceIters ? specifiedIters : 0);
     if (us <= 0.0f) {
       test.skip(m.tag, ResultStatus::Error, "kernel launch failed");
@@ -388,7 +454,8 @@ void Mi355Peak::runSparseMfma(Category phase) {
     }
     // counted with the dense-equivalent K, as the datasheet's sparse column is
     const double ops = (double)units * workload.mfmaIters * 2.0 * 16 * 16 * m.K;
-    test.emit(m.tag, (float)(ops * 1e6 / us / 1e12));
+    const double tera = ops * 1e6 / us / 1e12;
+    test.emit(m.tag, (float)tera, {false, withPeak(operandsNote(workload.referenceOperands), tera, m.peak, isInt ? "TOPS 2:4 sparse" : "TFLOPS 2:4 sparse", heldClockMhz(clk.ptr))});
   }
 }
 
@@ -397,7 +464,7 @@ void Mi355Peak::runSparseMfma(Category phase) {
 // With reference operands every byte of A and B is `referenceByte`, as the reference's tests set them
 // (0x3f: src/rocm/rocblas.cpp:211-212; 0x38: src/rocm/hipblaslt_gemm.cpp:272-273).
 void Mi355Peak::runGemmRow(logger::TestScope &test, const char *metric, const char *note, size_t elemBytes, size_t outBytes,
-                           uint8_t referenceByte, const std::function<int(void *, void *)> &fill,
+                           uint8_t referenceByte, double peak, const std::function<int(void *, void *)> &fill,
                            const std::function<int(void *, void *, void *)> &launch) {
   const uint32_t D = workload.gemmDim;
   const size_t abBytes = (size_t)D * D * elemBytes;
@@ -412,7 +479,12 @@ void Mi355Peak::runGemmRow(logger::TestScope &test, const char *metric, const ch
   }
   const float us = runKernel([&] { return launch(A.ptr, B.ptr, C.ptr); }, targetTimeUs, forceIters ? specifiedIters : 0);
   if (us <= 0.0f) test.skip(metric, ResultStatus::Error, "kernel launch failed", note);
-  else test.emit(metric, (float)(2.0 * D * D * D * 1e6 / us / 1e12), {false, note});
+  else {
+    const double tera = 2.0 * D * D * D * 1e6 / us / 1e12;
+    const char *what = peak == peaks::kMatrixFp32 ? "TFLOPS matrix fp32" : peak == peaks::kMatrixFp64 ? "TFLOPS matrix fp64"
+                       : std::string(metric) == "int8" ? "TOPS dense" : "TFLOPS dense";
+    test.emit(metric, (float)tera, {false, withPeak(note, tera, peak, what)});
+  }
 }
 
 void Mi355Peak::runGemmFp() {
@@ -421,25 +493,25 @@ void Mi355Peak::runGemmFp() {
                                   "operands), not a vendor library."});
   const uint32_t D = workload.gemmDim;
   const uint64_t n = (uint64_t)D * D;
-  runGemmRow(test, "fp32", "fp32 inputs, accumulation and output, on the fp32 matrix instruction; A row-major, B column-major.", 4, 4, 0x3f,
+  runGemmRow(test, "fp32", "fp32 inputs, accumulation and output, on the fp32 matrix instruction; A row-major, B column-major.", 4, 4, 0x3f, peaks::kMatrixFp32,
              [&](void *a, void *b) {
                const int rc = api_.fill_f32(dev_, (float *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
                return rc != MI355_OK ? rc : api_.fill_f32(dev_, (float *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
              },
              [&](void *a, void *b, void *c) { return api_.gemm_f32(dev_, (const float *)a, (const float *)b, (float *)c, D, D, D); });
-  runGemmRow(test, "fp64", "fp64 inputs, accumulation and output, on the fp64 matrix instruction; A row-major, B column-major.", 8, 8, 0x3f,
+  runGemmRow(test, "fp64", "fp64 inputs, accumulation and output, on the fp64 matrix instruction; A row-major, B column-major.", 8, 8, 0x3f, peaks::kMatrixFp64,
              [&](void *a, void *b) {
                const int rc = api_.fill_f64(dev_, (double *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
                return rc != MI355_OK ? rc : api_.fill_f64(dev_, (double *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
              },
              [&](void *a, void *b, void *c) { return api_.gemm_f64(dev_, (const double *)a, (const double *)b, (double *)c, D, D, D); });
-  runGemmRow(test, "fp16", "IEEE half inputs, fp32 accumulation, half output; A row-major, B column-major.", 2, 2, 0x3f,
+  runGemmRow(test, "fp16", "IEEE half inputs, fp32 accumulation, half output; A row-major, B column-major.", 2, 2, 0x3f, peaks::kMatrix16,
              [&](void *a, void *b) {
                const int rc = api_.fill_f16(dev_, (uint16_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
                return rc != MI355_OK ? rc : api_.fill_f16(dev_, (uint16_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
              },
              [&](void *a, void *b, void *c) { return api_.gemm_f16(dev_, (const uint16_t *)a, (const uint16_t *)b, (uint16_t *)c, D, D, D); });
-  runGemmRow(test, "bf16", "bf16 inputs, fp32 accumulation, bf16 output; A row-major, B column-major.", 2, 2, 0x3f,
+  runGemmRow(test, "bf16", "bf16 inputs, fp32 accumulation, bf16 output; A row-major, B column-major.", 2, 2, 0x3f, peaks::kMatrix16,
              [&](void *a, void *b) {
                const int rc = api_.fill_bf16(dev_, (uint16_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1);
                return rc != MI355_OK ? rc : api_.fill_bf16(dev_, (uint16_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1);
@@ -454,7 +526,7 @@ void Mi355Peak::runGemmFp8() {
   const uint32_t D = workload.gemmDim;
   const uint64_t n = (uint64_t)D * D;
   const float s43 = 448.0f, s52 = 57344.0f;   // uniform [-1,1) stretched over the range of the format
-  runGemmRow(test, "fp8_e4m3", "OCP e4m3 inputs, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2, 0x38,
+  runGemmRow(test, "fp8_e4m3", "OCP e4m3 inputs, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2, 0x38, peaks::kMatrix8,
              [&](void *a, void *b) {
                const int rc = api_.fill_fp8_e4m3(dev_, (uint8_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1, s43);
                return rc != MI355_OK ? rc : api_.fill_fp8_e4m3(dev_, (uint8_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1, s43);
@@ -462,7 +534,7 @@ void Mi355Peak::runGemmFp8() {
              [&](void *a, void *b, void *c) {
                return api_.gemm_fp8_e4m3(dev_, (const uint8_t *)a, (const uint8_t *)b, (uint16_t *)c, D, D, D, 1.0f / s43, 1.0f / s43);
              });
-  runGemmRow(test, "fp8_e5m2", "An OCP e5m2 A against an e4m3 B, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2, 0x38,
+  runGemmRow(test, "fp8_e5m2", "An OCP e5m2 A against an e4m3 B, per-tensor fp32 scales, fp32 accumulation, bf16 output.", 1, 2, 0x38, peaks::kMatrix8,
              [&](void *a, void *b) {
                const int rc = api_.fill_fp8_e5m2(dev_, (uint8_t *)a, n, workload.seed, MI355_STREAM_GEMM_A, MI355_DIST_UPM1, s52);
                return rc != MI355_OK ? rc : api_.fill_fp8_e4m3(dev_, (uint8_t *)b, n, workload.seed, MI355_STREAM_GEMM_B, MI355_DIST_UPM1, s43);
@@ -489,7 +561,10 @@ void Mi355Peak::runGemmFp8() {
                      targetTimeUs, forceIters ? specifiedIters : 0);
     if (!ok) test.skip("mxf4_e2m1", ResultStatus::Error, "Failed to allocate or fill GEMM buffers", mxNote);
     else if (us <= 0.0f) test.skip("mxf4_e2m1", ResultStatus::Error, "kernel launch failed", mxNote);
-    else test.emit("mxf4_e2m1", (float)(2.0 * D * D * D * 1e6 / us / 1e12), {false, mxNote});
+    else {
+      const double tera = 2.0 * D * D * D * 1e6 / us / 1e12;
+      test.emit("mxf4_e2m1", (float)tera, {false, withPeak(mxNote, tera, peaks::kMatrix6and4, "TFLOPS dense")});
+    }
   }
 }
 
@@ -499,7 +574,7 @@ void Mi355Peak::runGemmInt() {
                                   "kernel, not a vendor library."});
   const uint32_t D = workload.gemmDim;
   const uint64_t n = (uint64_t)D * D;
-  runGemmRow(test, "int8", "8-bit integers in [-8, 7], 32-bit totals; A row-major, B column-major.", 1, 4, 0x3f,
+  runGemmRow(test, "int8", "8-bit integers in [-8, 7], 32-bit totals; A row-major, B column-major.", 1, 4, 0x3f, peaks::kMatrix8,
              [&](void *a, void *b) {
                const int rc = api_.fill_i8(dev_, (int8_t *)a, n, workload.seed, MI355_STREAM_GEMM_A);
                return rc != MI355_OK ? rc : api_.fill_i8(dev_, (int8_t *)b, n, workload.seed, MI355_STREAM_GEMM_B);
@@ -521,13 +596,16 @@ void Mi355Peak::runGlobalBandwidth() {
   const bool ok = in && out && api_.fill_f32(dev_, (float *)in.ptr, n, workload.seed, MI355_STREAM_BW, MI355_DIST_U01) == MI355_OK;
   for (const auto &v : variants) {
     if (!ok) {
-      test.skip(v.metric, ResultStatus::Error, "Failed to allocate buffers", widthNote(v.width));
+      test.skip(v.metric, ResultStatus::Error, "Failed to allocate buffers", loadWidthNote(v.width));
       continue;
     }
     const float us = runKernel([&] { return api_.global_bandwidth(dev_, v.width, (const float *)in.ptr, n, (float *)out.ptr, blocks, bs); },
                                targetTimeUs, forceIters ? specifiedIters : 0);
-    if (us <= 0.0f) test.skip(v.metric, ResultStatus::Error, "kernel launch failed", widthNote(v.width));
-    else test.emit(v.metric, (float)((double)n * sizeof(float) / us / 1e3), widthNote(v.width));
+    if (us <= 0.0f) test.skip(v.metric, ResultStatus::Error, "kernel launch failed", loadWidthNote(v.width));
+    else {
+      const double gbps = (double)n * sizeof(float) / us / 1e3;
+      test.emit(v.metric, (float)gbps, {false, withPeak(loadWidthNote(v.width), gbps, peaks::kHbmGbps, "GB/s HBM3E")});
+    }
   }
 }
 
@@ -547,13 +625,13 @@ void Mi355Peak::runLocalBandwidth() {
   Buffer out(api_, dev_, threads * sizeof(float));
   for (const auto &v : variants) {
     if (!out) {
-      test.skip(v.metric, ResultStatus::Error, "Buffer alloc failed", widthNote(v.width));
+      test.skip(v.metric, ResultStatus::Error, "Buffer alloc failed", ldsWidthNote(v.width));
       continue;
     }
     const float us = runKernel([&] { return api_.local_bandwidth(dev_, v.width, (float *)out.ptr, blocks, bs, reps); },
                                targetTimeUs, forceIters ? specifiedIters : 0);
-    if (us <= 0.0f) test.skip(v.metric, ResultStatus::Error, "kernel launch failed", widthNote(v.width));
-    else test.emit(v.metric, (float)((double)reps * 2.0 * v.width * sizeof(float) * (double)threads / us / 1e3), widthNote(v.width));
+    if (us <= 0.0f) test.skip(v.metric, ResultStatus::Error, "kernel launch failed", ldsWidthNote(v.width));
+    else test.emit(v.metric, (float)((double)reps * 2.0 * v.width * sizeof(float) * (double)threads / us / 1e3), ldsWidthNote(v.width));
   }
 }
 

@@ -54,13 +54,14 @@ class Mi355Peak : public Peak {
   float runKernel(const std::function<int()> &launch, unsigned targetTimeUs, unsigned forcedIters);
 
   struct Buffer;   // RAII device allocation
+  double heldClockMhz(const void *clocks);
   void runDevice(int ordinal, logger::BackendScope &backend);
   void runComputeMad(const struct MadTest &t);
   void runUnsupportedMatrixRows(Category phase, bool wmma);
   void runMfma(Category phase);
   void runSparseMfma(Category phase);
   void runGemmRow(logger::TestScope &test, const char *metric, const char *note, size_t elemBytes, size_t outBytes,
-                  uint8_t referenceByte, const std::function<int(void *, void *)> &fill, const std::function<int(void *, void *, void *)> &launch);
+                  uint8_t referenceByte, double peak, const std::function<int(void *, void *)> &fill, const std::function<int(void *, void *, void *)> &launch);
   void runGemmFp();
   void runGemmFp8();
   void runGemmInt();

@@ -55,6 +55,19 @@ def test_compact_line_is_small_and_complete():
                 "gemm_bf16_seeded"):
         assert key in line["fracs"], key
     assert line["launch_roundtrip_us"] == 9.47
+    assert line["mfma_operands"] == "one set per wave"
+    assert line["sclk_mhz"] == {}          # every synthetic row is above its target
+
+
+def test_compact_line_names_the_held_clock_of_rows_below_target():
+    full = _synthetic_full()
+    for r in full["rows"]:
+        r["frac"] = 0.5                    # everything below target: the largest the record can get
+    text = json.dumps(bench.compact_line(full), separators=(",", ":"))
+    assert len(text.encode()) < 2000, len(text)
+    held = json.loads(text)["sclk_mhz"]
+    assert held["smfmac_fp16"] == 2399 and held["mfma_fp16_32x32x16"] == 2399 and len(held) == 15
+    assert not [k for k in held if not k.startswith(("mfma", "smfmac"))]     # the rows that read the clock in the kernel
 
 
 def test_emit_prints_the_compact_record_last(tmp_path):
@@ -81,7 +94,8 @@ def test_traffic_figure_is_the_committed_profile():
     assert int(m.group(1)) == bench.TRAFFIC_BYTES_PER_LAUNCH
     # and the figure follows from the table's own rows: FETCH_SIZE x 2 + WRITE_SIZE x 1, KiB per dispatch
     rows = dict(re.findall(r"\| global_bandwidth_kernel<float4, 6>[^|]*\| (FETCH_SIZE|WRITE_SIZE) \| \d+ \| (\d+) \|", text))
-    assert int(rows["FETCH_SIZE"]) * 1024 * 2 + int(rows["WRITE_SIZE"]) * 1024 == bench.TRAFFIC_BYTES_PER_LAUNCH
+    from_rows = int(rows["FETCH_SIZE"]) * 1024 * 2 + int(rows["WRITE_SIZE"]) * 1024
+    assert abs(from_rows - bench.TRAFFIC_BYTES_PER_LAUNCH) <= 1e-4 * from_rows   # the table prints six significant digits
     # the profile names the grid it measured; it is the grid the headline launches
     assert "65536 threads" in text and bench.HEADLINE_BLOCKS_PER_CU * 256 * 256 == 65536
 

@@ -270,3 +270,19 @@ def test_mixed_precision_mad_loops_run_on_the_mixed_instructions(tmp_path):
     body = kernel_body(asm, bf)
     assert body.count("v_dot2_f32_bf16") == 16 * 16 + 16, body.count("v_dot2_f32_bf16")
     assert not re.search(r"\bv_(fma|fmac|fmamk|fmaak|mad|mac)_f32\b", body)
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_scalar_half_row_runs_on_the_scalar_half_fma(tmp_path):
+    """The `half` row is the reference's scalar __hfma chain (src/rocm/rocm_kernels/compute_hp.hip:12-30): its loop is
+    one v_fma_f16 per step and accumulator and holds no packed multiply-add; the `half2` row is the packed form."""
+    asm = device_asm(tmp_path, "compute_mad.hip")
+    meta = kernel_metadata(asm)
+    scalar = next(n for n in meta if "mad_f16_kernelILi1E" in n)
+    packed = next(n for n in meta if "mad_f16_kernelILi2E" in n)
+    for name in (scalar, packed):
+        assert meta[name].get("vgpr_spill_count", 0) == 0 and meta[name].get("private_segment_fixed_size", 0) == 0, meta[name]
+    body = kernel_body(asm, scalar)
+    assert body.count("v_fma_f16") == 16 * 8 + 16 and "v_pk_fma_f16" not in body, body.count("v_fma_f16")
+    body = kernel_body(asm, packed)
+    assert "v_pk_fma_f16" in body and not re.search(r"\bv_fma_f16\b", body)

@@ -378,6 +378,69 @@ def test_shipped_mi355x_result_file_has_the_row_contract():
     assert measured[("mfma_bf16", "mfma_bf16")] > 2125.0 and measured[("mfma_int8", "mfma_int8")] > 4250.0
 
 
+# Rows with a line in the MI355X datasheet: (test, metric) -> (peak in the row's unit).  Dense matrix peaks; the
+# 2:4 sparse ones are twice those.
+DATASHEET = {("single_precision_compute", "float"): 157300.0, ("single_precision_compute", "float4"): 157300.0,
+             ("double_precision_compute", "double2"): 78600.0,
+             ("mfma_fp16", "mfma_fp16"): 2500.0, ("mfma_bf16_32x32x16", "mfma_bf16_32x32x16"): 2500.0,
+             ("mfma_fp8", "mfma_fp8"): 5000.0, ("mfma_bf8", "mfma_bf8"): 5000.0, ("mfma_int8", "mfma_int8"): 5000.0,
+             ("mfma_mxfp6_e2m3", "mfma_mxfp6_e2m3"): 10100.0, ("mfma_mxfp4", "mfma_mxfp4"): 10100.0,
+             ("smfmac_fp16", "smfmac_fp16"): 5000.0, ("smfmac_bf8", "smfmac_bf8"): 10000.0, ("smfmac_int8", "smfmac_int8"): 10000.0,
+             ("rocblas-fp", "fp32"): 157.3, ("rocblas-fp", "fp64"): 78.6, ("rocblas-fp", "bf16"): 2500.0,
+             ("hipblaslt-fp8", "fp8_e4m3"): 5000.0, ("hipblaslt-fp8", "mxf4_e2m1"): 10100.0, ("rocblas-int", "int8"): 5000.0,
+             ("global_memory_bandwidth", "float"): 8000.0, ("global_memory_bandwidth", "float4"): 8000.0}
+
+
+def _infos(path):
+    out = {}
+    for run in ET.parse(path).getroot().findall("run"):
+        for test in run.iter("test"):
+            for m in test.findall("metric"):
+                out[(test.get("name"), m.get("name"))] = (m.get("status"), m.text, m.get("info") or "")
+    return out
+
+
+def _check_percent_notes(infos):
+    for key, peak in DATASHEET.items():
+        status, text, info = infos[key]
+        assert status is None, key
+        m = re.search(r"(\d+\.\d) % of the MI355X datasheet peak \(([\d.]+) ", info)
+        assert m, (key, info)
+        assert float(m.group(2)) == peak, (key, info)
+        assert abs(float(m.group(1)) - 100.0 * float(text) / peak) <= 0.051, (key, info, text)
+    # rows without a datasheet line carry no percentage
+    for key in (("half_precision_compute", "half2"), ("integer_compute", "int4"), ("local_memory_bandwidth", "float4"),
+                ("transfer_bandwidth", "h2d_pinned"), ("kernel_launch_latency", "roundtrip")):
+        assert "datasheet" not in infos[key][2], key
+    # every family explains its own widths: no accumulators on the rows that load or pass data
+    for test in ("global_memory_bandwidth", "local_memory_bandwidth"):
+        for metric in ("float", "float2", "float4"):
+            info = infos[(test, metric)][2]
+            assert "accumulator" not in info and "bytes) per lane" in info, (test, metric, info)
+    assert "per lane and load instruction" in infos[("global_memory_bandwidth", "float4")][2]
+    assert "LDS store and load" in infos[("local_memory_bandwidth", "float2")][2]
+    assert "4 operations per instruction" in infos[("bfloat16_compute", "bf16")][2]
+
+
+def test_measured_rows_carry_their_fraction_of_the_datasheet_peak(tmp_path):
+    """Each reading with a datasheet line says what fraction of it was reached, in the one free-text field of a reading
+    (EmitOptions::description, include/common/logger.h:121-128, rendered by src/common/logger_text.cpp:238-243);
+    tags, metrics and units stay the reference's."""
+    x = tmp_path / "pct.xml"
+    assert run_cli("--xml-file", str(x)).returncode == 0
+    _check_percent_notes(_infos(x))
+    shown = run_cli("--describe", "--global-memory-bandwidth").stdout
+    assert "% of the MI355X datasheet" in " ".join(shown.split())
+
+
+def test_shipped_mi355x_result_file_carries_percentages_and_clocks():
+    infos = _infos(os.path.join(ROOT, "results", "AMD", "Instinct_MI355X.xml"))
+    _check_percent_notes(infos)
+    for key in (("mfma_fp16", "mfma_fp16"), ("smfmac_int8", "smfmac_int8"), ("mfma_mxfp4", "mfma_mxfp4")):
+        m = re.search(r"shader clock held: (\d+) MHz", infos[key][2])
+        assert m and 1000 <= int(m.group(1)) <= 2500, (key, infos[key][2])
+
+
 def test_the_product_holds_no_pretend_device(tmp_path):
     """The program and the library that ship know one device table, the entry points of libclpeak_mi355.so:
     no symbol or string of the tests' pretend device, no flag and no environment switch that selects one."""
