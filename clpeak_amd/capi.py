@@ -24,6 +24,7 @@ SYMBOLS = [
     "mi355_fill_f16", "mi355_fill_fp8_e5m2", "mi355_fill_i8", "mi355_gemm_f16", "mi355_gemm_i8", "mi355_gemm_fp8_e5m2",
     "mi355_gemm_f32", "mi355_gemm_f64", "mi355_fill_f64",
     "mi355_gemm_mxfp4", "mi355_gemm_mxfp4_static", "mi355_fill_bytes",
+    "mi355_gemm_mxfp4_prepare_scales", "mi355_gemm_mxfp4_prepared", "mi355_scratch_bytes",
 ]
 
 OK, ERR_ARG, ERR_HIP, ERR_NODEV, ERR_ARCH, ERR_OOM = 0, -1, -2, -3, -4, -5
@@ -98,6 +99,9 @@ def load_library(path=LIB_PATH):
     lib.mi355_gemm_fp8_e5m2.argtypes = [vp, vp, vp, vp, u32, u32, u32, C.c_float, C.c_float]
     lib.mi355_gemm_mxfp4.argtypes = [vp, vp, vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_gemm_mxfp4_static.argtypes = [vp, vp, vp, vp, vp, vp, u32, u32, u32]
+    lib.mi355_gemm_mxfp4_prepare_scales.argtypes = [vp, vp, vp, u32, u32, u32, vp]
+    lib.mi355_gemm_mxfp4_prepared.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32]
+    lib.mi355_scratch_bytes.argtypes = [vp, C.POINTER(C.c_size_t)]
     lib.mi355_fill_bytes.argtypes = [vp, vp, u64, u64, u32, u32, u32]
     lib.mi355_host_alloc.argtypes = [vp, C.c_size_t, C.POINTER(vp)]
     lib.mi355_host_free.argtypes = [vp, vp]
@@ -265,6 +269,17 @@ class Device:
 
     def gemm_mxfp4_static(self, A, B, SA, SB, Cbuf, M, N, K):
         self._check(self.lib.mi355_gemm_mxfp4_static(self.h, A.ptr, B.ptr, SA.ptr, SB.ptr, Cbuf.ptr, M, N, K))
+
+    def gemm_mxfp4_prepare_scales(self, SA, SB, M, N, K, prepared):
+        self._check(self.lib.mi355_gemm_mxfp4_prepare_scales(self.h, SA.ptr, SB.ptr, M, N, K, prepared.ptr))
+
+    def gemm_mxfp4_prepared(self, A, B, prepared, Cbuf, M, N, K):
+        self._check(self.lib.mi355_gemm_mxfp4_prepared(self.h, A.ptr, B.ptr, prepared.ptr, Cbuf.ptr, M, N, K))
+
+    def scratch_bytes(self):
+        n = C.c_size_t()
+        self._check(self.lib.mi355_scratch_bytes(self.h, C.byref(n)))
+        return n.value
 
     def fill_bytes(self, buf, n, seed, stream, lo, span):
         self._check(self.lib.mi355_fill_bytes(self.h, buf.ptr, n, seed, stream, lo, span))

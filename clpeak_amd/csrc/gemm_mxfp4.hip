@@ -64,28 +64,39 @@ mx_scale_layout_kernel(const uint8_t *__restrict__ SA, const uint8_t *__restrict
   }
 }
 
-// Shape and alignment checks shared by the two entry points.
-int check_mx_shapes(mi355_dev *dev, const void *A, const void *B, const void *scale_a, const void *scale_b, const void *C,
-                    uint32_t M, uint32_t N, uint32_t K) {
-  MI355_REQUIRE(dev, A && B && C && scale_a && scale_b, "gemm_mxfp4: null buffer");
+// A lane's offsets within its wave's 64 rows of a slab are 32-bit: a row of K (K/2 bytes) may be at most 64 MiB long.
+constexpr uint32_t kMaxRowBytes = 64u << 20;
+
+// Shape and alignment checks shared by the entry points; nothing is allocated or launched before they pass.
+int check_mx_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, uint32_t M, uint32_t N, uint32_t K) {
+  MI355_REQUIRE(dev, A && B && C, "gemm_mxfp4: null buffer");
   MI355_REQUIRE(dev, M > 0 && N > 0 && K > 0, "gemm_mxfp4: empty problem");
   MI355_REQUIRE(dev, M % kTile == 0 && N % kTile == 0, "gemm_mxfp4: M (%u) and N (%u) must be multiples of 256", M, N);
   MI355_REQUIRE(dev, K % 256 == 0, "gemm_mxfp4: K (%u) must be a multiple of 256", K);
+  MI355_REQUIRE(dev, K / 2u <= kMaxRowBytes, "gemm_mxfp4: a row of K is %u bytes, the kernel takes at most %u", K / 2u, kMaxRowBytes);
   MI355_REQUIRE(dev, (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15u) == 0, "gemm_mxfp4: buffers must be 16-byte aligned");
+  return MI355_OK;
+}
+int check_mx_scales(mi355_dev *dev, const void *scale_a, const void *scale_b) {
+  MI355_REQUIRE(dev, scale_a && scale_b, "gemm_mxfp4: null buffer");
   MI355_REQUIRE(dev, (((uintptr_t)scale_a | (uintptr_t)scale_b) & 7u) == 0, "gemm_mxfp4: scale arrays must be 8-byte aligned");
   return MI355_OK;
 }
 
-// Pre-pass into `lane_scales` (M*K/32 bytes for A, then N*K/32 for B), then the product.  Both on the handle's stream.
-int run_mx(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a, const uint8_t *scale_b,
-           uint16_t *C, uint32_t M, uint32_t N, uint32_t K, uint8_t *lane_scales) {
+// The pre-pass: scale_a / scale_b into `lane_scales` (M*K/32 bytes for A, then N*K/32 for B), on the handle's stream.
+int lay_out_scales(mi355_dev *dev, const uint8_t *scale_a, const uint8_t *scale_b, uint32_t M, uint32_t N, uint32_t K, uint8_t *lane_scales) {
   const uint32_t k32 = K / 32u, steps = K / 256u;
   uint8_t *sal = lane_scales, *sbl = sal + (size_t)M * k32;
   const uint32_t chunks = (steps + kLayoutSteps - 1) / kLayoutSteps;
   const uint32_t groups_a = M / 128u * chunks, groups_b = N / 128u * chunks;
   mx_scale_layout_kernel<<<groups_a + groups_b, 256, 0, dev->stream>>>(scale_a, scale_b, sal, sbl, k32, steps, groups_a, groups_b);
   MI355_LAUNCH_CHECK(dev, "mx_scale_layout");
-  return mi355_launch_gemm_quad_mx(dev, A, B, sal, sbl, C, M, N, K);
+  return MI355_OK;
+}
+
+// The product on scales already in per-lane order.
+int multiply_mx(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *lane_scales, uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
+  return mi355_launch_gemm_quad_mx(dev, A, B, lane_scales, lane_scales + (size_t)M * (K / 32u), C, M, N, K);
 }
 
 }  // namespace
@@ -109,7 +120,8 @@ int mi355_mx_resolve_static_scratch(mi355_dev *dev) {
 extern "C" int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
                                 const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
   MI355_ENTER(dev);
-  if (int rc = check_mx_shapes(dev, A, B, scale_a, scale_b, C, M, N, K)) return rc;
+  if (int rc = check_mx_shapes(dev, A, B, C, M, N, K)) return rc;
+  if (int rc = check_mx_scales(dev, scale_a, scale_b)) return rc;
   // lane-ordered copies of the scales live in a scratch buffer the handle keeps (same size as the scales)
   const size_t need = ((size_t)M + N) * (K / 32u);
   if (dev->mx_scratch_bytes < need) {
@@ -122,18 +134,47 @@ extern "C" int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t 
                                            "gemm_mxfp4: scratch of %zu bytes: %s", need, hipGetErrorString(e));
     dev->mx_scratch_bytes = need;
   }
-  return run_mx(dev, A, B, scale_a, scale_b, C, M, N, K, static_cast<uint8_t *>(dev->mx_scratch));
+  uint8_t *lane_scales = static_cast<uint8_t *>(dev->mx_scratch);
+  if (int rc = lay_out_scales(dev, scale_a, scale_b, M, N, K, lane_scales)) return rc;
+  return multiply_mx(dev, A, B, lane_scales, C, M, N, K);
+}
+
+extern "C" int mi355_gemm_mxfp4_prepare_scales(mi355_dev *dev, const uint8_t *scale_a, const uint8_t *scale_b, uint32_t M, uint32_t N,
+                                               uint32_t K, uint8_t *prepared) {
+  MI355_ENTER(dev);
+  MI355_REQUIRE(dev, prepared != nullptr && ((uintptr_t)prepared & 15u) == 0, "gemm_mxfp4_prepare_scales: the prepared buffer must be 16-byte aligned");
+  MI355_REQUIRE(dev, M > 0 && N > 0 && K > 0 && M % kTile == 0 && N % kTile == 0 && K % 256 == 0,
+                "gemm_mxfp4_prepare_scales: M (%u) and N (%u) must be multiples of 256 and K (%u) a multiple of 256", M, N, K);
+  if (int rc = check_mx_scales(dev, scale_a, scale_b)) return rc;
+  return lay_out_scales(dev, scale_a, scale_b, M, N, K, prepared);
+}
+
+extern "C" int mi355_gemm_mxfp4_prepared(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *prepared, uint16_t *C,
+                                         uint32_t M, uint32_t N, uint32_t K) {
+  MI355_ENTER(dev);
+  if (int rc = check_mx_shapes(dev, A, B, C, M, N, K)) return rc;
+  MI355_REQUIRE(dev, prepared != nullptr && ((uintptr_t)prepared & 15u) == 0, "gemm_mxfp4_prepared: the prepared scales must be 16-byte aligned");
+  return multiply_mx(dev, A, B, prepared, C, M, N, K);
 }
 
 extern "C" int mi355_gemm_mxfp4_static(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
                                        const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
   MI355_ENTER(dev);
-  if (int rc = check_mx_shapes(dev, A, B, scale_a, scale_b, C, M, N, K)) return rc;
+  if (int rc = check_mx_shapes(dev, A, B, C, M, N, K)) return rc;
+  if (int rc = check_mx_scales(dev, scale_a, scale_b)) return rc;
   const size_t need = ((size_t)M + N) * (K / 32u);
   MI355_REQUIRE(dev, need <= kStaticScaleBytes,
                 "gemm_mxfp4_static: (M + N) * K / 32 = %zu scale bytes exceed the static scratch of %zu bytes "
                 "(use mi355_gemm_mxfp4 for larger problems)", need, kStaticScaleBytes);
   MI355_REQUIRE(dev, dev->mx_static_scratch != nullptr, "gemm_mxfp4_static: the static scratch was not resolved when the device was opened");
   // The pre-pass overwrites every byte the product reads, so nothing of the previous call's contents has to be cleared.
-  return run_mx(dev, A, B, scale_a, scale_b, C, M, N, K, static_cast<uint8_t *>(dev->mx_static_scratch));
+  uint8_t *lane_scales = static_cast<uint8_t *>(dev->mx_static_scratch);
+  if (int rc = lay_out_scales(dev, scale_a, scale_b, M, N, K, lane_scales)) return rc;
+  return multiply_mx(dev, A, B, lane_scales, C, M, N, K);
+}
+
+extern "C" int mi355_scratch_bytes(mi355_dev *dev, size_t *handle_bytes) {
+  if (!dev || !handle_bytes) return mi355_fail(dev, MI355_ERR_ARG, "scratch_bytes: null argument");
+  *handle_bytes = dev->mx_scratch_bytes;
+  return MI355_OK;
 }

@@ -514,10 +514,9 @@ int mi355_launch_gemm_quad(mi355_dev *dev, int op, const char *what, const void 
   return mi355_fail(dev, MI355_ERR_ARG, "gemm: unknown operand kind %d", op);
 }
 
-// The block-scaled FP4 product; the caller (gemm_mxfp4.hip) has checked the shapes and laid the scale bytes out per
-// lane, both operands in blocks of 128 rows (16 bytes per lane and step).
+// The block-scaled FP4 product; the caller (gemm_mxfp4.hip) has checked the shapes (the row length among them) and
+// laid the scale bytes out per lane, both operands in blocks of 128 rows (16 bytes per lane and step).
 int mi355_launch_gemm_quad_mx(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scales_a, const uint8_t *scales_b,
                               uint16_t *C, uint32_t M, uint32_t N, uint32_t K) {
-  MI355_REQUIRE(dev, K / 2u <= kMaxRowBytes, "gemm_mxfp4: a row of K is %u bytes, the kernel takes at most %u", K / 2u, kMaxRowBytes);
   return launch_quad<kQuadMx>(dev, "gemm_mxfp4", A, B, C, M, N, K / 2u, 1.0f, scales_a, scales_b);
 }

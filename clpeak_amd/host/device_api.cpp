@@ -9,6 +9,7 @@ const Mi355Api &mi355_api() {
       mi355_mfma_dense, mi355_smfmac, mi355_gemm_bf16, mi355_gemm_fp8_e4m3,
       mi355_local_bandwidth, mi355_host_alloc, mi355_host_free, mi355_copy_async,
       mi355_fill_f16, mi355_fill_fp8_e5m2, mi355_fill_i8, mi355_gemm_f16, mi355_gemm_i8, mi355_gemm_fp8_e5m2,
-      mi355_gemm_mxfp4, mi355_fill_bytes, mi355_fill_f64, mi355_gemm_f32, mi355_gemm_f64};
+      mi355_gemm_mxfp4, mi355_fill_bytes, mi355_fill_f64, mi355_gemm_f32, mi355_gemm_f64,
+      mi355_gemm_mxfp4_prepare_scales, mi355_gemm_mxfp4_prepared};
   return api;
 }

@@ -43,6 +43,8 @@ struct Mi355Api {
   decltype(&mi355_fill_f64) fill_f64;
   decltype(&mi355_gemm_f32) gemm_f32;
   decltype(&mi355_gemm_f64) gemm_f64;
+  decltype(&mi355_gemm_mxfp4_prepare_scales) gemm_mxfp4_prepare_scales;
+  decltype(&mi355_gemm_mxfp4_prepared) gemm_mxfp4_prepared;
 };
 
 const Mi355Api &mi355_api();   // the table this binary is linked with

@@ -288,8 +288,20 @@ int mi355_gemm_f64(mi355_dev *dev, const double *A, const double *B, double *C,
  *          that the handle allocates on the first call and on growth, and frees in mi355_close. */
 int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
                      const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K);
-/*   The same product for callers that cannot allocate (code under HIP graph capture, tight serving
- *          loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Identical
+/*   The same product in two calls, for operands whose scales stay fixed over many products (weights): the
+ *          reference's timed loop hands the library the same scale pointers on every call
+ *          (src/rocm/hipblaslt_gemm.cpp:438-449 sets them once, :487-505 loops the product).
+ *          mi355_gemm_mxfp4_prepare_scales lays scale_a / scale_b out in the order the kernel loads them,
+ *          into `prepared` (caller-allocated device memory, (M + N) * K / 32 bytes, 16-byte aligned;
+ *          same M, N, K rules); mi355_gemm_mxfp4_prepared multiplies with them and launches nothing else.
+ *          The bytes of `prepared` mean something only to this library, for the M, N, K they were
+ *          prepared for.  Results are bit for bit those of mi355_gemm_mxfp4. */
+int mi355_gemm_mxfp4_prepare_scales(mi355_dev *dev, const uint8_t *scale_a, const uint8_t *scale_b,
+                                    uint32_t M, uint32_t N, uint32_t K, uint8_t *prepared);
+int mi355_gemm_mxfp4_prepared(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *prepared,
+                              uint16_t *C, uint32_t M, uint32_t N, uint32_t K);
+/*   The same product for callers that cannot allocate (tight serving loops, harnesses that forbid
+ *          hipMalloc).  No counterpart in the reference.  Identical
  *          arguments, checks and result; the lane-ordered scales go into a 4 MiB array that lives in
  *          the library's device image instead of a buffer of the handle, so the call performs no
  *          allocation and frees nothing.  Limit: (M + N) * K / 32 <= 4 MiB (8192^3 just fits);
@@ -299,6 +311,10 @@ int mi355_gemm_mxfp4(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const u
  *          overwrites all it reads. */
 int mi355_gemm_mxfp4_static(mi355_dev *dev, const uint8_t *A, const uint8_t *B, const uint8_t *scale_a,
                             const uint8_t *scale_b, uint16_t *C, uint32_t M, uint32_t N, uint32_t K);
+/* Bytes of device scratch memory the handle has allocated so far (today: the lane-ordered scales of
+ * mi355_gemm_mxfp4); 0 on a fresh handle, and unchanged by the entry points that allocate nothing.
+ * No counterpart in the reference; no HIP call. */
+int mi355_scratch_bytes(mi355_dev *dev, size_t *handle_bytes);
 /* Operands for it: dst[i] = lo + floor(span * (z >> 32) / 2^32), a uniform byte in [lo, lo+span)
  * (span 256, lo 0: random code pairs; lo 123, span 9: scales 2^-4 .. 2^4). */
 int mi355_fill_bytes(mi355_dev *dev, uint8_t *dst, uint64_t n, uint64_t seed, uint32_t stream,

@@ -88,6 +88,8 @@ int f_gemm_f16(mi355_dev *d, const uint16_t *, const uint16_t *, uint16_t *, uin
 int f_gemm_i8(mi355_dev *d, const int8_t *, const int8_t *, int32_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_i8"); return MI355_OK; }
 int f_gemm_e5m2(mi355_dev *d, const uint8_t *, const uint8_t *, uint16_t *, uint32_t, uint32_t, uint32_t, float, float) { FAKE_ENTRY(d, "gemm_fp8_e5m2"); return MI355_OK; }
 int f_gemm_mxfp4(mi355_dev *d, const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *, uint16_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_mxfp4"); return MI355_OK; }
+int f_mx_prepare(mi355_dev *d, const uint8_t *, const uint8_t *, uint32_t, uint32_t, uint32_t, uint8_t *) { FAKE_ENTRY(d, "gemm_mxfp4_prepare_scales"); return MI355_OK; }
+int f_mx_prepared(mi355_dev *d, const uint8_t *, const uint8_t *, const uint8_t *, uint16_t *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_mxfp4"); return MI355_OK; }
 int f_fill_bytes(mi355_dev *d, uint8_t *, uint64_t, uint64_t, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "fill_bytes"); return MI355_OK; }
 int f_fill_f64(mi355_dev *d, double *, uint64_t, uint64_t, uint32_t, int) { FAKE_ENTRY(d, "fill_f64"); return MI355_OK; }
 int f_gemm_f32(mi355_dev *d, const float *, const float *, float *, uint32_t, uint32_t, uint32_t) { FAKE_ENTRY(d, "gemm_f32"); return MI355_OK; }
@@ -101,6 +103,6 @@ const Mi355Api &mi355_api() {
       f_launch_roundtrip, f_mfma_dense, f_smfmac, f_gemm_bf16, f_gemm_fp8,
       f_local_bandwidth, f_host_alloc, f_host_free, f_copy_async,
       f_fill_f16, f_fill_e5m2, f_fill_i8, f_gemm_f16, f_gemm_i8, f_gemm_e5m2,
-      f_gemm_mxfp4, f_fill_bytes, f_fill_f64, f_gemm_f32, f_gemm_f64};
+      f_gemm_mxfp4, f_fill_bytes, f_fill_f64, f_gemm_f32, f_gemm_f64, f_mx_prepare, f_mx_prepared};
   return api;
 }

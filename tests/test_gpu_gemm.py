@@ -426,6 +426,49 @@ def test_gemm_mxfp4_workgroups_walk_several_tiles(dev, steps):
     _check_mx(dev, M, N, K, tiles, whole_output_finite=True)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (768, 512, 17 * 256), (17 * 256, 16 * 256, 2 * 256), (4096, 4096, 4096)])
+def test_gemm_mxfp4_prepared_scales_give_the_same_bits(dev, M, N, K):
+    """Scales laid out once (mi355_gemm_mxfp4_prepare_scales) and the product on them (mi355_gemm_mxfp4_prepared)
+    against the one-call form, which the tests above hold to the oracle: the same bits in every element of C, also on a
+    second product with the same prepared scales and new A, and nothing allocated by either call."""
+    dA, dB = dev.alloc(M * K // 2), dev.alloc(N * K // 2)
+    dSA, dSB = dev.alloc(M * K // 32), dev.alloc(N * K // 32)
+    prepared = dev.alloc((M + N) * K // 32)
+    c_one, c_two = dev.alloc(M * N * 2), dev.alloc(M * N * 2)
+    dev.fill_bytes(dB, N * K // 2, SEED, wl.STREAM_GEMM_B, 0, 256)
+    dev.fill_bytes(dSA, M * K // 32, SEED, wl.STREAM_SCALE_A, 123, 9); dev.fill_bytes(dSB, N * K // 32, SEED, wl.STREAM_SCALE_B, 123, 9)
+    before = dev.scratch_bytes()
+    dev.gemm_mxfp4_prepare_scales(dSA, dSB, M, N, K, prepared)
+    for salt in (0, 1):
+        dev.fill_bytes(dA, M * K // 2, SEED + salt, wl.STREAM_GEMM_A, 0, 256)
+        dev.memset(c_two, 0xff)
+        dev.gemm_mxfp4_prepared(dA, dB, prepared, c_two, M, N, K)
+        assert dev.scratch_bytes() == before
+        dev.memset(c_one, 0xff)
+        dev.gemm_mxfp4(dA, dB, dSA, dSB, c_one, M, N, K)
+        one, two = c_one.download(np.uint16, M * N), c_two.download(np.uint16, M * N)
+        assert not np.any((two & 0x7f80) == 0x7f80), "an element of C was never written"
+        assert np.array_equal(one, two), salt
+    for b in (dA, dB, dSA, dSB, prepared, c_one, c_two):
+        b.free()
+
+
+def test_gemm_mxfp4_refuses_before_it_allocates_or_launches(dev):
+    """A call that will be refused (a row of K past the 64 MiB the kernel's offsets reach, a misaligned scale array)
+    leaves the handle's scratch as it was: the checks come before the allocation and the pre-pass."""
+    small = dev.alloc(1 << 20)
+    before = dev.scratch_bytes()
+    K = (64 << 20) * 2 + 256           # 64 MiB + 128 bytes per row of two codes per byte
+    for call in (lambda: dev.gemm_mxfp4(small, small, small, small, small, 256, 256, K),
+                 lambda: dev.gemm_mxfp4_static(small, small, small, small, small, 256, 256, K),
+                 lambda: dev.gemm_mxfp4_prepared(small, small, small, small, 256, 256, K)):
+        with pytest.raises(capi.Mi355Error) as err:
+            call()
+        assert err.value.code == capi.ERR_ARG and "at most" in str(err.value)
+        assert dev.scratch_bytes() == before
+    small.free()
+
+
 def test_gemm_refuses_rows_longer_than_its_offsets_reach(dev):
     """A lane addresses its wave's 64 rows of a slab with 32-bit offsets: rows of K longer than 64 MiB are refused
     before anything is launched (the buffers here are never touched)."""

@@ -130,7 +130,7 @@ def test_describe_prints_wrapped_notes_under_headers_and_readings():
     assert desc.endswith("nothing but registers involved.")
     assert all(len(ln) <= 80 for ln in lines)
     f = next(i for i, ln in enumerate(lines) if re.fullmatch(r"      float    : \d+\.\d\d", ln))
-    assert lines[f + 1] == " " * (6 + 8 + 3) + "One value per lane at a time."
+    assert lines[f + 1].startswith(" " * (6 + 8 + 3) + "One value per lane at a time.")
     # a skipped reading carries its note too
     d = next(i for i, ln in enumerate(lines) if ln.startswith("      dispatch  : [unsupported] "))
     assert lines[d + 1].startswith(" " * (6 + 9 + 3)) and lines[d + 1].strip()

@@ -1,10 +1,10 @@
-"""Child process of test_gpu_vendor_parity.py: this library's GEMM next to the vendor library's (what the reference's
+"""Child process of test_zy_vendor_parity.py: this library's GEMM next to the vendor library's (what the reference's
 rocblas-fp / hipblaslt-fp8 / rocblas-int rows call, reached through torch.matmul, torch._scaled_mm and torch._int_mm) on
 the SAME operands, every element of C.  A process of its own: torch brings a HIP runtime that has to be the one to
 initialise the device in its process, so torch is imported first and this library is loaded behind it.
 
-Prints one line per kind, "<kind> ok ..." or "<kind> MISMATCH ...", or "SKIP <reason>"; exit status 0 unless a kind
-mismatches."""
+Prints "LOADED" once torch has initialised the device (the parent tells a slow import from a hung product by it), then
+one line per kind, "<kind> ok ..." or "<kind> MISMATCH ...", or "SKIP <reason>"; exit status 0 unless a kind mismatches."""
 import os
 import sys
 
@@ -17,6 +17,7 @@ try:
 except Exception as e:   # no torch, or no device for it
     print(f"SKIP torch not usable: {e!r}")
     sys.exit(0)
+print("LOADED", flush=True)
 import numpy as np  # noqa: E402
 
 from clpeak_amd import capi  # noqa: E402
