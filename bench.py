@@ -345,8 +345,45 @@ class _Telemetry:
         self.sclk = next(iter(sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))), None)
         cap = next(iter(sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"))), None)
         self.cap_w = self._read_uw(cap)
+        self.metrics = next(iter(sorted(glob.glob("/sys/class/drm/card*/device/gpu_metrics"))), None)
         self.samples = []
         self._run = False
+
+    # The driver's metrics table (sysfs gpu_metrics), format 1, content revision 8: the layout of the fields read here was
+    # checked on the box against the names `rocm-smi --showmetrics` gives the same numbers.  All little-endian.
+    #   @24 u64 energy_accumulator (units of 15.259 uJ)      @40 u32 accumulation_counter (one per millisecond)
+    #   @44.. u32 x5 accumulated throttler residencies: prochot, ppt (package power), socket thermal, vr thermal, hbm thermal
+    #   @288 u64 firmware_timestamp (10 ns)                   @296 u16 x8 current_gfxclk per XCD (MHz)
+    THROTTLERS = ("prochot", "ppt", "socket_thm", "vr_thm", "hbm_thm")
+
+    def snapshot(self):
+        """{"energy_j", "acc", residencies..., "gfxclk": [8], "fw_s"} or None when the table is absent or of another revision."""
+        import struct
+        try:
+            b = open(self.metrics, "rb").read()
+            size, fmt, rev = struct.unpack_from("<HBB", b, 0)
+            if (fmt, rev) != (1, 8) or len(b) < 312:
+                return None
+            out = {"energy_j": struct.unpack_from("<Q", b, 24)[0] * 15.259e-6, "acc": struct.unpack_from("<I", b, 40)[0],
+                   "fw_s": struct.unpack_from("<Q", b, 288)[0] * 1e-8, "gfxclk": list(struct.unpack_from("<8H", b, 296))}
+            out.update(zip(self.THROTTLERS, struct.unpack_from("<5I", b, 44)))
+            return out
+        except (OSError, TypeError, struct.error):
+            return None
+
+    @classmethod
+    def between(cls, a, b):
+        """What the table says happened between two snapshots: mean power from the energy counter, and for each throttler
+        the share of the firmware's accumulation cycles in which it was active (its residency)."""
+        if a is None or b is None:
+            return {}
+        cycles = (b["acc"] - a["acc"]) & 0xffffffff
+        dt = b["fw_s"] - a["fw_s"]
+        out = {"watts_energy_counter": round((b["energy_j"] - a["energy_j"]) / dt, 1) if dt > 0 else None,
+               "gfxclk_mhz_per_xcd": b["gfxclk"]}
+        for k in cls.THROTTLERS:
+            out[k + "_residency"] = round(((b[k] - a[k]) & 0xffffffff) / cycles, 4) if cycles else None
+        return out
 
     @staticmethod
     def _read_uw(path):
@@ -471,22 +508,44 @@ def power_table(dev, seconds):
     tel = _Telemetry()
     out = []
 
-    def run(label, fn, work, unit):
+    idle_w = [None]
+
+    def run(label, fn, work, unit, clock_buf=None):
+        """work: operations (or bytes) per launch; clock_buf: where the kernel leaves its two loop counters."""
         fn(); dev.sync()
         tel.start()
         t0 = time.perf_counter()
         n = 0
+        snap0 = None
         while time.perf_counter() - t0 < seconds:
+            if snap0 is None and time.perf_counter() - t0 >= 0.5:
+                snap0 = tel.snapshot()            # the driver's table from 0.5 s into the load ...
             us = dev.time_launches(fn, 50)      # HIP events around 50 launches; returns synchronised
             n += 50
             last_us = us / 50
+        snap1 = tel.snapshot()                    # ... to its end
         stats = tel.stop()
+        stats.update(tel.between(snap0, snap1))
         row = {"workload": label, "us_per_launch": round(last_us, 2), "value": round(work / last_us / 1e6, 1), "unit": unit, **stats}
+        if clock_buf is not None:
+            c = clock_buf.download(np.uint64, 2)
+            row["clock_in_kernel_mhz"] = round(float(c[0]) / max(float(c[1]), 1.0) * 100.0, 0)
+        if idle_w[0] and stats.get("watts_mean"):
+            # energy per operation (or byte) above the idle board, and the rate the package power cap would allow at that
+            # energy: value x (cap - idle) / (W - idle), in the unit of value
+            per_s = row["value"] * (1e12 if unit in ("tflops", "tops") else 1e9)
+            row["pj_per_op_above_idle"] = round((stats["watts_mean"] - idle_w[0]) / per_s * 1e12, 4)
+            if tel.cap_w:
+                row["rate_at_power_cap"] = round(row["value"] * (tel.cap_w - idle_w[0]) / (stats["watts_mean"] - idle_w[0]), 1)
+                row["of_rate_at_power_cap"] = round(row["value"] / row["rate_at_power_cap"], 4)
         out.append(row)
         print(json.dumps(row), flush=True)
 
     t0 = time.perf_counter()
+    snap0 = tel.snapshot()
     tel.start(); time.sleep(min(seconds, 2.0)); idle = tel.stop(skip_s=0.0)
+    idle.update(tel.between(snap0, tel.snapshot()))
+    idle_w[0] = idle.get("watts_mean")
     print(json.dumps({"workload": "idle", "power_cap_w": tel.cap_w, **idle}), flush=True)
     M = N = K = 8192
     dA, dB, dC = dev.alloc(M * K * 2), dev.alloc(N * K * 2), dev.alloc(M * N * 2)
@@ -513,29 +572,34 @@ def power_table(dev, seconds):
         b.free()
     waves, iters = 2048, 4096
     clk = dev.alloc(16)
-    for kind in (capi.MFMA_BF16_16x16x32, capi.MFMA_F16_32x32x16, capi.MFMA_MXFP6_E3M2):
+    # the register-resident rows as they are reported (one operand set per wave), every kind on seeded operands and four
+    # of them on zero operands as well
+    with_zero = (capi.MFMA_BF16_16x16x32, capi.MFMA_F16_32x32x16, capi.MFMA_MXFP6_E3M2)
+    for kind in sorted(wl.DENSE):
         sh = wl.DENSE[kind]
-        for zero in (False, True):
+        for zero in (False, True) if kind in with_zero else (False,):
             A, B, sA, sB = wl.dense_inputs(kind, waves, SEED)
             if zero:
                 A, B = np.zeros_like(A), np.zeros_like(B)
             bufs = [dev.from_host(A), dev.from_host(B), dev.from_host(sA) if sA is not None else None, dev.from_host(sB) if sB is not None else None]
             o = dev.alloc(waves * 4 * sh["M"] * sh["N"] * 4)
             run(f"{sh['name']} {sh['shape']}, {'zero' if zero else 'seeded'} operands",
-                lambda: dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], o, waves, iters, clk), wl.dense_flops(kind, waves, iters), "tflops")
+                lambda: dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], o, waves, iters, clk, one_set=True), wl.dense_flops(kind, waves, iters),
+                "tops" if sh["fmt"] == wl.I8 else "tflops", clock_buf=clk)
             for b in bufs + [o]:
                 if b is not None:
                     b.free()
-    for kind in (capi.SMFMAC_F16_16x16x64,):
+    for kind in sorted(wl.SPARSE):
         sh = wl.SPARSE[kind]
-        for zero in (False, True):
+        for zero in (False, True) if kind == capi.SMFMAC_F16_16x16x64 else (False,):
             Ac, meta, B = wl.sparse_inputs(kind, waves, SEED)
             if zero:
                 Ac, B = np.zeros_like(Ac), np.zeros_like(B)
             bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
             o = dev.alloc(waves * 4 * 256 * 4)
             run(f"{sh['name']} {sh['shape']}, {'zero' if zero else 'seeded'} operands",
-                lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk), wl.sparse_flops(kind, waves, iters), "tflops")
+                lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk, one_set=True), wl.sparse_flops(kind, waves, iters),
+                "tops" if sh["fmt"] == wl.I8 else "tflops", clock_buf=clk)
             for b in bufs + [o]:
                 b.free()
     # How fast the limit acts: isolated launches of increasing length (the board idle for 4 ms before each), with the

@@ -68,31 +68,35 @@ __global__ void __launch_bounds__(256)
 mad_f16_kernel(uint64_t seed, uint16_t a_bits, uint32_t steps, uint64_t n_items, uint16_t *__restrict__ out) {
   const uint64_t item = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (item >= n_items) return;
-  const _Float16 a = bits_to_half(a_bits);
+  const _Float16 a = bits_to_half(a_bits);   // 0x3bfe (the scalar form below carries it as a literal)
   _Float16 sum = (_Float16)0;
   if constexpr (W == 1) {
-    // One v_fma_f16 per step and accumulator, as the reference's scalar row (its __hfma chains,
+    // One scalar half multiply-add per step and accumulator, as the reference's scalar row (its __hfma chains,
     // src/rocm/rocm_kernels/compute_hp.hip:12-30).  Written as the instruction itself, on 32-bit registers
     // that hold a half in their low 16 bits: from the plain expression the compiler pairs neighbouring chains
     // into v_pk_fma_f16 and the row becomes the half2 row.  The arithmetic is the same correctly rounded half
     // FMA either way.
     uint32_t x0[kAcc], x[kAcc];
-    uint32_t a32 = a_bits;
-    asm volatile("" : "+v"(a32));   // a vector register: the 16-bit literal form would be another encoding
 #pragma unroll
     for (int j = 0; j < kAcc; j++) {
       x0[j] = mi355_f32_to_f16(mi355_rng_upm1(mi355_rng_word(seed, MI355_STREAM_MAD, item * kAcc + j)));
       x[j] = x0[j];
     }
+    // (v_fma_f16 issues once per 8 cycles and SIMD on this part, with the multiplier in a vector or in a scalar register
+    // alike: 38.5 TFLOP/s where the packed form, two lanes per instruction every 4 cycles, reaches 147.)
+    uint32_t a32 = a_bits;
+    asm volatile("" : "+v"(a32));
+#define MI355_HALF_STEP(j) asm volatile("v_fma_f16 %0, %0, %1, %2" : "+v"(x[j]) : "v"(a32), "v"(x0[j]))
     for (uint32_t b = 0; b < steps / 8; b++) {   // 128 instructions per trip: the branch of a shorter one shows
 #pragma unroll
       for (int t = 0; t < 8; t++)
 #pragma unroll
-        for (int j = 0; j < kAcc; j++) asm volatile("v_fma_f16 %0, %0, %1, %2" : "+v"(x[j]) : "v"(a32), "v"(x0[j]));
+        for (int j = 0; j < kAcc; j++) MI355_HALF_STEP(j);
     }
     for (uint32_t r = 0; r < steps % 8; r++)
 #pragma unroll
-      for (int j = 0; j < kAcc; j++) asm volatile("v_fma_f16 %0, %0, %1, %2" : "+v"(x[j]) : "v"(a32), "v"(x0[j]));
+      for (int j = 0; j < kAcc; j++) MI355_HALF_STEP(j);
+#undef MI355_HALF_STEP
 #pragma unroll
     for (int j = 0; j < kAcc; j++) sum += bits_to_half((uint16_t)x[j]);
   } else {

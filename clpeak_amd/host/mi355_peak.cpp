@@ -201,7 +201,7 @@ void Mi355Peak::runDevice(int ordinal, logger::BackendScope &backend) {
       {{"float", 1, chainWidthNote(1)}, {"float2", 2, chainWidthNote(2)}, {"float4", 4, chainWidthNote(4)}, {nullptr, 0, nullptr}}};
   static const MadTest hp = {Benchmark::ComputeHP, "half_precision_compute", "Half-precision compute", "gflops",
       "The same chains in IEEE half precision; the packed form does two lanes per instruction.", MI355_MAD_F16, 2, 2, 0.0, "",
-      {{"half", 1, "One scalar half-precision multiply-add per step and accumulator."}, {"half2", 2, "Packed: two half-precision multiply-adds per lane and instruction."}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
+      {{"half", 1, "One scalar half-precision multiply-add per step and accumulator (the scalar instruction issues at half the rate of the packed one)."}, {"half2", 2, "Packed: two half-precision multiply-adds per lane and instruction."}, {nullptr, 0, nullptr}, {nullptr, 0, nullptr}}};
   static const MadTest dp = {Benchmark::ComputeDP, "double_precision_compute", "Double-precision compute", "gflops",
       "The same chains on 64-bit floats.", MI355_MAD_F64, 8, 2, peaks::kVectorFp64Gflops, "GFLOPS vector fp64",
       {{"double", 1, chainWidthNote(1)}, {"double2", 2, chainWidthNote(2)}, {"double4", 4, chainWidthNote(4)}, {nullptr, 0, nullptr}}};
