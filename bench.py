@@ -1004,8 +1004,8 @@ def compact_line(full):
 HEADLINE_BLOCKS_PER_CU = 1
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in
 # KiB per dispatch), each scaled by what the counter reads for the plain copy kernel of known size
-# (FETCH_SIZE x 2.0000, WRITE_SIZE x 1.0000): profiles/hbm_float4_read_4GiB_traffic.md.
-TRAFFIC_BYTES_PER_LAUNCH = 4295168000
+# (FETCH_SIZE x 2.0000, WRITE_SIZE x 1.0000 to four decimals): profiles/hbm_float4_read_4GiB_traffic.md.
+TRAFFIC_BYTES_PER_LAUNCH = 4295171094
 
 if __name__ == "__main__":
     main()

@@ -92,10 +92,13 @@ def test_traffic_figure_is_the_committed_profile():
     m = re.search(r"=\s*\*\*(\d+) bytes\*\*", text)
     assert m, "no scaled traffic figure in the profile"
     assert int(m.group(1)) == bench.TRAFFIC_BYTES_PER_LAUNCH
-    # and the figure follows from the table's own rows: FETCH_SIZE x 2 + WRITE_SIZE x 1, KiB per dispatch
-    rows = dict(re.findall(r"\| global_bandwidth_kernel<float4, 6>[^|]*\| (FETCH_SIZE|WRITE_SIZE) \| \d+ \| (\d+) \|", text))
-    from_rows = int(rows["FETCH_SIZE"]) * 1024 * 2 + int(rows["WRITE_SIZE"]) * 1024
-    assert abs(from_rows - bench.TRAFFIC_BYTES_PER_LAUNCH) <= 1e-4 * from_rows   # the table prints six significant digits
+    # and the figure follows from the table's own rows: each counter (KiB per dispatch) scaled by what it reads for the
+    # copy kernel of known size (1 GiB each way)
+    kib = {(k, c): float(v) for k, c, v in re.findall(r"\| (copy_kernel|global_bandwidth_kernel<float4, 6>)[^|]*\| (FETCH_SIZE|WRITE_SIZE) \| \d+ \| ([\d.]+) \|", text)}
+    read = kib[("global_bandwidth_kernel<float4, 6>", "FETCH_SIZE")] * (1048576.0 / kib[("copy_kernel", "FETCH_SIZE")]) * 1024
+    written = kib[("global_bandwidth_kernel<float4, 6>", "WRITE_SIZE")] * (1048576.0 / kib[("copy_kernel", "WRITE_SIZE")]) * 1024
+    assert abs(read + written - bench.TRAFFIC_BYTES_PER_LAUNCH) <= 64        # the table prints two decimals of a KiB
+    assert 0.999 <= (1 << 32) / bench.TRAFFIC_BYTES_PER_LAUNCH <= 1.0         # the read kernel fetches what it must and no more
     # the profile names the grid it measured; it is the grid the headline launches
     assert "65536 threads" in text and bench.HEADLINE_BLOCKS_PER_CU * 256 * 256 == 65536
 
