@@ -40,14 +40,37 @@ PEAK = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "fp6": 101
 SEED = 0x5EEDC1BEA4D355
 
 
-def timed(dev, launch, min_us=300e3, warm_us=300e3, max_iters=10000):
+def timed(dev, launch, min_us=300e3, warm_us=300e3, max_iters=10000, board=None):
     """Reference discipline (warm-up, probe, batch sized to a time budget), with the warm-up
-    long enough for the clocks to settle under this kernel's load.  Returns us per launch."""
+    long enough for the clocks to settle under this kernel's load.  Returns us per launch.
+    board: a dict that receives what the board said during the timed batch (mean power, the share of the time the package
+    power limiter was active), where the machine lets an ordinary user read that."""
     launch(); dev.sync()
     probe = max(dev.time_launches(launch, 1), 1.0)
     dev.time_launches(launch, int(min(max(warm_us / probe, 2), max_iters)))
     n = int(min(max(min_us / probe, 1), max_iters))
-    return dev.time_launches(launch, n) / n, n
+    if board is None:
+        return dev.time_launches(launch, n) / n, n
+    tel = _board_telemetry()
+    snap0 = tel.snapshot()
+    tel.start()
+    us = dev.time_launches(launch, n) / n
+    stats = tel.stop(skip_s=0.0)
+    between = tel.between(snap0, tel.snapshot())
+    if stats.get("watts_mean") is not None:
+        board["watts"] = stats["watts_mean"]
+    if between.get("ppt_residency") is not None:
+        board["ppt_residency"] = between["ppt_residency"]
+    return us, n
+
+
+_TELEMETRY = []
+
+
+def _board_telemetry():
+    if not _TELEMETRY:
+        _TELEMETRY.append(_Telemetry())
+    return _TELEMETRY[0]
 
 
 def bench_rows(dev, quick, only):
@@ -168,11 +191,12 @@ def _matrix_rows(dev, wl, add, budget, only, zero, one_set, reference=False):
         bufs = [dev.from_host(A), dev.from_host(B), dev.from_host(sA) if sA is not None else None,
                 dev.from_host(sB) if sB is not None else None]
         o = dev.alloc(waves * 4 * s["M"] * s["N"] * 4)
-        us, _ = timed(dev, lambda: dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], o, waves, iters, clk, one_set=one_set), **budget)
+        board = {}
+        us, _ = timed(dev, lambda: dev.mfma_dense(kind, bufs[0], bufs[1], bufs[2], bufs[3], o, waves, iters, clk, one_set=one_set), board=board, **budget)
         c = clk.download(np.uint64, 2)
         unit = "tops" if s["fmt"] == wl.I8 else "tflops"
         add(s["name"], s["name"] + tail, wl.dense_flops(kind, waves, iters) / us / 1e6, unit, us, PEAK[peaks[kind]],
-            shape=s["shape"], sclk_mhz=round(float(c[0]) / max(float(c[1]), 1.0) * 100.0, 0))
+            shape=s["shape"], sclk_mhz=round(float(c[0]) / max(float(c[1]), 1.0) * 100.0, 0), **board)
         for b in bufs + [o]:
             if b is not None:
                 b.free()
@@ -184,11 +208,12 @@ def _matrix_rows(dev, wl, add, budget, only, zero, one_set, reference=False):
             Ac, B = np.zeros_like(Ac), np.zeros_like(B)
         bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
         o = dev.alloc(waves * 4 * 256 * 4)
-        us, _ = timed(dev, lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk, one_set=one_set), **budget)
+        board = {}
+        us, _ = timed(dev, lambda: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk, one_set=one_set), board=board, **budget)
         c = clk.download(np.uint64, 2)
         unit = "tops" if s["fmt"] == wl.I8 else "tflops"
         add(s["name"], s["name"] + tail, wl.sparse_flops(kind, waves, iters) / us / 1e6, unit, us, 2 * PEAK[speaks[kind]],
-            shape=s["shape"], sclk_mhz=round(float(c[0]) / max(float(c[1]), 1.0) * 100.0, 0))
+            shape=s["shape"], sclk_mhz=round(float(c[0]) / max(float(c[1]), 1.0) * 100.0, 0), **board)
         for b in bufs + [o]:
             b.free()
     clk.free()
@@ -252,8 +277,9 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
             # part holds a higher clock
             dev.memset(dA, const_byte); dev.memset(dB, const_byte)
             metric += " constant operands"
-        us, _ = timed(dev, fn, **budget)
-        add(test, metric, 2.0 * M * N * K / us / 1e6, unit, us, PEAK[peak], shape="8192x8192x8192")
+        board = {}
+        us, _ = timed(dev, fn, board=board, **budget)
+        add(test, metric, 2.0 * M * N * K / us / 1e6, unit, us, PEAK[peak], shape="8192x8192x8192", **board)
         if metric.startswith("mxf4_e2m1"):
             us, _ = timed(dev, lambda: dev.gemm_mxfp4(dA, dB, dSA, dSB, dC, M, N, K), **budget)
             add(test, metric + ", scale layout on every call", 2.0 * M * N * K / us / 1e6, unit, us, PEAK[peak], shape="8192x8192x8192")
@@ -984,18 +1010,24 @@ def compact_line(full):
     # which launch the matrix fractions are: the four accumulator chains of a wave share one A and one B
     # fragment (the rows "distinct operands per chain" in the rows file are the other launch)
     line["mfma_operands"] = "one set per wave"
-    # the shader clock the part held under each matrix row that is below its target
+    # for each matrix or GEMM row below its target: [clock held (MHz, read inside the kernel; null for the GEMMs, which do not
+    # read it), board power during the timed batch (W), share of the batch in which the package power limiter was active (%)]
     held = {}
     for key, test, metric in FRAC_KEYS:
         r = by_key.get((test, metric))
-        target = TARGET_FRAC.get(key.split("_")[0]) if key.startswith(("mfma", "smfmac")) else None   # the rows that read the clock
-        if r is not None and target and "sclk_mhz" in r and r.get("frac", 1.0) < target:
-            held[key] = int(r["sclk_mhz"])
-    line["sclk_mhz"] = held
+        target = TARGET_FRAC.get(key.split("_")[0]) if key.startswith(("mfma", "smfmac")) or key == "gemm_bf16_seeded" else None
+        if r is not None and target and r.get("frac", 1.0) < target and ("sclk_mhz" in r or "watts" in r):
+            ppt = r.get("ppt_residency")
+            held[key] = [int(r["sclk_mhz"]) if "sclk_mhz" in r else None, int(round(r["watts"])) if "watts" in r else None,
+                         int(round(100 * ppt)) if ppt is not None else None]
+    line["below_target_mhz_w_pptpct"] = held
     lat = by_key.get(("kernel_launch_latency", "roundtrip"))
     if lat is not None:
         line["launch_roundtrip_us"] = lat["value"]
     line["rows_file"] = full.get("rows_file")
+    # the record must fit a reader that keeps a 2000-byte tail of stdout: the free text gives way first (it is whole in the rows file)
+    while len(json.dumps(line, separators=(",", ":")).encode()) > 1950 and line["cpu_baseline"] and line["cpu_baseline"]["sample"]:
+        line["cpu_baseline"]["sample"] = line["cpu_baseline"]["sample"][:-20]
     return line
 
 

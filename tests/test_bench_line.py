@@ -16,7 +16,8 @@ def _synthetic_full(with_cpu=True):
     rows = []
     for _, test, metric in bench.FRAC_KEYS:
         rows.append({"test": test, "metric": metric, "value": 123456.78, "unit": "tflops", "us_per_launch": 12345.67,
-                     "peak": 10100.0, "frac": 0.98765, "shape": "8192x8192x8192", "sclk_mhz": 2399.0})
+                     "peak": 10100.0, "frac": 0.98765, "shape": "8192x8192x8192", "sclk_mhz": 2399.0, "watts": 1399.6,
+                     "ppt_residency": 0.8741})
     # rows without a peak and rows the compact record leaves out
     rows.append({"test": "kernel_launch_latency", "metric": "roundtrip", "value": 9.47, "unit": "us", "us_per_launch": 9.47})
     for i in range(80):
@@ -56,7 +57,7 @@ def test_compact_line_is_small_and_complete():
         assert key in line["fracs"], key
     assert line["launch_roundtrip_us"] == 9.47
     assert line["mfma_operands"] == "one set per wave"
-    assert line["sclk_mhz"] == {}          # every synthetic row is above its target
+    assert line["below_target_mhz_w_pptpct"] == {}          # every synthetic row is above its target
 
 
 def test_compact_line_names_the_held_clock_of_rows_below_target():
@@ -65,9 +66,9 @@ def test_compact_line_names_the_held_clock_of_rows_below_target():
         r["frac"] = 0.5                    # everything below target: the largest the record can get
     text = json.dumps(bench.compact_line(full), separators=(",", ":"))
     assert len(text.encode()) < 2000, len(text)
-    held = json.loads(text)["sclk_mhz"]
-    assert held["smfmac_fp16"] == 2399 and held["mfma_fp16_32x32x16"] == 2399 and len(held) == 15
-    assert not [k for k in held if not k.startswith(("mfma", "smfmac"))]     # the rows that read the clock in the kernel
+    held = json.loads(text)["below_target_mhz_w_pptpct"]
+    assert held["smfmac_fp16"] == [2399, 1400, 87] and held["mfma_fp16_32x32x16"] == [2399, 1400, 87] and len(held) == 16
+    assert [k for k in held if not k.startswith(("mfma", "smfmac"))] == ["gemm_bf16_seeded"]
 
 
 def test_emit_prints_the_compact_record_last(tmp_path):
