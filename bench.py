@@ -47,13 +47,13 @@ def timed(dev, launch, min_us=300e3, warm_us=300e3, max_iters=10000, board=None)
     power limiter was active), where the machine lets an ordinary user read that."""
     launch(); dev.sync()
     probe = max(dev.time_launches(launch, 1), 1.0)
+    tel = _board_telemetry() if board is not None else None
+    snap0 = tel.snapshot() if tel else None      # the driver's table: from the start of the warm-up to the end of the batch
     dev.time_launches(launch, int(min(max(warm_us / probe, 2), max_iters)))
     n = int(min(max(min_us / probe, 1), max_iters))
     if board is None:
         return dev.time_launches(launch, n) / n, n
-    tel = _board_telemetry()
-    snap0 = tel.snapshot()
-    tel.start()
+    tel.start()                                  # the power reading: sampled during the timed batch, behind the warm-up
     us = dev.time_launches(launch, n) / n
     stats = tel.stop(skip_s=0.0)
     between = tel.between(snap0, tel.snapshot())
@@ -628,6 +628,28 @@ def power_table(dev, seconds):
                 "tops" if sh["fmt"] == wl.I8 else "tflops", clock_buf=clk)
             for b in bufs + [o]:
                 b.free()
+    # Where the limit acts: the same seeded launch with only part of the chip taking part (the other workgroups return at
+    # once).  A limit on the package would let four busy XCDs, at half the power, run faster than eight.
+    subsets = (("XCDs 0-3 only", dict(on_xcds=(0, 1, 2, 3)), 0.5), ("XCDs 0-1 only", dict(on_xcds=(0, 1)), 0.25), ("XCD 0 only", dict(on_xcds=(0,)), 0.125),
+               ("XCDs 0 and 4 only", dict(on_xcds=(0, 4)), 0.25), ("half the CUs of every XCD", dict(half_cus=True), 0.5))
+    for sparse, kind in ((True, capi.SMFMAC_F16_16x16x64), (False, capi.MFMA_F16_32x32x16), (False, capi.MFMA_BF16_16x16x32)):
+        sh = (wl.SPARSE if sparse else wl.DENSE)[kind]
+        if sparse:
+            Ac, meta, B = wl.sparse_inputs(kind, waves, SEED)
+            bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
+            work = wl.sparse_flops(kind, waves, iters)
+            o = dev.alloc(waves * 4 * 256 * 4)
+            fn = lambda **kw: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, clk, one_set=True, **kw)
+        else:
+            A, B, _, _ = wl.dense_inputs(kind, waves, SEED)
+            bufs = [dev.from_host(A), dev.from_host(B)]
+            work = wl.dense_flops(kind, waves, iters)
+            o = dev.alloc(waves * 4 * sh["M"] * sh["N"] * 4)
+            fn = lambda **kw: dev.mfma_dense(kind, bufs[0], bufs[1], None, None, o, waves, iters, clk, one_set=True, **kw)
+        for label, kw, share in subsets:
+            run(f"{sh['name']} {sh['shape']}, seeded operands, {label}", lambda: fn(**kw), work * share, "tflops", clock_buf=clk)
+        for b in bufs + [o]:
+            b.free()
     # How fast the limit acts: isolated launches of increasing length (the board idle for 4 ms before each), with the
     # clock read inside the kernel (shader cycles over a constant-rate counter, by wave 0).  A limit on average power
     # would let a short launch from an idle board run at the boost clock.

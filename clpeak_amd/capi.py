@@ -34,6 +34,7 @@ MAD_F32, MAD_F16, MAD_F64, MAD_MP, MAD_BF16, MAD_I32, MAD_I8DP = range(7)
 (MFMA_F16_16x16x32, MFMA_BF16_16x16x32, MFMA_F16_32x32x16, MFMA_BF16_32x32x16, MFMA_I8_16x16x64,
  MFMA_FP8_16x16x128, MFMA_BF8_16x16x128, MFMA_MXFP6_E2M3, MFMA_MXFP6_E3M2, MFMA_MXFP4_E2M1) = range(10)
 SMFMAC_F16_16x16x64, SMFMAC_BF16_16x16x64, SMFMAC_FP8_16x16x128, SMFMAC_BF8_16x16x128, SMFMAC_I8_16x16x128 = range(5)
+MATRIX_ON_HALF_THE_CUS = 0x200   # diagnosis: only the workgroups of the first 16 CUs of every XCD take part
 MFMA_ONE_OPERAND_SET = 0x100   # OR into an MFMA / SMFMAC kind: every chain of a wave takes chain 0's operands
 
 # Stream ids of the seeded generator (clpeak_amd/csrc/seeded_rng.h).
@@ -246,14 +247,22 @@ class Device:
         self._check(self.lib.mi355_launch_roundtrip(self.h, warmup, launches, C.byref(us)))
         return us.value
 
-    def mfma_dense(self, kind, A, B, scaleA, scaleB, out, waves, iters, clocks=None, one_set=False):
-        kind |= MFMA_ONE_OPERAND_SET if one_set else 0
+    @staticmethod
+    def _subset(on_xcds, half_cus):
+        """The diagnosis bits of a matrix kind: on_xcds = iterable of XCD numbers that take part (None: all)."""
+        bits = MATRIX_ON_HALF_THE_CUS if half_cus else 0
+        if on_xcds is not None:
+            bits |= (sum(1 << x for x in on_xcds) & 0xff) << 16
+        return bits
+
+    def mfma_dense(self, kind, A, B, scaleA, scaleB, out, waves, iters, clocks=None, one_set=False, on_xcds=None, half_cus=False):
+        kind |= (MFMA_ONE_OPERAND_SET if one_set else 0) | self._subset(on_xcds, half_cus)
         self._check(self.lib.mi355_mfma_dense(self.h, kind, A.ptr, B.ptr, scaleA.ptr if scaleA else None,
                                               scaleB.ptr if scaleB else None, out.ptr, waves, iters,
                                               clocks.ptr if clocks else None))
 
-    def smfmac(self, kind, Ac, meta, B, out, waves, iters, clocks=None, one_set=False):
-        kind |= MFMA_ONE_OPERAND_SET if one_set else 0
+    def smfmac(self, kind, Ac, meta, B, out, waves, iters, clocks=None, one_set=False, on_xcds=None, half_cus=False):
+        kind |= (MFMA_ONE_OPERAND_SET if one_set else 0) | self._subset(on_xcds, half_cus)
         self._check(self.lib.mi355_smfmac(self.h, kind, Ac.ptr, meta.ptr, B.ptr, out.ptr, waves, iters,
                                           clocks.ptr if clocks else None))
 

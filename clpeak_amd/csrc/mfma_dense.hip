@@ -144,7 +144,9 @@ template <typename Tr, bool ONE_SET>
 __global__ void __launch_bounds__(256)
 mfma_dense_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B,
                   const uint8_t *__restrict__ sA, const uint8_t *__restrict__ sB,
-                  typename Tr::Out *__restrict__ out, uint32_t iters, uint64_t *__restrict__ clocks) {
+                  typename Tr::Out *__restrict__ out, uint32_t iters, uint64_t *__restrict__ clocks, uint32_t active) {
+  // diagnosis: only the workgroups of some XCDs (index mod 8) or of half the CUs of every XCD take part
+  if (!((active >> (blockIdx.x % 8u)) & 1u) || ((active & 0x100u) && (blockIdx.x / 8u) % 32u >= 16u)) return;
   const int lane = threadIdx.x % 64;
   const uint64_t wave = (uint64_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
   constexpr size_t a_bytes = (size_t)Tr::M * Tr::row_bytes, b_bytes = (size_t)Tr::N * Tr::row_bytes;
@@ -203,14 +205,14 @@ mfma_dense_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B,
 
 template <typename Tr>
 int launch(mi355_dev *dev, bool one_set, const void *A, const void *B, const uint8_t *sA, const uint8_t *sB, void *out,
-           uint32_t waves, uint32_t iters, uint64_t *clocks) {
+           uint32_t waves, uint32_t iters, uint64_t *clocks, uint32_t active) {
   if (Tr::scaled && (!sA || !sB)) return mi355_fail(dev, MI355_ERR_ARG, "mfma_dense: scaled kind needs scaleA and scaleB");
   if (one_set)
     mfma_dense_kernel<Tr, true><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)A, (const uint8_t *)B, sA, sB,
-                                                                   (typename Tr::Out *)out, iters, clocks);
+                                                                   (typename Tr::Out *)out, iters, clocks, active);
   else
     mfma_dense_kernel<Tr, false><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)A, (const uint8_t *)B, sA, sB,
-                                                                    (typename Tr::Out *)out, iters, clocks);
+                                                                    (typename Tr::Out *)out, iters, clocks, active);
   MI355_LAUNCH_CHECK(dev, "mfma_dense");
   return MI355_OK;
 }
@@ -224,18 +226,22 @@ extern "C" int mi355_mfma_dense(mi355_dev *dev, int kind, const void *A, const v
   MI355_REQUIRE(dev, waves > 0 && waves % 4 == 0, "mfma_dense: waves (%u) must be a positive multiple of 4", waves);
   MI355_REQUIRE(dev, (((uintptr_t)A | (uintptr_t)B | (uintptr_t)out) & 15u) == 0, "mfma_dense: buffers must be 16-byte aligned");
   const bool one_set = (kind & MI355_MFMA_ONE_OPERAND_SET) != 0;
-  kind &= ~MI355_MFMA_ONE_OPERAND_SET;
+  uint32_t active = ((uint32_t)kind >> 16) & 0xffu;   // MI355_MATRIX_ON_XCDS: 0 = every XCD
+  if (active == 0u) active = 0xffu;
+  MI355_REQUIRE(dev, (active & 1u) != 0u, "mfma_dense: XCD 0 must be among the XCDs that take part (its first wave reads the clocks)");
+  if (kind & MI355_MATRIX_ON_HALF_THE_CUS) active |= 0x100u;
+  kind &= 0xff;
   switch (kind) {
-    case MI355_MFMA_F16_16x16x32:  return launch<F16_16x16x32>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
-    case MI355_MFMA_BF16_16x16x32: return launch<BF16_16x16x32>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
-    case MI355_MFMA_F16_32x32x16:  return launch<F16_32x32x16>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
-    case MI355_MFMA_BF16_32x32x16: return launch<BF16_32x32x16>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
-    case MI355_MFMA_I8_16x16x64:   return launch<I8_16x16x64>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
-    case MI355_MFMA_FP8_16x16x128: return launch<FP8_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
-    case MI355_MFMA_BF8_16x16x128: return launch<BF8_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
-    case MI355_MFMA_MXFP6_E2M3:    return launch<FP6_E2M3_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
-    case MI355_MFMA_MXFP6_E3M2:    return launch<FP6_E3M2_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
-    case MI355_MFMA_MXFP4_E2M1:    return launch<FP4_E2M1_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks);
+    case MI355_MFMA_F16_16x16x32:  return launch<F16_16x16x32>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
+    case MI355_MFMA_BF16_16x16x32: return launch<BF16_16x16x32>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
+    case MI355_MFMA_F16_32x32x16:  return launch<F16_32x32x16>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
+    case MI355_MFMA_BF16_32x32x16: return launch<BF16_32x32x16>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
+    case MI355_MFMA_I8_16x16x64:   return launch<I8_16x16x64>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
+    case MI355_MFMA_FP8_16x16x128: return launch<FP8_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
+    case MI355_MFMA_BF8_16x16x128: return launch<BF8_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
+    case MI355_MFMA_MXFP6_E2M3:    return launch<FP6_E2M3_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
+    case MI355_MFMA_MXFP6_E3M2:    return launch<FP6_E3M2_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
+    case MI355_MFMA_MXFP4_E2M1:    return launch<FP4_E2M1_16x16x128>(dev, one_set, A, B, scaleA, scaleB, out, waves, iters, clocks, active);
     default: return mi355_fail(dev, MI355_ERR_ARG, "mfma_dense: unknown kind %d", kind);
   }
 }

@@ -57,7 +57,9 @@ MI355_SPARSE_TRAIT(SP_I8, 128, 1, i32x4v, i32x8v, i32x4v, int32_t, "v_smfmac_i32
 template <typename Tr, bool ONE_SET>
 __global__ void __launch_bounds__(256)
 smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, const uint8_t *__restrict__ B,
-              typename Tr::Out *__restrict__ out, uint32_t iters, uint64_t *__restrict__ clocks) {
+              typename Tr::Out *__restrict__ out, uint32_t iters, uint64_t *__restrict__ clocks, uint32_t active) {
+  // diagnosis: only the workgroups of some XCDs (index mod 8) or of half the CUs of every XCD take part
+  if (!((active >> (blockIdx.x % 8u)) & 1u) || ((active & 0x100u) && (blockIdx.x / 8u) % 32u >= 16u)) return;
   const int lane = threadIdx.x % 64;
   const uint64_t wave = (uint64_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
   constexpr int K = Tr::K;
@@ -114,13 +116,13 @@ smfmac_kernel(const uint8_t *__restrict__ Ac, const uint8_t *__restrict__ meta, 
 
 template <typename Tr>
 int launch(mi355_dev *dev, bool one_set, const void *Ac, const uint8_t *meta, const void *B, void *out, uint32_t waves,
-           uint32_t iters, uint64_t *clocks) {
+           uint32_t iters, uint64_t *clocks, uint32_t active) {
   if (one_set)
     smfmac_kernel<Tr, true><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)Ac, meta, (const uint8_t *)B,
-                                                               (typename Tr::Out *)out, iters, clocks);
+                                                               (typename Tr::Out *)out, iters, clocks, active);
   else
     smfmac_kernel<Tr, false><<<waves / 4, 256, 0, dev->stream>>>((const uint8_t *)Ac, meta, (const uint8_t *)B,
-                                                                (typename Tr::Out *)out, iters, clocks);
+                                                                (typename Tr::Out *)out, iters, clocks, active);
   MI355_LAUNCH_CHECK(dev, "smfmac");
   return MI355_OK;
 }
@@ -134,13 +136,17 @@ extern "C" int mi355_smfmac(mi355_dev *dev, int kind, const void *Ac, const uint
   MI355_REQUIRE(dev, waves > 0 && waves % 4 == 0, "smfmac: waves (%u) must be a positive multiple of 4", waves);
   MI355_REQUIRE(dev, (((uintptr_t)Ac | (uintptr_t)B | (uintptr_t)out) & 15u) == 0, "smfmac: buffers must be 16-byte aligned");
   const bool one_set = (kind & MI355_MFMA_ONE_OPERAND_SET) != 0;
-  kind &= ~MI355_MFMA_ONE_OPERAND_SET;
+  uint32_t active = ((uint32_t)kind >> 16) & 0xffu;   // MI355_MATRIX_ON_XCDS: 0 = every XCD
+  if (active == 0u) active = 0xffu;
+  MI355_REQUIRE(dev, (active & 1u) != 0u, "smfmac: XCD 0 must be among the XCDs that take part (its first wave reads the clocks)");
+  if (kind & MI355_MATRIX_ON_HALF_THE_CUS) active |= 0x100u;
+  kind &= 0xff;
   switch (kind) {
-    case MI355_SMFMAC_F16_16x16x64:  return launch<SP_F16>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
-    case MI355_SMFMAC_BF16_16x16x64: return launch<SP_BF16>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
-    case MI355_SMFMAC_FP8_16x16x128: return launch<SP_FP8>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
-    case MI355_SMFMAC_BF8_16x16x128: return launch<SP_BF8>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
-    case MI355_SMFMAC_I8_16x16x128:  return launch<SP_I8>(dev, one_set, Ac, meta, B, out, waves, iters, clocks);
+    case MI355_SMFMAC_F16_16x16x64:  return launch<SP_F16>(dev, one_set, Ac, meta, B, out, waves, iters, clocks, active);
+    case MI355_SMFMAC_BF16_16x16x64: return launch<SP_BF16>(dev, one_set, Ac, meta, B, out, waves, iters, clocks, active);
+    case MI355_SMFMAC_FP8_16x16x128: return launch<SP_FP8>(dev, one_set, Ac, meta, B, out, waves, iters, clocks, active);
+    case MI355_SMFMAC_BF8_16x16x128: return launch<SP_BF8>(dev, one_set, Ac, meta, B, out, waves, iters, clocks, active);
+    case MI355_SMFMAC_I8_16x16x128:  return launch<SP_I8>(dev, one_set, Ac, meta, B, out, waves, iters, clocks, active);
     default: return mi355_fail(dev, MI355_ERR_ARG, "smfmac: unknown kind %d", kind);
   }
 }

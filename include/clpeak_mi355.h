@@ -208,6 +208,14 @@ int mi355_launch_roundtrip(mi355_dev *dev, uint32_t warmup, uint32_t launches, d
  * their accumulator chains (src/rocm/rocm_kernels/mfma_bf16.hip:16-30).  The slots of chains 1..3 in
  * the operand arrays are then not read; all four output tiles of a wave are equal. */
 #define MI355_MFMA_ONE_OPERAND_SET 0x100
+/* Diagnosis of what holds the clock (no counterpart in the reference; also for mi355_smfmac).  OR into `kind`:
+ * MI355_MATRIX_ON_XCDS(mask): only the workgroups that the part places on the XCDs of `mask` (workgroup index mod 8,
+ * bit 0 = XCD 0, which must be among them: its wave 0 fills `clocks`) do their work, the others return at once and
+ * leave their output tiles untouched.  MI355_MATRIX_ON_HALF_THE_CUS: of every XCD's workgroups only those of the
+ * first 16 of its 32 CUs (workgroup index / 8 mod 32 < 16).  Same total work per active wave either way, so the
+ * clock an active XCD holds with its neighbours idle, or with half of its own CUs idle, can be read off. */
+#define MI355_MATRIX_ON_XCDS(mask) (((mask) & 0xff) << 16)
+#define MI355_MATRIX_ON_HALF_THE_CUS 0x200
 int mi355_mfma_dense(mi355_dev *dev, int kind, const void *A, const void *B,
                      const uint8_t *scaleA, const uint8_t *scaleB,
                      void *out, uint32_t waves, uint32_t iters, uint64_t *clocks);

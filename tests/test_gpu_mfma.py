@@ -210,3 +210,42 @@ def test_smfmac_on_the_reference_operands(dev, kind, one_set):
         assert np.array_equal(got, ref), (s["name"], iters)
         for b in bufs + [out]:
             b.free()
+
+
+# --- the diagnosis flags: only some workgroups take part ---------------------------------------------------------
+@pytest.mark.parametrize("on_xcds,half_cus", [((0, 1, 2, 3), False), ((0,), False), (None, True), ((0, 5), True)])
+def test_matrix_kernels_on_a_subset_of_the_part(dev, on_xcds, half_cus):
+    """MI355_MATRIX_ON_XCDS / MI355_MATRIX_ON_HALF_THE_CUS: the workgroups that take part (workgroup index mod 8 among
+    the XCDs named; index / 8 mod 32 below 16) give exactly what the whole launch gives, bit for bit, the others leave
+    their output tiles untouched; a subset without XCD 0 is refused."""
+    waves, iters = 2048, 64
+    for sparse, kind in ((False, capi.MFMA_I8_16x16x64), (True, capi.SMFMAC_F16_16x16x64)):
+        if sparse:
+            Ac, meta, B = wl.sparse_inputs(kind, waves, SEED)
+            bufs = [dev.from_host(Ac), dev.from_host(meta), dev.from_host(B)]
+            launch = lambda o, **kw: dev.smfmac(kind, bufs[0], bufs[1], bufs[2], o, waves, iters, **kw)
+            per_wave, dtype = 4 * 256, np.uint32
+        else:
+            A, B, _, _ = wl.dense_inputs(kind, waves, SEED)
+            bufs = [dev.from_host(A), dev.from_host(B)]
+            launch = lambda o, **kw: dev.mfma_dense(kind, bufs[0], bufs[1], None, None, o, waves, iters, **kw)
+            per_wave, dtype = 4 * 256, np.uint32
+        whole, part = dev.alloc(waves * per_wave * 4), dev.alloc(waves * per_wave * 4)
+        dev.memset(whole, 0xa5); dev.memset(part, 0xa5)
+        launch(whole)
+        launch(part, on_xcds=on_xcds, half_cus=half_cus)
+        w = whole.download(dtype, waves * per_wave).reshape(waves // 4, 4 * per_wave)     # one row per workgroup
+        p = part.download(dtype, waves * per_wave).reshape(waves // 4, 4 * per_wave)
+        wg = np.arange(waves // 4)
+        takes_part = np.ones(waves // 4, dtype=bool)
+        if on_xcds is not None:
+            takes_part &= np.isin(wg % 8, on_xcds)
+        if half_cus:
+            takes_part &= (wg // 8) % 32 < 16
+        assert 0 < takes_part.sum() < waves // 4
+        assert np.array_equal(p[takes_part], w[takes_part])
+        assert np.all(p[~takes_part] == 0xa5a5a5a5)
+        with pytest.raises(capi.Mi355Error, match="XCD 0 must be among"):
+            launch(part, on_xcds=(1, 2))
+        for b in bufs + [whole, part]:
+            b.free()
