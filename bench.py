@@ -43,24 +43,21 @@ SEED = 0x5EEDC1BEA4D355
 def timed(dev, launch, min_us=300e3, warm_us=300e3, max_iters=10000, board=None):
     """Reference discipline (warm-up, probe, batch sized to a time budget), with the warm-up
     long enough for the clocks to settle under this kernel's load.  Returns us per launch.
-    board: a dict that receives what the board said during the timed batch (mean power, the share of the time the package
-    power limiter was active), where the machine lets an ordinary user read that."""
+    board: a dict that receives the board's mean power during the timed batch, where the machine lets an ordinary user read it."""
     launch(); dev.sync()
     probe = max(dev.time_launches(launch, 1), 1.0)
-    tel = _board_telemetry() if board is not None else None
-    snap0 = tel.snapshot() if tel else None      # the driver's table: from the start of the warm-up to the end of the batch
     dev.time_launches(launch, int(min(max(warm_us / probe, 2), max_iters)))
     n = int(min(max(min_us / probe, 1), max_iters))
     if board is None:
         return dev.time_launches(launch, n) / n, n
+    # (The driver's throttler residencies are not read here: its accumulators trail the load by some tenths of a second, so
+    # over a batch this short they tell of the row before.  --power-table reads them over seconds.)
+    tel = _board_telemetry()
     tel.start()                                  # the power reading: sampled during the timed batch, behind the warm-up
     us = dev.time_launches(launch, n) / n
     stats = tel.stop(skip_s=0.0)
-    between = tel.between(snap0, tel.snapshot())
     if stats.get("watts_mean") is not None:
         board["watts"] = stats["watts_mean"]
-    if between.get("ppt_residency") is not None:
-        board["ppt_residency"] = between["ppt_residency"]
     return us, n
 
 
@@ -1032,17 +1029,15 @@ def compact_line(full):
     # which launch the matrix fractions are: the four accumulator chains of a wave share one A and one B
     # fragment (the rows "distinct operands per chain" in the rows file are the other launch)
     line["mfma_operands"] = "one set per wave"
-    # for each matrix or GEMM row below its target: [clock held (MHz, read inside the kernel; null for the GEMMs, which do not
-    # read it), board power during the timed batch (W), share of the batch in which the package power limiter was active (%)]
+    # for each matrix or bf16 GEMM row below its target: [clock held (MHz, read inside the kernel; null for the GEMM, which does
+    # not read it), board power during the timed batch (W)]
     held = {}
     for key, test, metric in FRAC_KEYS:
         r = by_key.get((test, metric))
         target = TARGET_FRAC.get(key.split("_")[0]) if key.startswith(("mfma", "smfmac")) or key == "gemm_bf16_seeded" else None
         if r is not None and target and r.get("frac", 1.0) < target and ("sclk_mhz" in r or "watts" in r):
-            ppt = r.get("ppt_residency")
-            held[key] = [int(r["sclk_mhz"]) if "sclk_mhz" in r else None, int(round(r["watts"])) if "watts" in r else None,
-                         int(round(100 * ppt)) if ppt is not None else None]
-    line["below_target_mhz_w_pptpct"] = held
+            held[key] = [int(r["sclk_mhz"]) if "sclk_mhz" in r else None, int(round(r["watts"])) if "watts" in r else None]
+    line["below_target_mhz_w"] = held
     lat = by_key.get(("kernel_launch_latency", "roundtrip"))
     if lat is not None:
         line["launch_roundtrip_us"] = lat["value"]
