@@ -112,3 +112,40 @@ def test_headline_grid_is_the_parity_tested_one():
     assert "bwBlocksPerCU = 1;" in header
     gpu_test = open(os.path.join(ROOT, "tests", "test_gpu_basic.py")).read()
     assert "for blocks_per_cu in (1, 8):" in gpu_test
+
+
+def test_metrics_table_fields_are_read_where_the_driver_puts_them(tmp_path):
+    """bench.py reads the driver's metrics table (gpu_metrics, format 1.8) at fixed offsets: a table built here with known
+    values in those places must come back as those values, a table of another revision as None, and the difference of two
+    snapshots as residencies (share of the accumulation cycles) and mean power (energy counter over firmware time)."""
+    import struct
+
+    def table(rev, energy_units, acc, residencies, fw_ticks, clocks):
+        b = bytearray(3872)
+        struct.pack_into("<HBB", b, 0, 3872, 1, rev)
+        struct.pack_into("<Q", b, 24, energy_units)
+        struct.pack_into("<I", b, 40, acc)
+        struct.pack_into("<5I", b, 44, *residencies)
+        struct.pack_into("<Q", b, 288, fw_ticks)
+        struct.pack_into("<8H", b, 296, *clocks)
+        return bytes(b)
+
+    tel = bench._Telemetry.__new__(bench._Telemetry)
+    path = tmp_path / "gpu_metrics"
+    tel.metrics = str(path)
+    path.write_bytes(table(8, 1_000_000, 0xfffffff0, (0, 0xffffff00, 3, 4, 5), 10_000_000_000, range(1700, 1708)))
+    a = tel.snapshot()
+    assert a["acc"] == 0xfffffff0 and a["ppt"] == 0xffffff00 and a["prochot"] == 0 and a["hbm_thm"] == 5
+    assert a["gfxclk"] == list(range(1700, 1708)) and abs(a["fw_s"] - 100.0) < 1e-9 and abs(a["energy_j"] - 15.259) < 1e-6
+    # two seconds later: 2000 accumulation cycles (the 32-bit counters wrap), the package limiter active in 500 of them, 2800 J
+    units = 1_000_000 + int(round(2800.0 / 15.259e-6))
+    path.write_bytes(table(8, units, (0xfffffff0 + 2000) & 0xffffffff, (0, (0xffffff00 + 500) & 0xffffffff, 3, 4, 5),
+                           10_000_000_000 + 200_000_000, range(1800, 1808)))
+    d = bench._Telemetry.between(a, tel.snapshot())
+    assert d["ppt_residency"] == 0.25 and d["prochot_residency"] == 0.0 and d["socket_thm_residency"] == 0.0
+    assert abs(d["watts_energy_counter"] - 1400.0) < 0.2 and d["gfxclk_mhz_per_xcd"] == list(range(1800, 1808))
+    path.write_bytes(table(7, 1, 2, (3, 4, 5, 6, 7), 8, range(8)))
+    assert tel.snapshot() is None                      # another revision: other offsets, not guessed at
+    assert bench._Telemetry.between(a, None) == {}
+    tel.metrics = str(tmp_path / "absent")
+    assert tel.snapshot() is None
