@@ -107,6 +107,9 @@ def bench_rows(dev, quick, only):
         _gemm_rows(dev, capi, wl, add, budget, constant=False)
     if "vendor" in only:
         _vendor_rows(dev, capi, wl, add, budget)
+    if "gemm_small" in only:
+        progress("gemm_small rows")
+        _gemm_small_rows(dev, capi, wl, add, budget)
     if "gemm_const" in only:
         progress("gemm_const rows")
         _gemm_rows(dev, capi, wl, add, budget, constant=True)
@@ -284,15 +287,58 @@ def _gemm_rows(dev, capi, wl, add, budget, constant):
             b.free()
 
 
+def _gemm_small_rows(dev, capi, wl, add, budget):
+    """2048 cubed, 64 tiles of 256 x 256 on a part of 256 CUs: the 8- and 16-bit kinds on the tiling the library picks
+    there (128 x 128, one tile per CU) and on the 256 x 256 tiles it would otherwise run on.  Seeded operands."""
+    M = N = K = 2048
+    s43, s52 = 448.0, 57344.0
+    for test, metric, eb, ob, peak, unit in (("rocblas-fp", "fp16", 2, 2, "f16", "tflops"), ("rocblas-fp", "bf16", 2, 2, "bf16", "tflops"),
+                                             ("hipblaslt-fp8", "fp8_e4m3", 1, 2, "fp8", "tflops"), ("hipblaslt-fp8", "fp8_e5m2", 1, 2, "fp8", "tflops"),
+                                             ("rocblas-int", "int8", 1, 4, "int8", "tops")):
+        dA, dB, dC = dev.alloc(M * K * eb), dev.alloc(N * K * eb), dev.alloc(M * N * ob)
+        if metric == "fp16":
+            dev.fill_f16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_f16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            fn = lambda: dev.gemm_f16(dA, dB, dC, M, N, K)
+        elif metric == "bf16":
+            dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            fn = lambda: dev.gemm_bf16(dA, dB, dC, M, N, K)
+        elif metric == "fp8_e4m3":
+            dev.fill_fp8_e4m3(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, s43); dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, s43)
+            fn = lambda: dev.gemm_fp8_e4m3(dA, dB, dC, M, N, K, 1 / s43, 1 / s43)
+        elif metric == "fp8_e5m2":
+            dev.fill_fp8_e5m2(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1, s52); dev.fill_fp8_e4m3(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1, s43)
+            fn = lambda: dev.gemm_fp8_e5m2(dA, dB, dC, M, N, K, 1 / s52, 1 / s43)
+        else:
+            dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
+            fn = lambda: dev.gemm_i8(dA, dB, dC, M, N, K)
+        for tiling, name in ((capi.GEMM_TILING_128, "128x128 tiles"), (capi.GEMM_TILING_256, "256x256 tiles")):
+            dev.gemm_tiling(tiling)
+            us, _ = timed(dev, fn, **budget)
+            dev.gemm_tiling(capi.GEMM_TILING_AUTO)
+            add(test, f"{metric} on {name}", 2.0 * M * N * K / us / 1e6, unit, us, PEAK[peak], shape="2048x2048x2048")
+        for b in (dA, dB, dC):
+            b.free()
+
+
 def _vendor_rows(dev, capi, wl, add, budget):
     """The vendor library the reference's GEMM rows call (rocBLAS / hipBLASLt, reached here through torch.matmul,
     torch._scaled_mm and torch._int_mm), timed in this process on this board right beside this library's kernel of the
     same row, on operands of the same distribution (uniform [-1,1) rounded to the type; int8 uniform in [-8,7]) and on
     the reference's constant fill.  Not part of the default rows: it needs torch, whose first import takes a minute."""
-    import time
     import torch
-    M = N = K = 8192
+    g = torch.Generator(device="cuda")
+    g.manual_seed(SEED & 0x7fffffff)
+    # 8192 cubed: the rows' own shape.  2048 cubed: 64 tiles of 256 x 256 on a part of 256 CUs, the shape this library
+    # gives to its kernel on 128 x 128 tiles (timed on the 256 x 256 tiles as well).
+    for D in (8192, 2048):
+        _vendor_rows_of(dev, capi, wl, add, budget, torch, g, D)
+
+
+def _vendor_rows_of(dev, capi, wl, add, budget, torch, g, D):
+    import time
+    M = N = K = D
     flops = 2.0 * M * N * K
+    shape = f"{D}x{D}x{D}"
 
     def t_torch(fn):
         torch.cuda.synchronize()
@@ -301,7 +347,7 @@ def _vendor_rows(dev, capi, wl, add, budget):
             for _ in range(10):
                 fn()
             torch.cuda.synchronize()
-        reps = max(10, int(budget.get("min_us", 300e3) / 600.0))
+        reps = max(10, int(budget.get("min_us", 300e3) / (600.0 * (D / 8192.0) ** 3 + 10.0)))
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
@@ -310,8 +356,6 @@ def _vendor_rows(dev, capi, wl, add, budget):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / reps
 
-    g = torch.Generator(device="cuda")
-    g.manual_seed(SEED & 0x7fffffff)
     one = torch.ones((), device="cuda")
     cases = [("rocblas-fp", "bf16", torch.bfloat16, "bf16", "tflops", 0x3f), ("rocblas-fp", "fp16", torch.float16, "f16", "tflops", 0x3f),
              ("hipblaslt-fp8", "fp8_e4m3", torch.float8_e4m3fn, "fp8", "tflops", 0x38), ("rocblas-int", "int8", torch.int8, "int8", "tops", 0x3f)]
@@ -329,7 +373,7 @@ def _vendor_rows(dev, capi, wl, add, budget):
             if what.startswith("constant"):
                 A.view(torch.uint8).fill_(const_byte); B.view(torch.uint8).fill_(const_byte)
             us = t_torch(fn)
-            add(test, f"{metric} vendor library, {what}", flops / us / 1e6, unit, us, PEAK[peak], shape="8192x8192x8192")
+            add(test, f"{metric} vendor library, {what}", flops / us / 1e6, unit, us, PEAK[peak], shape=shape)
         del A, B
         torch.cuda.empty_cache()
         # this library's kernel of the same row, right behind it on the same board
@@ -347,11 +391,17 @@ def _vendor_rows(dev, capi, wl, add, budget):
         else:
             dev.fill_i8(dA, M * K, SEED, wl.STREAM_GEMM_A); dev.fill_i8(dB, N * K, SEED, wl.STREAM_GEMM_B)
             mine = lambda: dev.gemm_i8(dA, dB, dC, M, N, K)
+        small = 2 * (M // 256) * (N // 256) <= dev.props.num_cus     # the library's own choice of tiling at this shape
         for what in ("seeded operands", "constant operands"):
             if what.startswith("constant"):
                 dev.memset(dA, const_byte); dev.memset(dB, const_byte)
             us, _ = timed(dev, mine, **budget)
-            add(test, f"{metric} this library, {what}", flops / us / 1e6, unit, us, PEAK[peak], shape="8192x8192x8192")
+            add(test, f"{metric} this library, {what}", flops / us / 1e6, unit, us, PEAK[peak], shape=shape)
+            if small:
+                dev.gemm_tiling(capi.GEMM_TILING_256)
+                us, _ = timed(dev, mine, **budget)
+                dev.gemm_tiling(capi.GEMM_TILING_AUTO)
+                add(test, f"{metric} this library on 256x256 tiles, {what}", flops / us / 1e6, unit, us, PEAK[peak], shape=shape)
         for b in (dA, dB, dC):
             b.free()
 
@@ -453,8 +503,6 @@ def _vendor_child():
     because torch brings a HIP runtime that has to be the one to initialise the device in its process."""
     import torch
     M = N = K = 8192
-    g = torch.Generator(device="cuda")
-    g.manual_seed(SEED & 0x7fffffff)
     one = torch.ones((), device="cuda")
     out = {}
 
@@ -863,7 +911,8 @@ def main():
                          "shader clock are sampled from sysfs every 10 ms; one JSON line per workload")
     ap.add_argument("--only", default="mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer",
                     help="comma list of extra row groups to run: mad,latency,mfma,smfmac,matrix_distinct,matrix_zero,matrix_ref,gemm,gemm_const,lds,transfer; "
-                         "and, not among the defaults, vendor: the vendor library's GEMM beside this library's (needs torch)")
+                         "and, not among the defaults, vendor: the vendor library's GEMM beside this library's (needs torch); "
+                         "gemm_small: 2048 cubed on the 128x128 and on the 256x256 tiles")
     ap.add_argument("--no-vendor", action="store_true", help="skip the vendor library's bf16 / fp8 / FP4 GEMM beside this library's (a child process that imports torch)")
     ap.add_argument("--vendor-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()

@@ -24,7 +24,7 @@ SYMBOLS = [
     "mi355_fill_f16", "mi355_fill_fp8_e5m2", "mi355_fill_i8", "mi355_gemm_f16", "mi355_gemm_i8", "mi355_gemm_fp8_e5m2",
     "mi355_gemm_f32", "mi355_gemm_f64", "mi355_fill_f64",
     "mi355_gemm_mxfp4", "mi355_gemm_mxfp4_static", "mi355_fill_bytes",
-    "mi355_gemm_mxfp4_prepare_scales", "mi355_gemm_mxfp4_prepared", "mi355_scratch_bytes",
+    "mi355_gemm_mxfp4_prepare_scales", "mi355_gemm_mxfp4_prepared", "mi355_scratch_bytes", "mi355_gemm_tiling",
 ]
 
 OK, ERR_ARG, ERR_HIP, ERR_NODEV, ERR_ARCH, ERR_OOM = 0, -1, -2, -3, -4, -5
@@ -34,6 +34,7 @@ MAD_F32, MAD_F16, MAD_F64, MAD_MP, MAD_BF16, MAD_I32, MAD_I8DP = range(7)
 (MFMA_F16_16x16x32, MFMA_BF16_16x16x32, MFMA_F16_32x32x16, MFMA_BF16_32x32x16, MFMA_I8_16x16x64,
  MFMA_FP8_16x16x128, MFMA_BF8_16x16x128, MFMA_MXFP6_E2M3, MFMA_MXFP6_E3M2, MFMA_MXFP4_E2M1) = range(10)
 SMFMAC_F16_16x16x64, SMFMAC_BF16_16x16x64, SMFMAC_FP8_16x16x128, SMFMAC_BF8_16x16x128, SMFMAC_I8_16x16x128 = range(5)
+GEMM_TILING_AUTO, GEMM_TILING_256, GEMM_TILING_128 = 0, 1, 2
 MATRIX_ON_HALF_THE_CUS = 0x200   # diagnosis: only the workgroups of the first 16 CUs of every XCD take part
 MFMA_ONE_OPERAND_SET = 0x100   # OR into an MFMA / SMFMAC kind: every chain of a wave takes chain 0's operands
 
@@ -93,6 +94,7 @@ def load_library(path=LIB_PATH):
     lib.mi355_fill_fp8_e5m2.argtypes = [vp, vp, u64, u64, u32, i32, C.c_float]
     lib.mi355_fill_i8.argtypes = [vp, vp, u64, u64, u32]
     lib.mi355_gemm_f16.argtypes = [vp, vp, vp, vp, u32, u32, u32]
+    lib.mi355_gemm_tiling.argtypes = [vp, C.c_int]
     lib.mi355_gemm_i8.argtypes = [vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_gemm_f32.argtypes = [vp, vp, vp, vp, u32, u32, u32]
     lib.mi355_gemm_f64.argtypes = [vp, vp, vp, vp, u32, u32, u32]
@@ -269,6 +271,10 @@ class Device:
     def mfma_raw(self, sparse, kind, a, b, c, aux0, aux1, sel0, sel1, d):
         self._check(self.lib.mi355_mfma_raw(self.h, int(sparse), kind, a.ptr, b.ptr, c.ptr, aux0.ptr, aux1.ptr,
                                             sel0, sel1, d.ptr))
+
+    def gemm_tiling(self, tiling):
+        """GEMM_TILING_AUTO / _256 / _128 for the 8- and 16-bit GEMM calls of this handle."""
+        self._check(self.lib.mi355_gemm_tiling(self.h, tiling))
 
     def gemm_bf16(self, A, B, Cbuf, M, N, K):
         self._check(self.lib.mi355_gemm_bf16(self.h, A.ptr, B.ptr, Cbuf.ptr, M, N, K))

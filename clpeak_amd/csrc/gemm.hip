@@ -190,14 +190,29 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
   return MI355_OK;
 }
 
-// The 4-, 8- and 16-bit kinds run on the four-wave kernel of gemm_quad.hip.
+// The 8- and 16-bit kinds run on the four-wave kernel of gemm_quad.hip (256x256 tiles, one persistent workgroup per
+// CU), or, when that tiling has too few tiles for the part, on the 128x128 tiles of gemm_small.hip: four times the
+// workgroups at half the arithmetic per byte of operand.  "Too few" is at most half a tile per CU: from there up the
+// big tiles keep at least every second CU busy at twice the efficiency.
 int launch_quad(mi355_dev *dev, int op, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N, uint32_t K,
                 uint32_t elem, float scale) {
   if (int rc = check_shapes(dev, A, B, C, M, N, K, elem)) return rc;
+  const uint64_t tiles = (uint64_t)(M / kTile) * (N / kTile);
+  const bool small = dev->gemm_tiling == MI355_GEMM_TILING_128 ||
+                     (dev->gemm_tiling == MI355_GEMM_TILING_AUTO && 2u * tiles <= (uint64_t)(dev->props.num_cus > 0 ? dev->props.num_cus : 1));
+  if (small) return mi355_launch_gemm_small(dev, op, what, A, B, C, M, N, K * elem, scale);
   return mi355_launch_gemm_quad(dev, op, what, A, B, C, M, N, K * elem, scale);
 }
 
 }  // namespace
+
+extern "C" int mi355_gemm_tiling(mi355_dev *dev, int tiling) {
+  if (!dev) return mi355_fail(nullptr, MI355_ERR_ARG, "null device handle");
+  MI355_REQUIRE(dev, tiling == MI355_GEMM_TILING_AUTO || tiling == MI355_GEMM_TILING_256 || tiling == MI355_GEMM_TILING_128,
+                "gemm_tiling: unknown tiling %d", tiling);
+  dev->gemm_tiling = tiling;
+  return MI355_OK;
+}
 
 extern "C" int mi355_gemm_bf16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C, uint32_t M,
                                uint32_t N, uint32_t K) {

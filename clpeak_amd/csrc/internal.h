@@ -20,6 +20,8 @@ struct mi355_dev {
   void        *mx_static_scratch = nullptr;
   // GEMM kernels that have been allowed the whole LDS of a CU on this device (one bit per kernel)
   uint32_t     full_lds_allowed = 0;
+  // which tiling the 4-, 8- and 16-bit GEMM entry points take (MI355_GEMM_TILING_*; set by mi355_gemm_tiling)
+  int          gemm_tiling = 0;
 };
 
 // Error text for failures that have no handle to hang on (open, device_count).

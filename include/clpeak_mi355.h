@@ -275,6 +275,17 @@ int mi355_gemm_i8(mi355_dev *dev, const int8_t *A, const int8_t *B, int32_t *C,
                   uint32_t M, uint32_t N, uint32_t K);
 int mi355_gemm_fp8_e5m2(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint16_t *C,
                         uint32_t M, uint32_t N, uint32_t K, float scale_a, float scale_b);
+/* Which tiling the five calls above take (no counterpart in the reference: the vendor libraries behind its tests
+ * pick their own kernel per shape).  256: every workgroup owns a 256x256 tile of C and a whole CU, the schedule for
+ * the sizes the reference's tests pick on a part of this many CUs (pickGemmDim, src/rocm/hipblaslt_gemm.cpp:41-55,
+ * and pickRocblasGemmDim, src/rocm/rocblas.cpp:71: thousands of rows).  128: one
+ * workgroup per 128x128 tile, four times as many workgroups at half the arithmetic per operand byte.  AUTO (the
+ * default of a new handle): 128 when the product has at most half a 256x256 tile per CU (2048 cubed: 64 tiles on
+ * 256 CUs), 256 otherwise.  Both tilings take the same shapes; their results agree within rounding (int8 exactly). */
+#define MI355_GEMM_TILING_AUTO 0
+#define MI355_GEMM_TILING_256  1
+#define MI355_GEMM_TILING_128  2
+int mi355_gemm_tiling(mi355_dev *dev, int tiling);
 /*   "fp32" of runRocblas (src/rocm/rocblas.cpp:246-254, rocblas_sgemm): fp32 operands, accumulation
  *          and output, on the fp32 matrix instruction; K a multiple of 32;
  *   "fp64" of runRocblas (src/rocm/rocblas.cpp:256-263, rocblas_dgemm): all fp64, on the fp64 matrix

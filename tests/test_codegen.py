@@ -286,3 +286,91 @@ def test_scalar_half_row_runs_on_the_scalar_half_fma(tmp_path):
     assert body.count("v_fma_f16") == 16 * 8 + 16 and "v_pk_fma_f16" not in body, body.count("v_fma_f16")
     body = kernel_body(asm, packed)
     assert "v_pk_fma_f16" in body and not re.search(r"\bv_fma_f16\b", body)
+
+
+def _registers(operand):
+    """Vector registers an operand text names: v7 -> {7}, v[4:7] -> {4..7}."""
+    out = set()
+    for lo, hi in re.findall(r"\bv\[(\d+):(\d+)\]", operand):
+        out |= set(range(int(lo), int(hi) + 1))
+    out |= {int(x) for x in re.findall(r"\bv(\d+)\b", operand)}
+    return out
+
+
+def registers_touched_while_a_read_is_in_flight(body):
+    """Instructions that name a destination register of an LDS read between the read and the next wait for all LDS
+    reads, and branches or labels in that stretch (where paths join, register copies appear).  Instruction text in
+    program order; the body must wait with lgkmcnt(0), as the 128x128 GEMM kernel does."""
+    pending, found = set(), []
+    for line in body.splitlines():
+        text = line.split(";")[0].strip()
+        if not text or text.startswith("."):
+            if pending and re.match(r"\.LBB\d+_\d+:", text):
+                found.append(("label", text))
+            continue
+        op, _, rest = text.partition(" ")
+        if op == "s_waitcnt" and "lgkmcnt(0)" in rest:
+            pending = set()
+        elif op.startswith("ds_read"):
+            dst = rest.split(",")[0]
+            if _registers(rest) & pending:
+                found.append(("reuse", text))
+            pending |= _registers(dst)
+        elif pending and (op.startswith("s_cbranch") or op == "s_branch"):
+            found.append(("branch", text))
+        elif pending and _registers(rest) & pending:
+            found.append(("touch", text))
+    if pending:
+        found.append(("end", sorted(pending)[:4]))
+    return found
+
+
+def test_the_checker_of_reads_in_flight_sees_what_it_is_for():
+    good = "ds_read_b128 v[4:7], v1 offset:0\n v_mfma_f32_16x16x32_bf16 v[8:11], v[12:15], v[16:19], v[8:11]\n s_waitcnt lgkmcnt(0)\n v_add_u32 v4, v4, v5\n"
+    assert registers_touched_while_a_read_is_in_flight(good) == []
+    early = "ds_read_b128 v[4:7], v1 offset:0\n v_lshlrev_b32_e32 v5, 2, v9\n s_waitcnt lgkmcnt(0)\n"
+    assert [k for k, _ in registers_touched_while_a_read_is_in_flight(early)] == ["touch"]
+    copy = "ds_read_b128 v[4:7], v1 offset:0\n v_mov_b64_e32 v[20:21], v[6:7]\n s_waitcnt lgkmcnt(0)\n"
+    assert [k for k, _ in registers_touched_while_a_read_is_in_flight(copy)] == ["touch"]
+    join = "ds_read_b128 v[4:7], v1 offset:0\n s_cbranch_scc1 .LBB0_3\n.LBB0_3:\n s_waitcnt lgkmcnt(0)\n"
+    assert [k for k, _ in registers_touched_while_a_read_is_in_flight(join)] == ["branch", "label"]
+    never = "ds_read_b128 v[4:7], v1 offset:0\n s_endpgm\n"
+    assert [k for k, _ in registers_touched_while_a_read_is_in_flight(never)] == ["end"]
+
+
+SMALL_KINDS = {"ILi0E": ("v_mfma_f32_16x16x128_f8f6f4", 16), "ILi1E": ("v_mfma_f32_16x16x128_f8f6f4", 16),
+               "ILi2E": ("v_mfma_f32_16x16x32_bf16", 32), "ILi3E": ("v_mfma_f32_16x16x32_f16", 32), "ILi4E": ("v_mfma_i32_16x16x64_i8", 32)}
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+def test_gemm_small_kernels(tmp_path):
+    """The kernel on 128x128 tiles.  Nothing spills.  No register that an LDS read is still writing is named before
+    the wait for it, and no branch lies in between (a last step that read fragments nobody takes once had their
+    registers reused for the addresses of the stores).  The accumulators are the 64 accumulation registers the source
+    names, touched by nothing but its matrix instructions, its zeroing and, behind the wait states that follow the last
+    matrix instruction, its reads (held as values of the compiler's they were once copied, where two paths joined,
+    right behind the matrix instructions that wrote them).  The loop holds two steps, the code behind it one more with
+    reads and loads and two without (an even and an odd count of steps)."""
+    asm = device_asm(tmp_path, "gemm_small.hip")
+    meta = kernel_metadata(asm)
+    for tag, (insn, per_step) in SMALL_KINDS.items():
+        name = next(k for k in meta if "gemm_small_kernel" + tag in k)
+        m = meta[name]
+        assert m["vgpr_spill_count"] == 0 and m.get("sgpr_spill_count", 0) == 0 and m["private_segment_fixed_size"] == 0, (name, m)
+        assert m["agpr_count"] == 64 and m["vgpr_count"] <= 256 and m.get("group_segment_fixed_size", 0) == 0, (name, m)
+        body = kernel_body(asm, name)
+        assert registers_touched_while_a_read_is_in_flight(body) == [], name
+        lines = [l.split(";")[0].strip() for l in body.splitlines()]
+        lines = [l for l in lines if l and not l.startswith(".")]
+        on_acc = [(n, l) for n, l in enumerate(lines) if re.search(r"\ba\[?\d+", l)]
+        mfma = [n for n, l in on_acc if l.startswith(insn + " ")]
+        zero = [n for n, l in on_acc if re.fullmatch(r"v_accvgpr_write_b32 a\[?\d+\]?, 0", l)]
+        take = [n for n, l in on_acc if re.fullmatch(r"v_accvgpr_read_b32 v\d+, a\[?\d+\]?", l)]
+        assert len(mfma) + len(zero) + len(take) == len(on_acc), [l for _, l in on_acc if not l.startswith(insn)][:3]
+        assert len(mfma) == 5 * per_step and len(zero) == 64 and len(take) == 64, (name, len(mfma), len(zero), len(take))
+        assert max(zero) < min(mfma) and max(mfma) < min(take), name
+        assert all(re.search(r"a\[(\d+):(\d+)\], v\[\d+:\d+\], v\[\d+:\d+\], a\[\1:\2\]", lines[n]) for n in mfma), name
+        assert [l for l in lines[max(mfma) + 1:min(take)] if l.startswith("s_nop 15")] == ["s_nop 15"] * 2, name
+        assert sum(l.startswith("ds_read_b128 ") for l in lines) == 16 * 4, name          # prologue, two steps, one tail step
+        assert sum(l.startswith("global_load_lds_dwordx4 ") for l in lines) == 8 * (4 + 3), name
+        assert sum(l == "s_barrier" for l in lines) == 4, name

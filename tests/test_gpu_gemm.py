@@ -15,6 +15,15 @@ SEED = wl.DEFAULT_SEED
 FP8_SCALE = 448.0   # per-tensor scale: uniform [-1,1) * 448 fills the e4m3 range
 
 
+@pytest.fixture(autouse=True, scope="module")
+def _on_the_256_tiles(dev):
+    """This file is about the kernels on 256x256 tiles, also at shapes the library would give to the 128x128 kernel
+    (test_gpu_gemm_small.py covers that one and the choice between the two)."""
+    dev.gemm_tiling(capi.GEMM_TILING_256)
+    yield
+    dev.gemm_tiling(capi.GEMM_TILING_AUTO)
+
+
 def _operands(dev, fp8, M, N, K):
     eb = 1 if fp8 else 2
     dA, dB = dev.alloc(M * K * eb), dev.alloc(N * K * eb)
