@@ -19,11 +19,11 @@
 // slab the loads wrap around to the start of the rows (fetches nobody reads, so that every step but the last is the
 // same code); they are waited for before the wave ends.
 //
-// What bounds it: a 128x128 tile needs twice the operand bytes per operation of a 256x256 tile.  A step brings
-// 32 KiB into the CU against 512 cycles of matrix instructions, 64 bytes per cycle, which is all that the vector
-// memory path of a CU delivers; the LDS moves 96 KiB in the same time (64 KiB of fragment reads, 32 KiB written by the
-// loads).  So the loads, not the matrix pipe, set the pace of a step (measured: about 900 cycles), and waves spend a
-// third of their time waiting for them.
+// What bounds it: the LDS.  A 128x128 tile moves twice the LDS bytes per operation of a 256x256 tile: per step 64 KiB
+// of fragment reads and 32 KiB written by the loads, 96 KiB at the 128 bytes per cycle the LDS of a CU moves, 768
+// cycles against the 512 of the matrix instructions.  Measured: 0.34 us per step (0.32 us is 768 cycles at 2.4 GHz) with
+// up to half the CUs busy; 0.40-0.43 us on the whole part under random operands, where the clock is lower.  Taking
+// the loads out leaves 512 cycles; four slabs in flight instead of three change nothing.
 //
 // The sums run over K in order, one step after the other: results differ from the 256x256 kernel's only in rounding
 // (that kernel starts its walk over K at a different place on every XCD); the int8 kind is exact either way.
