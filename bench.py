@@ -503,6 +503,8 @@ def _vendor_child():
     because torch brings a HIP runtime that has to be the one to initialise the device in its process."""
     import torch
     M = N = K = 8192
+    g = torch.Generator(device="cuda")
+    g.manual_seed(SEED & 0x7fffffff)
     one = torch.ones((), device="cuda")
     out = {}
 
@@ -552,6 +554,8 @@ def vendor_beside(timeout_s=150):
     try:
         r = subprocess.run([sys.executable, os.path.abspath(__file__), "--vendor-child"], capture_output=True, text=True, timeout=timeout_s)
         got = json.loads(r.stdout.strip().splitlines()[-1]) if r.returncode == 0 and r.stdout.strip() else {}
+        if not got:
+            sys.stderr.write(f"bench.py: vendor library leg gave nothing (exit status {r.returncode}): {r.stderr.strip()[-300:]}\n")
     except (subprocess.TimeoutExpired, OSError, ValueError) as e:
         sys.stderr.write(f"bench.py: vendor library leg skipped: {e!r}\n")
         return []

@@ -149,3 +149,28 @@ def test_metrics_table_fields_are_read_where_the_driver_puts_them(tmp_path):
     assert bench._Telemetry.between(a, None) == {}
     tel.metrics = str(tmp_path / "absent")
     assert tel.snapshot() is None
+
+
+def test_every_name_the_gpu_only_code_uses_exists():
+    """Most of bench.py, the C-ABI mirror and the smoke test run only on a GPU box; a name that a function reads and
+    nothing defines (a line lost in an edit) would show there at the earliest, in a child process perhaps not at all.
+    Every name a function takes from the module must be bound at module level or be a builtin."""
+    import builtins
+    import symtable
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for rel in ("bench.py", "__graft_entry__.py", os.path.join("clpeak_amd", "capi.py"), os.path.join("clpeak_amd", "workloads.py"),
+                os.path.join("tests", "vendor_parity_child.py")):
+        path = os.path.join(root, rel)
+        top = symtable.symtable(open(path).read(), path, "exec")
+        bound = {s.get_name() for s in top.get_symbols() if s.is_assigned() or s.is_imported() or s.is_namespace()} | {"__file__", "__name__"}
+        missing = []
+
+        def walk(table):
+            for child in table.get_children():
+                for s in child.get_symbols():
+                    if s.is_referenced() and s.is_global() and not s.is_assigned() and s.get_name() not in bound \
+                            and not hasattr(builtins, s.get_name()):
+                        missing.append((child.get_name(), s.get_name()))
+                walk(child)
+        walk(top)
+        assert missing == [], (rel, missing)
