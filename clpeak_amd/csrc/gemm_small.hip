@@ -4,9 +4,8 @@
 // tiles (2048^3 has 64) then runs on a fraction of the CUs.  This kernel is the small sibling: one workgroup of four
 // waves per 128x128 tile (a wave owns 64x64 = 4x4 tiles of 16x16, in 64 accumulation registers), K walked in steps of
 // one 128-byte row segment, a slab of 128 rows x 128 B = 16 KiB per operand and step, global memory straight into
-// LDS with a row swizzle: the 16-byte chunk c of row r lies at position c ^ ((r >> 1) & 7) of the row, so that the 16
-// rows of which a fragment read takes one chunk each (8 positions, times the two halves of the banks that even and odd
-// rows fall into) cover the 64 banks once.
+// LDS with the row swizzle of the other GEMM kernels (the 16-byte chunk c of row r lies at position c ^ (r & 7) of the
+// row: fragment reads without bank conflicts).
 //
 // A step is 32 matrix instructions per wave (16 for fp8), 512 cycles of the matrix pipe, a fifth of a microsecond: far
 // less than a load takes to arrive.  So the LDS of the CU is a ring of five 32 KiB slots (A and B slab of a step side
@@ -55,7 +54,7 @@ struct SmallFrags {
 struct SmallWalk {
   uint32_t a0, a1, b0, b1;   // LDS addresses of this lane's first A / B fragment in the slab to read, K halves lo / hi
   uint32_t dst;              // LDS destination of the wave's first rows in the slot to fill
-  uint32_t voff[2], row8;    // this lane's offset within an even / odd group of 8 rows; bytes between rows r and r + 8
+  uint32_t voff, row8;       // this lane's offset within a group of 8 rows; bytes between rows r and r + 8
   uint64_t ga, gb;           // the wave's A / B rows in the slab to fetch
 };
 
@@ -122,8 +121,8 @@ __device__ __forceinline__ void small_read(SmallFrags &f, const SmallWalk &w) {
 // Load number Q of 8 of a slab: 8 rows of A (Q < 4) or of B into the slot being filled.
 template <int Q>
 __device__ __forceinline__ void small_load(const SmallWalk &w) {
-  if constexpr (Q < 4) MI355_LOAD_LDS(w.voff[Q % 2], w.ga + (uint64_t)Q * w.row8, w.dst + Q * 1024u);
-  else MI355_LOAD_LDS(w.voff[Q % 2], w.gb + (uint64_t)(Q - 4) * w.row8, w.dst + kSmallSlab + (Q - 4) * 1024u);
+  if constexpr (Q < 4) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)Q * w.row8, w.dst + Q * 1024u);
+  else MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(Q - 4) * w.row8, w.dst + kSmallSlab + (Q - 4) * 1024u);
 }
 
 // The reads of a fragment set have arrived.  The registers ride along so that nothing that uses them can be placed
@@ -208,15 +207,11 @@ gemm_small_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, 
   auto after = [](uint32_t slot_off) { return slot_off + kSmallSlot == kRing ? 0u : slot_off + kSmallSlot; };
 
   // global -> LDS: wave w fills rows [32w, 32w+32) of the A slab and of the B slab, 8 rows per instruction; lane i is
-  // position i%8 of row i/8 of its 8 rows, which holds the logical chunk that the swizzle puts there
+  // position i%8 of row i/8, which holds logical chunk (i%8) ^ (i/8)
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const uint32_t dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 32u * (uint32_t)kRowBytes);
   SmallWalk w;
-  {
-    const uint32_t t = lane / 8u, pos = lane % 8u;   // row t of a group of 8 rows; rows 8g + t of a slab, g even / odd
-    w.voff[0] = t * k_bytes + (pos ^ (t >> 1)) * 16u;
-    w.voff[1] = t * k_bytes + (pos ^ (4u + (t >> 1))) * 16u;
-  }
+  w.voff = (lane / 8u) * k_bytes + ((lane % 8u) ^ (lane / 8u)) * 16u;
   w.row8 = 8u * k_bytes;
   w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kSmallTile + wave * 32u) * k_bytes);
   w.gb = (uint64_t)(uintptr_t)(B + ((size_t)tn * kSmallTile + wave * 32u) * k_bytes);
@@ -228,8 +223,8 @@ gemm_small_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, 
     fill = after(fill);
   };
   // LDS -> fragments: row lane%16 of the wave's part, chunk lane/16 (+4 for the second K half: bit 6 of the address),
-  // swizzled with bits 1..3 of the row = of lane % 16
-  const uint32_t swz0 = ((lane / 16u) ^ ((lane % 16u) >> 1)) << 4;
+  // swizzled with row & 7 = lane & 7
+  const uint32_t swz0 = ((lane / 16u) ^ (lane & 7u)) << 4;
   const uint32_t lane_a = lds_base + (wm * 64u + lane % 16u) * kRowBytes + swz0;
   const uint32_t lane_b = lds_base + kSmallSlab + (wn * 64u + lane % 16u) * kRowBytes + swz0;
   auto place = [&]() {
