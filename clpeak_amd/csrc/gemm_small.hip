@@ -18,11 +18,15 @@
 // slab the loads wrap around to the start of the rows (fetches nobody reads, so that every step but the last is the
 // same code); they are waited for before the wave ends.
 //
-// What bounds it: the LDS.  A 128x128 tile moves twice the LDS bytes per operation of a 256x256 tile: per step 64 KiB
-// of fragment reads and 32 KiB written by the loads, 96 KiB at the 128 bytes per cycle the LDS of a CU moves, 768
-// cycles against the 512 of the matrix instructions.  Measured: 0.34 us per step (0.32 us is 768 cycles at 2.4 GHz) with
-// up to half the CUs busy; 0.40-0.43 us on the whole part under random operands, where the clock is lower.  Taking
-// the loads out leaves 512 cycles; four slabs in flight instead of three change nothing.
+// What bounds it: the issue slots of the wave.  With one wave per SIMD every instruction of a step is issued by the
+// wave whose matrix instructions it sits between, about one per four cycles: beside the 32 matrix instructions a step
+// has 16 reads, 8 loads with their M0 writes and some scalar bookkeeping, and a direct-to-LDS load holds the issue
+// port longer than other instructions.  Measured on constant operands, per step: 0.29-0.30 us (0.21 us is the 512
+// cycles of the matrix instructions at 2.4 GHz); with the loads taken out 0.24, with the reads taken out 0.29.  The
+// same on 4 and on 128 CUs and for operands of 0.5 MiB (L2) and of 128 MiB (HBM): not a matter of where the data comes
+// from, and four slabs in flight instead of three change nothing.  On the whole part under random operands a step
+// takes 0.40 us (the clock is lower there, and waves wait more).  (An earlier form of the loads - M0 written, a wait state and the address
+// arithmetic in front of every load, all eight behind matrix instructions of the first half - took 0.34 us.)
 //
 // The sums run over K in order, one step after the other: results differ from the 256x256 kernel's only in rounding
 // (that kernel starts its walk over K at a different place on every XCD); the int8 kind is exact either way.
@@ -54,7 +58,7 @@ struct SmallFrags {
 struct SmallWalk {
   uint32_t a0, a1, b0, b1;   // LDS addresses of this lane's first A / B fragment in the slab to read, K halves lo / hi
   uint32_t dst;              // LDS destination of the wave's first rows in the slot to fill
-  uint32_t voff, row8;       // this lane's offset within a group of 8 rows; bytes between rows r and r + 8
+  uint32_t voff[4];          // this lane's byte offset from ga / gb in each of the wave's four groups of 8 rows
   uint64_t ga, gb;           // the wave's A / B rows in the slab to fetch
 };
 
@@ -88,21 +92,28 @@ __device__ __forceinline__ i32x4v small_take_tile() {
 // wave's 4x4 tiles is instructions 8i .. 8i+7, its four first halves and then its four second halves, so that an
 // instruction never waits for the one just before it.  fp8 takes 16, one K = 128 instruction on both halves (the A
 // fragment is the second source of the transposed product: format field blgp for an e5m2 A).
-template <int OP, int S>
-__device__ __forceinline__ void small_mfma(const SmallFrags &f) {
-#define S_MFMA(insn, fmt, T, b, a) asm volatile(insn " a[%2:%3], %0, %1, a[%2:%3]" fmt :: "v"(b), "v"(a), "n"(4 * (T)), "n"(4 * (T) + 3))
+// Q >= 0: load number Q of the slab to fetch rides along (8 rows of A for Q < 4, of B otherwise, into the slot being
+// filled): M0, which holds the LDS destination, is written in front of the matrix instruction, which is the wait state
+// M0 needs before a load reads it, and the load is issued behind it; three instructions in all.
+template <int OP, int S, int Q = -1>
+__device__ __forceinline__ void small_mfma(const SmallFrags &f, const SmallWalk &w) {
+#define S_MFMA(insn, fmt, T, b, a)                                                                                              \
+  if constexpr (Q < 0) asm volatile(insn " a[%2:%3], %0, %1, a[%2:%3]" fmt :: "v"(b), "v"(a), "n"(4 * (T)), "n"(4 * (T) + 3));    \
+  else asm volatile("s_add_u32 m0, %4, %5\n " insn " a[%2:%3], %0, %1, a[%2:%3]" fmt "\n global_load_lds_dwordx4 %6, %7"         \
+                    :: "v"(b), "v"(a), "n"(4 * (T)), "n"(4 * (T) + 3), "s"(w.dst), "n"(Q < 4 ? Q * 1024 : (int)kSmallSlab + (Q - 4) * 1024), \
+                       "v"(w.voff[Q < 0 ? 0 : Q % 4]), "s"(Q < 4 ? w.ga : w.gb) : "memory", "m0", "scc")
   if constexpr (small_is_fp8(OP)) {
     constexpr int i = S / 4, j = S % 4;
     const i32x8v a8 = __builtin_shufflevector(f.a_lo[i], f.a_hi[i], 0, 1, 2, 3, 4, 5, 6, 7);
     const i32x8v b8 = __builtin_shufflevector(f.b_lo[j], f.b_hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
-    if constexpr (OP == kQuadE5m2) S_MFMA("v_mfma_f32_16x16x128_f8f6f4", " blgp:1", 4 * i + j, b8, a8);
-    else S_MFMA("v_mfma_f32_16x16x128_f8f6f4", "", 4 * i + j, b8, a8);
+    if constexpr (OP == kQuadE5m2) { S_MFMA("v_mfma_f32_16x16x128_f8f6f4", " blgp:1", 4 * i + j, b8, a8); }
+    else { S_MFMA("v_mfma_f32_16x16x128_f8f6f4", "", 4 * i + j, b8, a8); }
   } else {
     constexpr int i = S / 8, hi = (S % 8) / 4, j = S % 4;
     const i32x4v &a = hi ? f.a_hi[i] : f.a_lo[i], &b = hi ? f.b_hi[j] : f.b_lo[j];
-    if constexpr (OP == kQuadBf16) S_MFMA("v_mfma_f32_16x16x32_bf16", "", 4 * i + j, b, a);
-    else if constexpr (OP == kQuadF16) S_MFMA("v_mfma_f32_16x16x32_f16", "", 4 * i + j, b, a);
-    else S_MFMA("v_mfma_i32_16x16x64_i8", "", 4 * i + j, b, a);
+    if constexpr (OP == kQuadBf16) { S_MFMA("v_mfma_f32_16x16x32_bf16", "", 4 * i + j, b, a); }
+    else if constexpr (OP == kQuadF16) { S_MFMA("v_mfma_f32_16x16x32_f16", "", 4 * i + j, b, a); }
+    else { S_MFMA("v_mfma_i32_16x16x64_i8", "", 4 * i + j, b, a); }
   }
 #undef S_MFMA
 }
@@ -118,11 +129,11 @@ __device__ __forceinline__ void small_read(SmallFrags &f, const SmallWalk &w) {
   }
 }
 
-// Load number Q of 8 of a slab: 8 rows of A (Q < 4) or of B into the slot being filled.
+// Load number Q of 8 of a slab on its own (filling the ring before the first step).
 template <int Q>
 __device__ __forceinline__ void small_load(const SmallWalk &w) {
-  if constexpr (Q < 4) MI355_LOAD_LDS(w.voff, w.ga + (uint64_t)Q * w.row8, w.dst + Q * 1024u);
-  else MI355_LOAD_LDS(w.voff, w.gb + (uint64_t)(Q - 4) * w.row8, w.dst + kSmallSlab + (Q - 4) * 1024u);
+  if constexpr (Q < 4) MI355_LOAD_LDS(w.voff[Q], w.ga, w.dst + Q * 1024u);
+  else MI355_LOAD_LDS(w.voff[Q - 4], w.gb, w.dst + kSmallSlab + (Q - 4) * 1024u);
 }
 
 // The reads of a fragment set have arrived.  The registers ride along so that nothing that uses them can be placed
@@ -135,21 +146,22 @@ __device__ __forceinline__ void small_arrived(SmallFrags &f) {
   asm volatile("" : S_TIE4(f.b_lo), S_TIE4(f.b_hi));
 }
 
-// One step: the matrix instructions on `cur`, and in their shadow (a wave issues other work while the matrix pipe is
-// busy with its last instruction) the 16 reads of the next step's fragments into `nxt` and the 8 loads of the slab
-// four steps on, all behind the instructions of the first half of the step, so that the reads have arrived when the
-// second half is through: 16-bit and int8 kinds a read behind each of the first 16 instructions and a load behind
-// every second of them, fp8 two reads and a load behind each of the first 8.
+// One step: the matrix instructions on `cur`, and in their shadow the 16 reads of the next step's fragments into
+// `nxt` and the 8 loads of the slab four steps on.  A lone wave issues an instruction every four cycles or so, whatever
+// it is, so a 16-cycle matrix instruction has room for three others beside it: the loads ride one on every fourth
+// matrix instruction (every second for fp8) over the whole step, the reads one behind each of the first 16 (fp8: two
+// behind each of the first 8), so that they have arrived when the second half is through.
 // LAST: the step behind which nothing follows reads and loads nothing.
 template <int OP, bool LAST, int S>
 __device__ __forceinline__ void small_slot(const SmallFrags &cur, SmallFrags &nxt, const SmallWalk &w) {
-  small_mfma<OP, S>(cur);
+  constexpr int kEvery = small_is_fp8(OP) ? 2 : 4;
+  if constexpr (LAST || S % kEvery != 0) small_mfma<OP, S>(cur, w);
+  else small_mfma<OP, S, S / kEvery>(cur, w);
   if constexpr (LAST) return;
   if constexpr (small_is_fp8(OP)) {
-    if constexpr (S < 8) { small_read<2 * S>(nxt, w); small_read<2 * S + 1>(nxt, w); small_load<S>(w); }
+    if constexpr (S < 8) { small_read<2 * S>(nxt, w); small_read<2 * S + 1>(nxt, w); }
   } else {
     if constexpr (S < 16) small_read<S>(nxt, w);
-    if constexpr (S < 16 && S % 2 == 0) small_load<S / 2>(w);
   }
 }
 
@@ -211,8 +223,8 @@ gemm_small_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, 
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
   const uint32_t dst_wave = __builtin_amdgcn_readfirstlane(lds_base + wave * 32u * (uint32_t)kRowBytes);
   SmallWalk w;
-  w.voff = (lane / 8u) * k_bytes + ((lane % 8u) ^ (lane / 8u)) * 16u;
-  w.row8 = 8u * k_bytes;
+#pragma unroll
+  for (uint32_t q = 0; q < 4; q++) w.voff[q] = (lane / 8u + 8u * q) * k_bytes + ((lane % 8u) ^ (lane / 8u)) * 16u;
   w.ga = (uint64_t)(uintptr_t)(A + ((size_t)tm * kSmallTile + wave * 32u) * k_bytes);
   w.gb = (uint64_t)(uintptr_t)(B + ((size_t)tn * kSmallTile + wave * 32u) * k_bytes);
   uint32_t fetch_left = steps, fill = 0, look = 0;   // slot offsets: the one to fill, the one to read

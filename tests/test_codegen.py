@@ -368,9 +368,16 @@ def test_gemm_small_kernels(tmp_path):
         take = [n for n, l in on_acc if re.fullmatch(r"v_accvgpr_read_b32 v\d+, a\[?\d+\]?", l)]
         assert len(mfma) + len(zero) + len(take) == len(on_acc), [l for _, l in on_acc if not l.startswith(insn)][:3]
         assert len(mfma) == 5 * per_step and len(zero) == 64 and len(take) == 64, (name, len(mfma), len(zero), len(take))
-        assert max(zero) < min(mfma) and max(mfma) < min(take), name
+        assert max(zero) < min(mfma), name
         assert all(re.search(r"a\[(\d+):(\d+)\], v\[\d+:\d+\], v\[\d+:\d+\], a\[\1:\2\]", lines[n]) for n in mfma), name
-        assert [l for l in lines[max(mfma) + 1:min(take)] if l.startswith("s_nop 15")] == ["s_nop 15"] * 2, name
+        # the reads of the accumulators: one stretch of straight-line code that begins with the wait states and holds
+        # no matrix instruction (the compiler is free to place that block anywhere in the text)
+        waits = [n for n, l in enumerate(lines) if l == "s_nop 15"]
+        assert len(waits) == 2 and waits[1] == waits[0] + 1 and waits[1] < min(take), (name, waits)
+        stretch = [l.split(";")[0].strip() for l in body.splitlines()]
+        stretch = [l for l in stretch if l]
+        begin, end = stretch.index("s_nop 15"), max(n for n, l in enumerate(stretch) if l.startswith("v_accvgpr_read_b32"))
+        assert not any(l.startswith((insn, ".LBB", "s_cbranch", "s_branch")) for l in stretch[begin:end]), name
         assert sum(l.startswith("ds_read_b128 ") for l in lines) == 16 * 4, name          # prologue, two steps, one tail step
         assert sum(l.startswith("global_load_lds_dwordx4 ") for l in lines) == 8 * (4 + 3), name
         assert sum(l == "s_barrier" for l in lines) == 4, name
