@@ -179,10 +179,10 @@ gemm_f32_kernel(const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, fl
 }
 
 int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, uint32_t M, uint32_t N, uint32_t K,
-                 uint32_t elem) {
+                 uint32_t elem, uint32_t tile = kTile) {
   MI355_REQUIRE(dev, A && B && C, "gemm: null buffer");
   MI355_REQUIRE(dev, M > 0 && N > 0 && K > 0, "gemm: empty problem");
-  MI355_REQUIRE(dev, M % kTile == 0 && N % kTile == 0, "gemm: M (%u) and N (%u) must be multiples of 256", M, N);
+  MI355_REQUIRE(dev, M % tile == 0 && N % tile == 0, "gemm: M (%u) and N (%u) must be multiples of %u", M, N, tile);
   MI355_REQUIRE(dev, (uint64_t)K * elem <= (64u << 20), "gemm: a row of K is %llu bytes, the kernels take at most 64 MiB (32-bit lane offsets)",
                 (unsigned long long)K * elem);
   MI355_REQUIRE(dev, (K * elem) % kRowBytes == 0, "gemm: K (%u) must be a multiple of %u", K, kRowBytes / elem);
@@ -193,12 +193,16 @@ int check_shapes(mi355_dev *dev, const void *A, const void *B, const void *C, ui
 // The 8- and 16-bit kinds run on the four-wave kernel of gemm_quad.hip (256x256 tiles, one persistent workgroup per
 // CU), or, when that tiling has too few tiles for the part, on the 128x128 tiles of gemm_small.hip: four times the
 // workgroups at half the arithmetic per byte of operand.  "Too few" is at most half a tile per CU: from there up the
-// big tiles keep at least every second CU busy at twice the efficiency.
+// big tiles keep at least every second CU busy at twice the efficiency.  A product whose M or N is a multiple of 128
+// only has no 256x256 tiling and runs on the small tiles whatever its size.
 int launch_quad(mi355_dev *dev, int op, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N, uint32_t K,
                 uint32_t elem, float scale) {
-  if (int rc = check_shapes(dev, A, B, C, M, N, K, elem)) return rc;
+  if (int rc = check_shapes(dev, A, B, C, M, N, K, elem, kTile / 2)) return rc;
+  const bool big_fits = M % kTile == 0 && N % kTile == 0;
+  MI355_REQUIRE(dev, big_fits || dev->gemm_tiling != MI355_GEMM_TILING_256,
+                "gemm: M (%u) and N (%u) must be multiples of 256 on the 256x256 tiles this handle is set to", M, N);
   const uint64_t tiles = (uint64_t)(M / kTile) * (N / kTile);
-  const bool small = dev->gemm_tiling == MI355_GEMM_TILING_128 ||
+  const bool small = !big_fits || dev->gemm_tiling == MI355_GEMM_TILING_128 ||
                      (dev->gemm_tiling == MI355_GEMM_TILING_AUTO && 2u * tiles <= (uint64_t)(dev->props.num_cus > 0 ? dev->props.num_cus : 1));
   if (small) return mi355_launch_gemm_small(dev, op, what, A, B, C, M, N, K * elem, scale);
   return mi355_launch_gemm_quad(dev, op, what, A, B, C, M, N, K * elem, scale);

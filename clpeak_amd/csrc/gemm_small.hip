@@ -302,8 +302,8 @@ int launch_small(mi355_dev *dev, const char *what, const void *A, const void *B,
 
 }  // namespace
 
-// Shapes have been checked by the caller (multiples of 256 x 256, hence of 128 x 128; K a multiple of 128 bytes; 16-byte
-// aligned buffers; a row of K at most 64 MiB).
+// Shapes have been checked by the caller (M and N multiples of 128; K a multiple of 128 bytes; 16-byte aligned buffers;
+// a row of K at most 64 MiB).
 int mi355_launch_gemm_small(mi355_dev *dev, int op, const char *what, const void *A, const void *B, void *C, uint32_t M, uint32_t N,
                             uint32_t k_bytes, float scale) {
   switch (op) {

@@ -255,8 +255,8 @@ int mi355_mfma_raw(mi355_dev *dev, int sparse, int kind,
  * (src/rocm/rocblas.cpp:122-342 row "bf16"; src/rocm/hipblaslt_gemm.cpp:214-525 row
  * "fp8_e4m3"; both with K contiguous in A and B, fp32 accumulation, bf16 output).
  *   A[M][K] row-major, B[N][K] (column-major B), C[M][N] row-major bf16.
- * M, N multiples of 256, K a multiple of 128 bytes (64 bf16 values, 128 fp8 values) and a row of
- * K at most 64 MiB; buffers 16-byte aligned.  fp8: C = scale_a*scale_b * (A.B).  Sums along K are
+ * M, N multiples of 128 (fp32: of 256; see mi355_gemm_tiling), K a multiple of 128 bytes (64 bf16 values, 128 fp8
+ * values) and a row of K at most 64 MiB; buffers 16-byte aligned.  fp8: C = scale_a*scale_b * (A.B).  Sums along K are
  * formed in an order that depends on the tile (results agree within rounding; int8 exactly). */
 int mi355_gemm_bf16(mi355_dev *dev, const uint16_t *A, const uint16_t *B, uint16_t *C,
                     uint32_t M, uint32_t N, uint32_t K);
@@ -281,13 +281,14 @@ int mi355_gemm_fp8_e5m2(mi355_dev *dev, const uint8_t *A, const uint8_t *B, uint
  * and pickRocblasGemmDim, src/rocm/rocblas.cpp:71: thousands of rows).  128: one
  * workgroup per 128x128 tile, four times as many workgroups at half the arithmetic per operand byte.  AUTO (the
  * default of a new handle): 128 when the product has at most half a 256x256 tile per CU (2048 cubed: 64 tiles on
- * 256 CUs), 256 otherwise.  Both tilings take the same shapes; their results agree within rounding (int8 exactly). */
+ * 256 CUs), 256 otherwise.  The 256 tiling needs M and N to be multiples of 256: a product with a multiple of 128 only
+ * runs on the 128 tiling under AUTO and is refused under 256.  Results of the two agree within rounding (int8 exactly). */
 #define MI355_GEMM_TILING_AUTO 0
 #define MI355_GEMM_TILING_256  1
 #define MI355_GEMM_TILING_128  2
 int mi355_gemm_tiling(mi355_dev *dev, int tiling);
 /*   "fp32" of runRocblas (src/rocm/rocblas.cpp:246-254, rocblas_sgemm): fp32 operands, accumulation
- *          and output, on the fp32 matrix instruction; K a multiple of 32;
+ *          and output, on the fp32 matrix instruction; M, N multiples of 256, K a multiple of 32;
  *   "fp64" of runRocblas (src/rocm/rocblas.cpp:256-263, rocblas_dgemm): all fp64, on the fp64 matrix
  *          instruction; M, N multiples of 128, K a multiple of 16, buffers 32-byte aligned.
  *          Same operand layout as the rows above (K contiguous in A and in B). */

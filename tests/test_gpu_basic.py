@@ -37,7 +37,7 @@ def test_argument_errors_are_reported_not_launched(dev):
     assert "scale" in str(e.value)
     with pytest.raises(capi.Mi355Error) as e:
         dev.gemm_bf16(out, out, out, 100, 256, 64)
-    assert "multiples of 256" in str(e.value)
+    assert "multiples of 128" in str(e.value)
     # every GEMM entry point refuses a shape its tiling cannot cover, before anything is launched
     for call, text in ((lambda: dev.gemm_f16(out, out, out, 256, 256, 96), "multiple of 64"),
                        (lambda: dev.gemm_i8(out, out, out, 256, 256, 64), "multiple of 128"),

@@ -92,9 +92,37 @@ def test_the_library_picks_by_the_number_of_tiles(dev):
     assert not np.array_equal(small, large) and np.array_equal(many, large)
 
 
-def test_refuses_what_the_big_tiles_refuse(dev):
+def test_multiples_of_128_that_have_no_256_tiling(dev):
+    """M or N a multiple of 128 only: the whole of C against a float64 product of the decoded operands, under the
+    library's own choice of tiling (there is only one) as under the pinned one; the 256x256 tiling refuses."""
+    for tiling in (capi.GEMM_TILING_AUTO, capi.GEMM_TILING_128):
+        dev.gemm_tiling(tiling)
+        for M, N, K in [(128, 128, 64), (384, 640, 7 * 64), (2176, 2432, 192)]:
+            dA, dB, dC = dev.alloc(M * K * 2), dev.alloc(N * K * 2), dev.alloc(M * N * 2)
+            dev.memset(dC, 0xff)
+            dev.fill_bf16(dA, M * K, SEED, wl.STREAM_GEMM_A, capi.DIST_UPM1); dev.fill_bf16(dB, N * K, SEED, wl.STREAM_GEMM_B, capi.DIST_UPM1)
+            dev.gemm_bf16(dA, dB, dC, M, N, K)
+            a = (dA.download(np.uint16, M * K).astype(np.uint32) << 16).view(np.float32).astype(np.float64).reshape(M, K)
+            b = (dB.download(np.uint16, N * K).astype(np.uint32) << 16).view(np.float32).astype(np.float64).reshape(N, K)
+            ref = a @ b.T
+            got = (dC.download(np.uint16, M * N).astype(np.uint32) << 16).view(np.float32).astype(np.float64).reshape(M, N)
+            rms = float(np.sqrt((ref ** 2).mean()))
+            assert np.all(np.isfinite(got)), (M, N, K)
+            assert np.all(np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-2 * rms), (M, N, K, float(np.abs(got - ref).max()), rms)
+            for buf in (dA, dB, dC):
+                buf.free()
+    dev.gemm_tiling(capi.GEMM_TILING_256)
     a = dev.alloc(1 << 20)
-    for M, N, K in [(128, 256, 64), (256, 256, 32), (0, 256, 64)]:
+    with pytest.raises(capi.Mi355Error) as e:
+        dev.gemm_bf16(a, a, a, 384, 256, 64)
+    assert "multiples of 256" in str(e.value)
+    a.free()
+    dev.gemm_tiling(capi.GEMM_TILING_128)
+
+
+def test_refuses_what_no_tiling_covers(dev):
+    a = dev.alloc(1 << 20)
+    for M, N, K in [(64, 256, 64), (256, 192, 64), (256, 256, 32), (0, 256, 64)]:
         with pytest.raises(capi.Mi355Error):
             dev.gemm_bf16(a, a, a, M, N, K)
     with pytest.raises(capi.Mi355Error):
