@@ -13,8 +13,9 @@
 // they are multiplied, into the other of two fragment sets, in the shadow of the matrix instructions of the step
 // before.  Step s: wait until this wave's loads of slab s+1 have landed (loads complete in order: all but the newest
 // 16), barrier (now everybody's have, and everybody holds the fragments of slab s in registers, so the slot of slab
-// s-1 is free); the matrix instructions on the fragments of slab s, with the 16 reads of slab s+1 and the 8 loads of
-// slab s+4 behind those of the first half; wait for the reads.  The last step reads and loads nothing.  Past the last
+// s-1 is free); the matrix instructions on the fragments of slab s, with the 16 reads of slab s+1 behind those of the
+// first half and the 8 loads of slab s+4 riding on every fourth; wait for the reads.  The last step reads and loads
+// nothing.  Past the last
 // slab the loads wrap around to the start of the rows (fetches nobody reads, so that every step but the last is the
 // same code); they are waited for before the wave ends.
 //
